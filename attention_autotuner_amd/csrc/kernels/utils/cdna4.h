@@ -1,0 +1,211 @@
+// CDNA4 (gfx950) primitives shared by every kernel template in this tree: vector types, the
+// 32x32x16 fp16 MFMA, LDS-DMA tile copies, swizzled LDS addressing, barriers with explicit wait
+// counts, RNE fp16 packing and the lane<->lane^32 exchange used by all row reductions.
+//
+// This file plays the part that csrc/kernels/utils/{gmem_copy,matmul,misc}.h play in the reference
+// (reference: csrc/kernels/utils/gmem_copy.h:41-202, matmul.h:10-267, misc.h:7-67), but nothing here is
+// derived from CuTe: the layouts below are the native MFMA operand layouts of a 64-lane wavefront.
+//
+// MFMA v_mfma_f32_32x32x16_f16, one wave, lane l, half h = l/32, column n = l%32:
+//   A (32 x 16): lane holds A[n][8h .. 8h+7]          (8 halfs, one 16-byte chunk)
+//   B (16 x 32): lane holds B[8h .. 8h+7][n]
+//   C (32 x 32): lane holds C[8*(v/4) + 4h + v%4][n]  for v = 0..15
+// The contraction pairs slot (h, j) of A with slot (h, j) of B, so any consistent assignment of real
+// k indices to slots is valid.  All kernels here compute the *transposed* score tile S^T = K * Q^T:
+// then a lane owns ONE query row (n) and 16 of every 32 kv positions, row reductions are in-lane plus
+// one exchange with lane^32, and the C registers of S^T are already a valid B operand for O^T = V^T * P^T.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+namespace aat {
+
+typedef _Float16 half_t;
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef __fp16 fp16x4_t __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef float f2v __attribute__((ext_vector_type(2)));
+typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+
+#define AAT_DEV __device__ __forceinline__
+#define AAT_AS1 __attribute__((address_space(1)))
+#define AAT_AS3 __attribute__((address_space(3)))
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---------------------------------------------------------------------------------------------------
+// MFMA
+AAT_DEV f16v mfma_32x32x16(h8 a, h8 b, f16v c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+AAT_DEV f16v zero16() {
+  f16v z;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) z[i] = 0.f;
+  return z;
+}
+// Row of the 32x32 C tile that accumulator register v of a lane in half h holds.
+AAT_DEV constexpr int c_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3); }
+
+// ---------------------------------------------------------------------------------------------------
+// Wait counters and barriers.  s_barrier is issued through inline asm with a memory clobber so the
+// compiler keeps LDS accesses on their side of it; the hardware waits are spelled out by the caller
+// (vmcnt covers global loads AND LDS-DMA writes, lgkmcnt covers ds_read/ds_write).
+template <int N> AAT_DEV void wait_vmcnt() {
+  if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else if constexpr (N == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+  else if constexpr (N == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else if constexpr (N == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+  else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else if constexpr (N == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else if constexpr (N == 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+  else if constexpr (N == 32) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // unknown count: be conservative
+}
+AAT_DEV void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// Workgroup barrier that makes this thread's finished LDS traffic (ds ops and, when the caller has
+// already waited on vmcnt, LDS-DMA writes) visible to the other waves of the block.
+AAT_DEV void block_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// ---------------------------------------------------------------------------------------------------
+// Swizzles over 16-byte chunk indices of a row-major fp16 tile in LDS.  NC = chunks per row
+// (a multiple of 8 because every head dimension is a multiple of 64).  LDS has 64 banks x 4 B; a
+// ds_read_b128 is served 16 lanes per cycle, a ds_read_b64 32 lanes per cycle.
+//
+// swz_rows16: for "16 consecutive rows, same chunk" reads (MFMA A/B operand fetched as one b128 per
+// lane, rows across lanes).  Conflict-free for NC in {8,16,32,64}; 2-way for the other multiples of 8.
+template <int NC> AAT_DEV constexpr int swz_rows16(int row, int c) {
+  if constexpr (NC % 16 == 0) return c ^ (row & 15);
+  else if constexpr (NC == 8) return c ^ ((row >> 1) & 7);
+  else return c ^ (row & 7);
+}
+// swz_rows4: for the transposing read ds_read_b64_tr_b16, where one 32-lane phase touches 4
+// consecutive rows x 64 contiguous bytes.  Conflict-free for every NC that is a multiple of 8.
+template <int NC> AAT_DEV constexpr int swz_rows4(int row, int c) {
+  if constexpr (NC % 16 == 0) return c ^ ((row & 3) << 2);
+  else return c ^ (((row >> 1) & 1) << 2);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// LDS-DMA tile copy (global_load_lds_dwordx4): each lane names a 16-byte global source, the hardware
+// writes lane i's data at  lds_base + 16*i  with lds_base wave-uniform.  No VGPR staging; completion is
+// tracked by vmcnt.  A tile of ROWS x (NC*8) halfs is ROWS*NC chunks; thread t of NT copies chunks
+// t, t+NT, ...  Chunk slot s sits at LDS byte 16*s and holds global chunk (row = s/NC, c = SWZ(row, s%NC)).
+enum class Swz { Rows16, Rows4 };
+
+template <int NC, Swz MODE> AAT_DEV constexpr int swz(int row, int c) {
+  if constexpr (MODE == Swz::Rows16) return swz_rows16<NC>(row, c);
+  else return swz_rows4<NC>(row, c);
+}
+
+template <int ROWS, int NC, int NT, Swz MODE>
+struct TileDma {
+  static constexpr int kChunks = ROWS * NC;
+  static_assert(kChunks % NT == 0, "tile chunks must divide evenly over the block's threads");
+  static constexpr int kIters = kChunks / NT;          // LDS-DMA instructions per thread per tile
+  static constexpr int kBytes = kChunks * 16;
+  int goff[kIters];                                    // byte offset of this thread's source chunk inside a tile
+
+  AAT_DEV void init(int tid, int row_stride_bytes) {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      const int s = i * NT + tid;
+      const int row = s / NC, cs = s % NC;
+      goff[i] = row * row_stride_bytes + swz<NC, MODE>(row, cs) * 16;
+    }
+  }
+  // Issue the copy of one tile.  `g` points at the tile's first row in global memory, `lds` at the
+  // destination buffer (block-uniform); wave_base = 64 * wave index (wave-uniform).
+  AAT_DEV void issue(const char* g, char* lds, int wave_base) const {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) {
+      __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(g + goff[i]),
+                                       (AAT_AS3 void*)(lds + (i * NT + wave_base) * 16), 16, 0, 0);
+    }
+  }
+};
+
+// Byte offset of chunk (row, c) inside a swizzled LDS tile.
+template <int NC, Swz MODE> AAT_DEV int lds_chunk_off(int row, int c) {
+  return (row * NC + swz<NC, MODE>(row, c)) * 16;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// LDS reads in MFMA operand layouts.
+AAT_DEV h8 lds_read_h8(const char* p) { return *reinterpret_cast<const h8*>(p); }
+
+// Transposing read: within each group of 16 lanes, source lane s points at 4 contiguous halfs of row
+// s/4, column group s%4 of a 4-row x 16-column patch; destination lane i receives column i, rows 0..3.
+AAT_DEV h4 lds_read_tr_h4(const char* p) {
+  fp16x4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((AAT_AS3 fp16x4_t*)(p));
+  h4 o;
+  __builtin_memcpy(&o, &r, 8);
+  return o;
+}
+AAT_DEV h8 cat_h4(h4 lo, h4 hi) {
+  h8 r;
+  r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+  r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// fp32 -> fp16 round-to-nearest-even, two at a time (v_cvt_pk_f16_f32).  The reference converts P, S,
+// dS and every output with cutlass::NumericArrayConverter, which is RNE as well
+// (reference: csrc/kernels/attention/regfuse/regfuse.h:298-301, retnet/bwd/bwd_colblock.h:69-78).
+AAT_DEV h2 pack_rne(float a, float b) {
+  f2v p = {a, b};
+  return __builtin_convertvector(p, h2);
+}
+// Eight accumulator registers v0..v0+7 of a C tile -> one MFMA B/A operand.
+AAT_DEV h8 pack8_rne(const f16v& c, int v0) {
+  h8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    h2 p = pack_rne(c[v0 + 2 * i], c[v0 + 2 * i + 1]);
+    r[2 * i] = p[0];
+    r[2 * i + 1] = p[1];
+  }
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Exchange with lane^32 (v_permlane32_swap): the two lanes that share a query row in the S^T layout.
+AAT_DEV float other_half(float x) {
+  u2v r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  const float lo = __uint_as_float(r[0]), hi = __uint_as_float(r[1]);
+  // r[0] holds the lower half's value in all lanes, r[1] the upper half's.
+  return (threadIdx.x & 32) ? lo : hi;
+}
+AAT_DEV float pair_max(float x) {
+  u2v r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+AAT_DEV float pair_sum(float x) {
+  u2v r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+AAT_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+AAT_DEV float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// ---------------------------------------------------------------------------------------------------
+// Workgroup id -> tile id so that tiles sharing one (batch, head) -- and therefore one K/V stream --
+// run on the same XCD and hit the same L2.  Hardware deals consecutive workgroup ids round-robin over
+// the 8 XCDs; this undoes that when the grid is a multiple of 8.
+AAT_DEV int xcd_remap(int wg, int grid) {
+  constexpr int kXcd = 8;
+  if (grid % kXcd != 0) return wg;
+  return (wg % kXcd) * (grid / kXcd) + wg / kXcd;
+}
+
+}  // namespace aat

@@ -1,0 +1,141 @@
+"""fp32 restatement of the reference's torch math for attention and RetNet parallel retention.
+
+TEST INFRASTRUCTURE ONLY -- the product path never imports this file.
+
+Every function upcasts its (fp16) inputs to fp32 on the CPU and evaluates the closed form the
+reference uses as its own correctness check:
+
+* ``attention_ref``   follows reference python/utils/ref_op.py:2-6  (``softmax(q k^T * scale) v``); the
+  reference hard-codes scale = 0.125, here it is an argument (``None`` -> 1/sqrt(d_qk)) and a causal
+  lower-triangular mask (aligned to the bottom-right corner when S_q != S_kv) can be applied.
+* ``retnet_ref``      follows reference python/utils/ref_op.py:8-13 (``S = q k^T * mask``,
+  ``r = clamp(sum|S|, min=1)`` detached, ``o = (S / r) v``) and also returns ``r``.
+* ``retnet_bwd_ref``  is the closed form the backward kernel evaluates, reference
+  csrc/kernels/retnet/bwd/bwd_colblock.h:522-576: with r constant, ``P = S / r``,
+  ``dV = P^T dO``, ``dS = (dO V^T / r) * mask``, ``dK = dS^T Q``, ``dQ = dS K``.
+* ``retnet_decay_mask`` is the decay matrix of the benchmark configuration:
+  ``D[h, n, m] = gamma_h^(n-m)`` for n >= m else 0, ``gamma_h = 1 - 2^(-5-h)``.
+* ``attention_online_ref`` / ``retnet_online_ref`` restate the tile-by-tile recurrences sketched in
+  reference README.md:81-99 and python/tests/attntuner_demo.py:59-97,122-161; they exist so a test
+  can show the online form equals the one-shot form.
+
+Pinned by tests/test_oracle.py against torch's scaled_dot_product_attention, fp64 brute force
+(oracle/brute.c), closed-form special cases, autograd and gradcheck.  No function here is
+"parity unpinned".
+"""
+import math
+
+import torch
+
+REFERENCE_SOFTMAX_SCALE = 0.125  # reference python/utils/ref_op.py:3
+
+
+def _f32(x):
+    return x.detach().to(device="cpu", dtype=torch.float32)
+
+
+def causal_allowed(seq_q, seq_k):
+    """Boolean [seq_q, seq_k]: query i sees kv j iff j <= i + (seq_k - seq_q)."""
+    i = torch.arange(seq_q).unsqueeze(1)
+    j = torch.arange(seq_k).unsqueeze(0)
+    return j <= i + (seq_k - seq_q)
+
+
+def attention_ref(q, k, v, softmax_scale=None, causal=False, return_lse=False):
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(q.shape[-1])
+    s = (q @ k.transpose(-1, -2)) * softmax_scale
+    if causal:
+        s = s.masked_fill(~causal_allowed(q.shape[-2], k.shape[-2]), float("-inf"))
+    lse = torch.logsumexp(s, dim=-1)
+    p = torch.exp(s - lse.unsqueeze(-1))
+    p = torch.nan_to_num(p, nan=0.0)  # rows with no visible kv produce 0, not NaN
+    o = p @ v
+    return (o, lse) if return_lse else o
+
+
+def retnet_ref(q, k, v, mask, return_r=False):
+    q, k, v, mask = _f32(q), _f32(k), _f32(v), _f32(mask)
+    s = (q @ k.transpose(-1, -2)) * mask
+    r = s.abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
+    o = (s / r) @ v
+    return (o, r.squeeze(-1)) if return_r else o
+
+
+def retnet_bwd_ref(q, k, v, mask, do, r=None):
+    """Gradients of ``retnet_ref`` w.r.t. q, k, v with r treated as a constant."""
+    q, k, v, mask, do = _f32(q), _f32(k), _f32(v), _f32(mask), _f32(do)
+    s = (q @ k.transpose(-1, -2)) * mask
+    if r is None:
+        r = s.abs().sum(dim=-1).clamp(min=1.0)
+    r = _f32(r).unsqueeze(-1)
+    p = s / r
+    dv = p.transpose(-1, -2) @ do
+    ds = ((do @ v.transpose(-1, -2)) / r) * mask
+    dk = ds.transpose(-1, -2) @ q
+    dq = ds @ k
+    return dq, dk, dv
+
+
+def retnet_decay_mask(nheads, seq_q, seq_k, dtype=torch.float16):
+    n = torch.arange(seq_q, dtype=torch.float64).view(1, seq_q, 1)
+    m = torch.arange(seq_k, dtype=torch.float64).view(1, 1, seq_k)
+    gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(nheads, dtype=torch.float64)).view(nheads, 1, 1)
+    d = torch.where(n >= m, gamma ** (n - m).clamp(min=0), torch.zeros((), dtype=torch.float64))
+    return d.to(torch.float32).to(dtype)
+
+
+def attention_online_ref(q, k, v, softmax_scale=None, causal=False, block_kv=64):
+    """Tile-by-tile recurrence with an unscaled running max, as the kernels evaluate it."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(q.shape[-1])
+    sq, sk = q.shape[-2], k.shape[-2]
+    allowed = causal_allowed(sq, sk) if causal else None
+    m = torch.full(q.shape[:-1], float("-inf"))
+    l = torch.zeros(q.shape[:-1])
+    o = torch.zeros(*q.shape[:-1], v.shape[-1])
+    for j0 in range(0, sk, block_kv):
+        s = q @ k[..., j0:j0 + block_kv, :].transpose(-1, -2)
+        if causal:
+            s = s.masked_fill(~allowed[:, j0:j0 + block_kv], float("-inf"))
+        m_new = torch.maximum(m, s.amax(dim=-1))
+        m_use = torch.where(torch.isinf(m_new), torch.zeros_like(m_new), m_new)
+        alpha = torch.exp((m - m_use) * softmax_scale)
+        p = torch.exp((s - m_use.unsqueeze(-1)) * softmax_scale)
+        l = l * alpha + p.sum(dim=-1)
+        o = o * alpha.unsqueeze(-1) + p.half().float() @ v[..., j0:j0 + block_kv, :]
+        m = m_new
+    return o / l.unsqueeze(-1)
+
+
+def retnet_online_ref(q, k, v, mask, block_kv=64):
+    """Running abs-sum recurrence: R += sum|S|, r = max(R, 1), O = O r_old/r_new + half(S/r_new) V."""
+    q, k, v, mask = _f32(q), _f32(k), _f32(v), _f32(mask)
+    sk = k.shape[-2]
+    big_r = torch.zeros(q.shape[:-1])
+    r_old = torch.ones(q.shape[:-1])
+    o = torch.zeros(*q.shape[:-1], v.shape[-1])
+    for j0 in range(0, sk, block_kv):
+        s = (q @ k[..., j0:j0 + block_kv, :].transpose(-1, -2)) * mask[..., j0:j0 + block_kv]
+        big_r = big_r + s.abs().sum(dim=-1)
+        r_new = big_r.clamp(min=1.0)
+        o = o * (r_old / r_new).unsqueeze(-1) + (s / r_new.unsqueeze(-1)).half().float() @ v[..., j0:j0 + block_kv, :]
+        r_old = r_new
+    return o, r_old
+
+
+def attention_split_merge_ref(q, k, v, softmax_scale=None, n_splits=2):
+    """Split the kv range, run each part independently, merge with the log-sum-exp weights."""
+    sk = k.shape[-2]
+    step = sk // n_splits
+    outs, lses = [], []
+    for i in range(n_splits):
+        o_i, lse_i = attention_ref(q, k[..., i * step:(i + 1) * step, :], v[..., i * step:(i + 1) * step, :],
+                                   softmax_scale, False, return_lse=True)
+        outs.append(o_i)
+        lses.append(lse_i)
+    lse = torch.logsumexp(torch.stack(lses), dim=0)
+    o = sum(o_i * torch.exp(l_i - lse).unsqueeze(-1) for o_i, l_i in zip(outs, lses))
+    return o
