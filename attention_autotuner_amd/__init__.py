@@ -1,0 +1,13 @@
+"""MI355X-native fused attention / RetNet kernels with an autotuner.
+
+Public surface (same names as the reference's python/ tree):
+    flash_attn_func(q, k, v, device_type[, causal[, softmax_scale]])
+    RetNetAttnFunc(q, k, v, mask, device_type[, causal])
+    arch.MI355X, autotuner.{AttnTunner, RetTunner, RetBwdTunner, Runtime, AttnConfig, RetConfig, RetBwdConfig}
+"""
+from . import arch, autotuner, ops, utils
+from .arch import MI355X, Arch
+from .ops import flash_attn_func, RetNetAttnFunc, REFERENCE_SOFTMAX_SCALE
+
+__all__ = ["arch", "autotuner", "ops", "utils", "MI355X", "Arch", "flash_attn_func", "RetNetAttnFunc",
+           "REFERENCE_SOFTMAX_SCALE"]

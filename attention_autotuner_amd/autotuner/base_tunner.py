@@ -1,0 +1,202 @@
+"""Tuning loop: enumerate -> validate -> compile in parallel -> time through the C ABI -> log + cache.
+
+Mirrors reference python/autotuner/base_tunner.py:68-208 (``BaseTunner``) in interface -- a tuner is
+built from ``(arch, torch_array)`` and ``tune(log_path)`` returns the best configuration, consulting
+an on-disk cache first -- with these deliberate changes:
+
+* the cache key is the whole problem (arch, operator, head dims, B, H, S_q, S_kv, causal), not just
+  the two head dims, because the best tile for S_q=256/S_kv=16384 is not the best for 2048/2048;
+  the reference's ``best_config_{op}_{dqk}_{dv}.json`` name is still read as a fallback;
+* a configuration whose compile fails or times out is skipped (the reference dereferences None);
+* timing calls ``profile_ex`` on the caller's stream with the caller's softmax scale / causal flag;
+* compiled libraries are kept (content-addressed), so a later ``Runtime`` reuses the tuned binary.
+"""
+import ctypes
+import json
+import os
+import pprint
+import time
+
+import torch
+
+from . import codegen, library
+from .configs import supported_configs
+
+_PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
+DEFAULT_CACHE_DIR = os.environ.get("AAT_CACHE_DIR", os.path.join(_PKG, "cache"))
+FAILED = 1e8                          # latency recorded for a configuration that errored at run time
+
+_memo = {}                            # in-process memo of resolved best configs
+
+
+class CompileResult:
+    def __init__(self, config, lib_name):
+        self.config = config
+        self.lib_name = lib_name
+
+
+def _stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class BaseTunner:
+    operation = None                  # config operation name ("attn", ...)
+
+    def __init__(self, arch, torch_array, op_name, causal=False, softmax_scale=None):
+        self.arch = arch
+        self.torch_array = torch_array
+        self.op_name = op_name
+        self.causal = bool(causal)
+        self.softmax_scale = softmax_scale
+        self.Br_list = [32, 64, 128, 256]
+        self.Bc_list = [32, 64, 128, 256]
+        self.cache_path = DEFAULT_CACHE_DIR
+        self.build_dir = None
+        self.verbose = os.environ.get("AAT_VERBOSE", "0") == "1"
+        q, k, v = torch_array[0], torch_array[1], torch_array[2]
+        self.problem_key = {"dim_qk": int(q.shape[-1]), "dim_v": int(v.shape[-1])}
+        self.problem_shape = {"B": int(q.shape[0]), "H": int(q.shape[1]), "Sq": int(q.shape[2]), "Sk": int(k.shape[2])}
+
+    # ---- search space (filled in by subclasses) -------------------------------------------------------
+    def generate_configs(self, Br, Bc, dim_qk, dim_v):
+        return []
+
+    def validate_register_fuse(self, config):
+        return False
+
+    def validate_shared_fuse(self, config):
+        return False
+
+    def validate_kernel(self, config):
+        return False
+
+    def _is_valid(self, config):
+        if config.fuse_type == "register":
+            return self.validate_register_fuse(config)
+        if config.fuse_type == "shared":
+            return self.validate_shared_fuse(config)
+        return self.validate_kernel(config)
+
+    def _fits_problem(self, config):
+        s = self.problem_shape
+        return s["Sq"] % config.Br == 0 and s["Sk"] % config.Bc == 0
+
+    def get_tuned_configs(self):
+        dq, dv = self.problem_key["dim_qk"], self.problem_key["dim_v"]
+        return [c for Br in self.Br_list for Bc in self.Bc_list
+                for c in self.generate_configs(Br, Bc, dq, dv) if self._is_valid(c)]
+
+    # ---- compile + time --------------------------------------------------------------------------------
+    def compile(self, configs, temp_dir=None, timeout=None):
+        return [self._result(c, codegen.compile_config(c, self.arch, temp_dir or self.build_dir, timeout)) for c in configs]
+
+    def compile_parallel(self, configs, temp_dir=None, timeout=None):
+        libs = codegen.compile_parallel(configs, self.arch, temp_dir or self.build_dir, timeout)
+        return [self._result(c, lib) for c, lib in zip(configs, libs)]
+
+    @staticmethod
+    def _result(config, lib):
+        return CompileResult(config, lib)
+
+    def _ex_args(self):
+        """Operator-specific scalar arguments between the sizes and the workspace."""
+        return [ctypes.c_int(int(self.causal))]
+
+    def profile(self, libname, device="cuda:0"):
+        """Mean milliseconds of one launch of ``libname`` on this tuner's tensors (FAILED on error)."""
+        lib = library.load(libname, self.operation)
+        s = self.problem_shape
+        need = lib.workspace_size(s["B"], s["H"], s["Sq"], s["Sk"])
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=self.torch_array[0].device) if need else None
+        ptrs = [ctypes.c_void_p(t.data_ptr()) for t in self.torch_array]
+        ms = lib.profile_ex(*ptrs, s["B"], s["H"], s["Sq"], s["Sk"], *self._ex_args(),
+                            ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
+        return FAILED if ms < 0 else float(ms)
+
+    # ---- cache -----------------------------------------------------------------------------------------
+    def _cache_file(self):
+        k, s = self.problem_key, self.problem_shape
+        return os.path.join(self.cache_path, "best_config_{}_{}_{}_{}_b{}h{}q{}k{}_c{}.json".format(
+            self.op_name, self.arch.name, k["dim_qk"], k["dim_v"], s["B"], s["H"], s["Sq"], s["Sk"], int(self.causal)))
+
+    def _legacy_cache_file(self):
+        k = self.problem_key
+        return os.path.join(self.cache_path, "best_config_{}_{}_{}.json".format(self.op_name, k["dim_qk"], k["dim_v"]))
+
+    def _memo_key(self):
+        return (self._cache_file(),)
+
+    def check_cache(self):
+        hit = _memo.get(self._memo_key())
+        if hit is not None:
+            return hit
+        for path in (self._cache_file(), self._legacy_cache_file()):
+            try:
+                with open(path) as f:
+                    dd = json.load(f)
+                cfg = supported_configs[dd["operation"]].from_dict(dd)
+            except (OSError, ValueError, KeyError):
+                continue                                  # missing or corrupt cache file: fall through
+            if self._fits_problem(cfg):
+                _memo[self._memo_key()] = cfg
+                return cfg
+        return None
+
+    def _write_cache(self, config):
+        os.makedirs(self.cache_path, exist_ok=True)
+        with open(self._cache_file(), "w") as f:
+            json.dump(config.to_dict(), f)
+        _memo[self._memo_key()] = config
+
+    # ---- the loop --------------------------------------------------------------------------------------
+    def tune(self, log_path="../logs/", timeout=120, use_cache=True):
+        started = time.time()
+        if use_cache:
+            cached = self.check_cache()
+            if cached is not None:
+                return cached
+        configs = [c for c in self.get_tuned_configs() if self._fits_problem(c)]
+        if not configs:
+            raise RuntimeError(f"no valid {self.op_name} configuration for {self.problem_key} {self.problem_shape}")
+        if self.verbose:
+            print("Configs to be tuned: ")
+            for c in configs:
+                pprint.pprint(c)
+        results = self.compile_parallel(configs, timeout=timeout)
+        timings, best, best_ms = {}, None, FAILED
+        for res in results:
+            if res.lib_name is None:
+                continue                                  # compile failed or timed out
+            ms = self.profile(res.lib_name)
+            if ms == FAILED and self.verbose:
+                pprint.pprint(res.config)
+                print("profile runtime error")
+            timings[res.config] = ms
+            if ms < best_ms:
+                best, best_ms = res.config, ms
+        if best is None:
+            raise RuntimeError(f"every {self.op_name} candidate failed to compile or run")
+        elapsed = time.time() - started
+        if self.verbose:
+            print("#" * 58)
+            print("Operation type: ", best.operation)
+            print("Best config: ")
+            pprint.pprint(best)
+            print("Latency: ", best_ms)
+        self._write_log(log_path, timings, best, best_ms, elapsed)
+        self._write_cache(best)
+        self.last_timings = timings
+        return best
+
+    def _write_log(self, log_path, timings, best, best_ms, elapsed):
+        """Same text layout as the reference's profile_result_*.txt (base_tunner.py:178-188)."""
+        if log_path is None:
+            return
+        k = self.problem_key
+        os.makedirs(log_path, exist_ok=True)
+        name = "profile_result_{}_{}_{}.txt".format(best.operation, k["dim_qk"], k["dim_v"])
+        with open(os.path.join(log_path, name), "w") as f:
+            for cfg, ms in timings.items():
+                f.write(repr(cfg) + "\n" + str(ms) + "\n")
+            f.write("\nbest config: \n" + repr(best) + "\n" + str(best_ms) + "\n")
+            f.write("\nsearch time: " + str(elapsed) + "s")

@@ -1,0 +1,129 @@
+"""Wrapper generation and hipcc driver.
+
+One configuration -> one ``.hip`` wrapper (template text from ``csrc/kernels/**/profile_code.py`` filled
+with ``vars(config)``) -> one shared object exporting the C ABI of include/aat_kernel_abi.h.  Same job
+as ``_create_code_for_profiling`` / ``_compile`` in reference python/autotuner/base_tunner.py:25-66 and
+``Runtime.compile`` in reference python/autotuner/runtime.py:42-72, with three changes: libraries
+are content-addressed (configuration + a hash of every kernel source), they live in a persistent
+in-tree directory so a tuned library is never rebuilt, and a failed or timed-out compile yields
+``None`` that callers skip instead of crashing on.
+"""
+import functools
+import hashlib
+import importlib.util
+import os
+import shutil
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+_PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
+CSRC_DIR = os.path.join(_PKG, "csrc")
+INCLUDE_DIR = os.path.normpath(os.path.join(_PKG, "..", "include"))
+DEFAULT_BUILD_DIR = os.environ.get("AAT_BUILD_DIR", os.path.join(_PKG, "build"))
+
+# -packed-fp32-ops is switched OFF on purpose: hipcc would otherwise fuse scalar fp32 math into
+# v_pk_*_f32 instructions.
+HIPCC_FLAGS = ["-std=c++17", "-O3", "-fno-math-errno", "-ffp-contract=fast", "-fPIC", "-shared", "-w",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def hipcc_exe():
+    exe = os.environ.get("HIPCC")
+    if exe:
+        return exe
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cand = os.path.join(rocm, "bin", "hipcc")
+    return cand if os.path.exists(cand) else (shutil.which("hipcc") or "hipcc")
+
+
+def _template_file(config):
+    sub = {"register": "regfuse", "shared": "smemfuse"}.get(config.fuse_type, "")
+    return os.path.join(config.template_dir, sub, "profile_code.py")
+
+
+@functools.lru_cache(maxsize=None)
+def _load_template(path):
+    spec = importlib.util.spec_from_file_location("aat_profile_code_" + hashlib.sha1(path.encode()).hexdigest()[:8], path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def render(config, kind="kernel"):
+    """Source text of the wrapper for ``config``; ``kind`` is "kernel" or "profile" (the same text
+    here, both entry points live in one library)."""
+    mod = _load_template(_template_file(config))
+    text = mod.kernel_code if kind == "kernel" else mod.profile_code
+    fields = dict(vars(config))
+    fields["config_name"] = f"{config.operation}:{config}"
+    return text.format_map(fields)
+
+
+@functools.lru_cache(maxsize=1)
+def source_digest():
+    """Hash of every file that can change the machine code of a config library."""
+    h = hashlib.sha1()
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    for root in (os.path.join(CSRC_DIR, "kernels"), INCLUDE_DIR):
+        for dirpath, dirnames, filenames in sorted(os.walk(root)):
+            dirnames.sort()
+            for fn in sorted(filenames):
+                if fn.endswith((".h", ".py", ".hip")):
+                    with open(os.path.join(dirpath, fn), "rb") as f:
+                        h.update(fn.encode())
+                        h.update(f.read())
+    return h.hexdigest()[:10]
+
+
+def library_name(config):
+    return f"{config}-{source_digest()}.so"
+
+
+def library_path(config, build_dir=None):
+    return os.path.join(build_dir or DEFAULT_BUILD_DIR, config.operation, library_name(config))
+
+
+def hipcc_command(src, out, arch):
+    target = getattr(arch, "hipcc_arch", None) or arch.compute_capability
+    return [hipcc_exe(), *HIPCC_FLAGS, f"--offload-arch={target}", f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", src, "-o", out]
+
+
+def compile_config(config, arch, build_dir=None, timeout=None, force=False):
+    """Build the library for ``config``; returns its path, or None if hipcc failed or timed out."""
+    if getattr(arch, "platform", "ROCm") != "ROCm":
+        return None
+    out = library_path(config, build_dir)
+    if os.path.exists(out) and not force:
+        return out
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    src = out[:-3] + ".hip"
+    try:
+        text = render(config)
+    except (KeyError, FileNotFoundError, AttributeError):
+        return None
+    with open(src, "w") as f:
+        f.write(text)
+    tmp = out + f".tmp{os.getpid()}"
+    try:
+        ret = subprocess.run(hipcc_command(src, tmp, arch), timeout=timeout, capture_output=True, text=True)
+    except subprocess.TimeoutExpired:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        return None
+    if ret.returncode != 0:
+        with open(out[:-3] + ".log", "w") as f:
+            f.write(ret.stdout + ret.stderr)
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        return None
+    os.replace(tmp, out)
+    return out
+
+
+def compile_parallel(configs, arch, build_dir=None, timeout=None, max_workers=None):
+    """Compile many configurations with a pool of hipcc subprocesses; result list is aligned with
+    ``configs`` and holds None where a compile failed."""
+    workers = max_workers or int(os.environ.get("MAX_JOBS", 0)) or os.cpu_count() or 1
+    workers = max(1, min(workers, 16, len(configs) or 1))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        return list(pool.map(lambda c: compile_config(c, arch, build_dir, timeout), configs))

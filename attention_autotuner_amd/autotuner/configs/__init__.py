@@ -1,0 +1,13 @@
+from .base_config import BaseConfig, balanced_wave_split, factor_pairs
+from .attention import AttnConfig
+from .retnet import RetConfig
+from .retnet_bwd import RetBwdConfig
+
+supported_configs = {
+    "attn": AttnConfig,
+    "ret": RetConfig,
+    "ret_bwd": RetBwdConfig,
+}
+
+__all__ = ["BaseConfig", "AttnConfig", "RetConfig", "RetBwdConfig", "supported_configs",
+           "balanced_wave_split", "factor_pairs"]

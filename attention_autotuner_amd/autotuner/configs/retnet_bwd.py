@@ -1,0 +1,34 @@
+from .base_config import BaseConfig
+
+
+class RetBwdConfig(BaseConfig):
+    """RetNet parallel backward (reference python/autotuner/configs/retnet_bwd.py:4-26).
+
+    The ``mmawarpsN*`` fields say how the block's waves are split along the N side of each of the
+    contractions (S/dS, dV, dK, dQ)."""
+    operation = "ret_bwd"
+    kernel_subdir = "retnet/bwd"
+    _fields = ("Br", "Bc", "Kd", "D", "mmawarpsN", "mmawarpsN_dv", "mmawarpsN_dk", "mmawarpsN_dq", "Nthreads",
+               "unrollLastIter", "BlockKSmem", "num_stages_qk", "num_stages_mask", "num_stages_dv",
+               "num_stages_ds", "num_stages_dq")
+
+    def __init__(self, Br, Bc, Kd, D, mmawarpsN, mmawarpsN_dv, mmawarpsN_dk, mmawarpsN_dq, Nthreads=256,
+                 unrollLastIter=True, BlockKSmem=256, num_stages_qk=1, num_stages_mask=1, num_stages_dv=1,
+                 num_stages_ds=1, num_stages_dq=1, waves_per_eu=1):
+        super().__init__(Br, Bc, Kd, D, BlockKSmem, num_stages_qk, Nthreads, unrollLastIter)
+        self.num_stages_mask = num_stages_mask
+        self.mmawarpsN = mmawarpsN
+        self.mmawarpsN_dv = mmawarpsN_dv
+        self.mmawarpsN_dk = mmawarpsN_dk
+        self.mmawarpsN_dq = mmawarpsN_dq
+        self.num_stages_dv = num_stages_dv
+        self.num_stages_ds = num_stages_ds
+        self.num_stages_dq = num_stages_dq
+        self.waves_per_eu = waves_per_eu
+        self.fuse_type = "bwd"
+
+    def __repr__(self):
+        return "RetBwdConfig(" + ", ".join(f"{f}={getattr(self, f)}" for f in self._fields) + ")"
+
+    def __str__(self):
+        return "_".join([self.operation] + [str(getattr(self, f)) for f in self._fields] + self._extras())

@@ -1,0 +1,104 @@
+"""Search space and validity model for MI355X (gfx950).
+
+The knobs that matter on CDNA4 are not the ones that matter on Ampere: tiles are built from
+32x32x16 MFMAs so every wave owns whole 32-row groups; K/V reach LDS by LDS-DMA so "stages" are
+whole-tile buffers; and the register file is split between the resident waves of a SIMD, so the
+occupancy target (``waves_per_eu``) is itself a knob.  Validity is LDS bytes (160 KB per CU, shared by
+all resident blocks) and a per-lane register estimate (512 / waves_per_eu).
+"""
+from .configs import AttnConfig, RetConfig, RetBwdConfig
+
+WAVE = 64
+MFMA_M = 32
+BR_LIST = (64, 128, 256)
+BC_LIST = (32, 64, 128)
+THREADS = (128, 256, 512)
+STAGES = ((1, 1), (2, 2), (2, 1), (1, 2))
+
+
+def _waves(cfg):
+    return cfg.Nthreads // WAVE
+
+
+def rows_per_wave(cfg):
+    return cfg.Br // _waves(cfg)
+
+
+def blocks_per_cu(cfg):
+    """Resident blocks per CU implied by the occupancy target (4 SIMDs per CU)."""
+    return max(1, (cfg.waves_per_eu * 4) // _waves(cfg))
+
+
+def dma_divisible(cfg):
+    nt = cfg.Nthreads
+    return (cfg.Bc * cfg.Kd // 8) % nt == 0 and (cfg.Bc * cfg.D // 8) % nt == 0
+
+
+# ---- forward (attention and RetNet) ------------------------------------------------------------------
+def forward_lds_bytes(cfg):
+    main = cfg.num_stages_qk * cfg.Bc * cfg.Kd * 2 + cfg.num_stages_v * cfg.Bc * cfg.D * 2
+    if cfg.operation == "ret":
+        main += cfg.num_stages_mask * cfg.Br * cfg.Bc * 2
+    if cfg.fuse_type == "shared":
+        main += cfg.Br * (cfg.Bc * 2 + 16)            # P tile, fp16, padded rows
+    epilogue = cfg.Br * (cfg.D * 2 + 16)
+    return max(main, epilogue)
+
+
+def forward_reg_estimate(cfg):
+    """Per-lane 32-bit registers of the dominant live set."""
+    rt = rows_per_wave(cfg) // MFMA_M
+    q_regs = rt * (cfg.Kd // 16) * 4
+    s_regs = rt * (cfg.Bc // 32) * 16
+    p_regs = rt * (cfg.Bc // 32) * 8
+    if cfg.fuse_type == "register":
+        o_regs = rt * (cfg.D // 32) * 16
+    else:
+        # shared fuse: the waves split D between them for the second contraction
+        o_regs = (cfg.Br // MFMA_M) * (cfg.D // 32) * 16 // _waves(cfg)
+    return q_regs + s_regs + p_regs + o_regs + 48
+
+
+def forward_valid(cfg, arch):
+    if cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * _waves(cfg)):
+        return False
+    if cfg.Bc % 32 or cfg.Kd % 64 or cfg.D % 64:
+        return False
+    if _waves(cfg) > 4 * cfg.waves_per_eu:           # the block itself needs that many waves per SIMD
+        return False
+    if not dma_divisible(cfg):
+        return False
+    if forward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
+        return False
+    return forward_reg_estimate(cfg) <= arch.register_per_thread // cfg.waves_per_eu
+
+
+def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "shared")):
+    out = []
+    for nthreads in THREADS:
+        for st_qk, st_v in STAGES:
+            for wpe in (1, 2):
+                for fuse in fuse_types:
+                    if op == "attn":
+                        cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, waves_per_eu=wpe)
+                    else:
+                        cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, 1, st_v, nthreads, True, waves_per_eu=wpe)
+                    out.append(cfg.set_fuse_type(fuse))
+    return out
+
+
+def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
+    """A configuration that is valid for every supported head size; used before/without tuning."""
+    prefs = [(128, 64, 256, 2, 2, 2), (128, 64, 256, 1, 1, 2), (128, 64, 256, 1, 1, 1), (128, 32, 256, 1, 1, 1),
+             (64, 32, 128, 1, 1, 1)]
+    for br, bc, nt, sq, sv, wpe in prefs:
+        if (seq_q and seq_q % br) or (seq_k and seq_k % bc):
+            continue
+        if op == "attn":
+            cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, sq, sv, nt, True, waves_per_eu=wpe)
+        else:
+            cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, sq, 1, sv, nt, True, waves_per_eu=wpe)
+        cfg.set_fuse_type("register")
+        if forward_valid(cfg, arch):
+            return cfg
+    raise ValueError(f"no default {op} configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")

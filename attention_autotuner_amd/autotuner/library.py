@@ -1,0 +1,53 @@
+"""ctypes binding of a config library (the Python side of include/aat_kernel_abi.h)."""
+import ctypes
+import threading
+
+_VP, _I, _F, _SZ = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+
+# number of device-pointer arguments per operator
+N_POINTERS = {"attn": 4, "ret": 6, "ret_bwd": 10}
+
+_handles = {}
+_lock = threading.Lock()
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+def _bind(lib, op):
+    n = N_POINTERS[op]
+    ptrs = [_VP] * n
+    lib.abi_version.restype = _I
+    lib.abi_version.argtypes = []
+    lib.config_string.restype = ctypes.c_char_p
+    lib.config_string.argtypes = []
+    lib.workspace_size.restype = _SZ
+    lib.workspace_size.argtypes = [_I] * 4
+    lib.profile.restype = _F
+    lib.profile.argtypes = ptrs + [_I] * 4
+    lib.kernel_entry.restype = _I
+    lib.kernel_entry.argtypes = ptrs + [_I] * 4
+    extra = [_F, _I] if op == "attn" else [_I]       # attention: scale + causal; RetNet: causal
+    tail = extra + [_VP, _SZ, _VP]                   # workspace, bytes, stream
+    lib.profile_ex.restype = _F
+    lib.profile_ex.argtypes = ptrs + [_I] * 4 + tail
+    lib.kernel_entry_ex.restype = _I
+    lib.kernel_entry_ex.argtypes = ptrs + [_I] * 4 + tail
+    return lib
+
+
+def load(path, op):
+    """dlopen ``path`` once per process and set the prototypes for operator ``op``."""
+    key = (path, op)
+    lib = _handles.get(key)
+    if lib is None:
+        with _lock:
+            lib = _handles.get(key)
+            if lib is None:
+                try:
+                    lib = _bind(ctypes.CDLL(path), op)
+                except (OSError, AttributeError) as e:
+                    raise KernelLibraryError(f"cannot load kernel library {path}: {e}") from e
+                _handles[key] = lib
+    return lib

@@ -1,0 +1,94 @@
+"""The set of config libraries built ahead of time (``python -m attention_autotuner_amd.autotuner.prebuilt``).
+
+JIT compilation works anywhere hipcc is installed, but a first call that has to compile is slow and
+a machine without a compiler cannot run at all; so the default configuration of every head-size pair
+in common use, plus every configuration recorded in the tuning cache, is built into the in-tree
+library directory up front.
+"""
+import glob
+import json
+import os
+import sys
+
+from ..arch import MI355X
+from . import codegen, gfx950_space
+from .base_tunner import DEFAULT_CACHE_DIR
+from .configs import supported_configs
+
+# (operator, d_qk, d_v) pairs whose default configuration is always built
+DEFAULT_PROBLEMS = [
+    ("attn", 64, 64), ("attn", 128, 128), ("attn", 256, 256), ("attn", 192, 192), ("attn", 256, 128), ("attn", 64, 128),
+]
+
+
+# Tile/wave/buffer combinations built for every head-size pair below so that the parity suite can
+# show that all of them compute the same thing: (Br, Bc, Nthreads, K buffers, V buffers, waves per SIMD).
+PARITY_TILES = [
+    (128, 64, 256, 2, 2, 2), (128, 64, 256, 1, 1, 2), (128, 64, 256, 2, 1, 1), (128, 64, 256, 1, 2, 1),
+    (128, 32, 256, 2, 2, 2), (128, 128, 256, 1, 1, 1), (64, 64, 128, 2, 2, 2), (128, 64, 128, 1, 1, 1),
+    (256, 64, 512, 2, 2, 2),
+]
+PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
+
+
+def extra_configs(arch=None):
+    """Additional libraries built ahead of time: the parity matrix."""
+    from .configs import AttnConfig
+    arch = arch or MI355X()
+    out = []
+    for dqk, dv in PARITY_DIMS:
+        for br, bc, nt, sq, sv, wpe in PARITY_TILES:
+            cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+            if gfx950_space.forward_valid(cfg, arch):
+                out.append(cfg)
+    return out
+
+
+def cached_configs(cache_dir=None):
+    out = []
+    for path in sorted(glob.glob(os.path.join(cache_dir or DEFAULT_CACHE_DIR, "best_config_*.json"))):
+        try:
+            with open(path) as f:
+                dd = json.load(f)
+            out.append(supported_configs[dd["operation"]].from_dict(dd))
+        except (OSError, ValueError, KeyError):
+            continue
+    return out
+
+
+def shipping_set(arch=None):
+    arch = arch or MI355X()
+    cfgs = []
+    for op, dqk, dv in DEFAULT_PROBLEMS:
+        if op in ("attn", "ret"):
+            cfgs.append(gfx950_space.default_forward_config(op, dqk, dv, arch))
+    cfgs += extra_configs(arch)
+    cfgs += cached_configs()
+    seen, unique = set(), []
+    for c in cfgs:
+        key = (c.operation, str(c))
+        if key not in seen:
+            seen.add(key)
+            unique.append(c)
+    return unique
+
+
+def build_all(arch=None, force=True, timeout=600, verbose=True):
+    arch = arch or MI355X()
+    cfgs = shipping_set(arch)
+    if force:
+        for c in cfgs:
+            p = codegen.library_path(c)
+            if os.path.exists(p):
+                os.remove(p)
+    libs = codegen.compile_parallel(cfgs, arch, timeout=timeout)
+    failed = [c for c, l in zip(cfgs, libs) if l is None]
+    if verbose:
+        print(f"built {len(cfgs) - len(failed)}/{len(cfgs)} config libraries into {codegen.DEFAULT_BUILD_DIR}")
+    if failed:
+        raise RuntimeError("hipcc failed for: " + ", ".join(f"{c.operation}:{c}" for c in failed))
+    return libs
+
+
+if __name__ == "__main__":
+    build_all(force="--force" in sys.argv)

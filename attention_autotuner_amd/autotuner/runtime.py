@@ -1,0 +1,75 @@
+"""Launcher for one configuration (reference python/autotuner/runtime.py:32-89).
+
+``Runtime(arch, config).apply(torch_array)`` builds (or finds) the configuration's library and
+enqueues one launch on the current PyTorch stream.  Unlike the reference, the dlopen handle is kept
+for the life of the process, the return code of the kernel entry is checked, and a missing library
+is an error -- there is no CPU fallback.
+"""
+import ctypes
+import math
+import os
+
+import torch
+
+from . import codegen, library
+
+
+class KernelLaunchError(RuntimeError):
+    pass
+
+
+_ERRORS = {-2: "sequence lengths are not multiples of the configuration's tile (Br, Bc)",
+           -3: "workspace missing or too small"}
+
+
+class Runtime:
+    def __init__(self, arch, config, tmp_dir=None, libname=None):
+        self.arch = arch
+        self.config = config
+        self.tmp_dir = tmp_dir
+        self.libname = libname
+        if self.libname is None:
+            self.libname = self.compile()
+        if self.libname is None:
+            log = codegen.library_path(config, tmp_dir)[:-3] + ".log"
+            raise KernelLaunchError(f"could not build kernel library for {config.operation}:{config} (see {log})")
+
+    def compile(self, timeout=None):
+        return codegen.compile_config(self.config, self.arch, self.tmp_dir, timeout)
+
+    def _path(self):
+        if os.path.isabs(self.libname):
+            return self.libname
+        return os.path.join(self.tmp_dir or codegen.DEFAULT_BUILD_DIR, self.libname)
+
+    def workspace_size(self, B, H, Sq, Sk):
+        return int(library.load(self._path(), self.config.operation).workspace_size(B, H, Sq, Sk))
+
+    def apply(self, torch_array, device=None, softmax_scale=None, causal=False, workspace=None):
+        q, k = torch_array[0], torch_array[1]
+        if not q.is_cuda:
+            raise KernelLaunchError("kernel libraries run on the GPU only; got CPU tensors")
+        B, H, Sq, Sk = int(q.shape[0]), int(q.shape[1]), int(q.shape[2]), int(k.shape[2])
+        op = self.config.operation
+        lib = library.load(self._path(), op)
+        need = int(lib.workspace_size(B, H, Sq, Sk))
+        if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        ws_ptr = ctypes.c_void_p(workspace.data_ptr() if workspace is not None else 0)
+        ws_bytes = ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0)
+        if op == "attn":
+            scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])
+            extra = [ctypes.c_float(scale), ctypes.c_int(int(bool(causal)))]
+        else:
+            extra = [ctypes.c_int(int(bool(causal)))]
+        with torch.cuda.device(q.device):
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            rc = lib.kernel_entry_ex(*[ctypes.c_void_p(t.data_ptr()) for t in torch_array], B, H, Sq, Sk,
+                                     *extra, ws_ptr, ws_bytes, stream)
+        if rc != 0:
+            raise KernelLaunchError(f"{op}:{self.config} failed with code {rc}: {_ERRORS.get(rc, 'HIP error')}")
+        return rc
+
+
+def compile_parallel(configs, arch, tmp_dir=None):
+    return codegen.compile_parallel(configs, arch, tmp_dir)

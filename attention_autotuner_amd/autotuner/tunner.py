@@ -1,0 +1,84 @@
+"""Per-operator tuners (reference python/autotuner/tunner.py:13-225).
+
+Each tuner picks its search space from the architecture's platform: "ROCm" uses the gfx950 space,
+"CUDA" uses the restated reference space (enumeration only -- those configurations cannot be built
+here and ``tune`` refuses to try).
+"""
+import ctypes
+import math
+
+from . import gfx950_space, legacy_space
+from .base_tunner import BaseTunner
+
+
+def _is_rocm(arch):
+    return getattr(arch, "platform", "") == "ROCm"
+
+
+class _ForwardTunner(BaseTunner):
+    def __init__(self, arch, torch_array, op_name, **kw):
+        super().__init__(arch, torch_array, op_name, **kw)
+        if _is_rocm(arch):
+            self.Br_list = list(gfx950_space.BR_LIST)
+            self.Bc_list = list(gfx950_space.BC_LIST)
+
+    def generate_configs(self, Br, Bc, dim_qk, dim_v):
+        space = gfx950_space if _is_rocm(self.arch) else legacy_space
+        return space.forward_candidates(self.operation, Br, Bc, dim_qk, dim_v)
+
+    def _validate(self, config):
+        space = gfx950_space if _is_rocm(self.arch) else legacy_space
+        return space.forward_valid(config, self.arch)
+
+    validate_register_fuse = _validate
+    validate_shared_fuse = _validate
+
+    def tune(self, *a, **kw):
+        if not _is_rocm(self.arch):
+            raise RuntimeError(f"{self.arch.name} configurations can be enumerated but not built on this platform")
+        return super().tune(*a, **kw)
+
+
+class AttnTunner(_ForwardTunner):
+    operation = "attn"
+
+    def __init__(self, arch, torch_array, causal=False, softmax_scale=None):
+        super().__init__(arch, torch_array, "attention", causal=causal, softmax_scale=softmax_scale)
+
+    def _ex_args(self):
+        scale = self.softmax_scale
+        if scale is None:
+            scale = 1.0 / math.sqrt(self.problem_key["dim_qk"])
+        return [ctypes.c_float(scale), ctypes.c_int(int(self.causal))]
+
+
+class RetTunner(_ForwardTunner):
+    operation = "ret"
+
+    def __init__(self, arch, torch_array, causal=False):
+        super().__init__(arch, torch_array, "retnet", causal=causal)
+
+
+class RetBwdTunner(BaseTunner):
+    operation = "ret_bwd"
+
+    def __init__(self, arch, torch_array, causal=False):
+        super().__init__(arch, torch_array, "retnet_bwd", causal=causal)
+        if _is_rocm(arch):
+            self.Br_list = list(getattr(gfx950_space, "BWD_BR_LIST", (64, 128)))
+            self.Bc_list = list(getattr(gfx950_space, "BWD_BC_LIST", (32, 64, 128)))
+
+    def generate_configs(self, Br, Bc, dim_qk, dim_v):
+        if _is_rocm(self.arch):
+            return gfx950_space.backward_candidates(Br, Bc, dim_qk, dim_v)
+        return legacy_space.backward_candidates(Br, Bc, dim_qk, dim_v)
+
+    def validate_kernel(self, config):
+        if _is_rocm(self.arch):
+            return gfx950_space.backward_valid(config, self.arch)
+        return legacy_space.backward_valid(config, self.arch)
+
+    def tune(self, *a, **kw):
+        if not _is_rocm(self.arch):
+            raise RuntimeError(f"{self.arch.name} configurations can be enumerated but not built on this platform")
+        return super().tune(*a, **kw)

@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Headline benchmark: flash-attention forward, B4 H32 S2048 D128 fp16, non-causal, on one MI355X.
+
+A step is one launch of the fused forward kernel, through the C ABI of its config library, on inputs
+already resident in HBM.  Prints one JSON line (throughput in TFLOP/s with the dominant kernel's MFMA
+roofline fraction and a host-CPU baseline of the same math), preceded by human-readable lines on
+stderr.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+os.environ.setdefault("AAT_TUNE_ON_MISS", "0")
+
+PEAK_TFLOPS = 2500.0          # MI355X dense fp16 MFMA
+B, H, S, D = 4, 32, 2048, 128
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def attn_flops(b, h, sq, sk, dqk, dv, causal=False):
+    f = 2.0 * b * h * sq * sk * (dqk + dv)
+    return f / 2 if causal else f
+
+
+def resolve_config(aat, arch, tensors, causal):
+    from attention_autotuner_amd.autotuner import AttnTunner, gfx950_space
+    t = AttnTunner(arch, tensors, causal=causal)
+    cfg = t.check_cache()
+    if cfg is None:
+        q, k, v = tensors[:3]
+        cfg = gfx950_space.default_forward_config("attn", q.shape[-1], v.shape[-1], arch, q.shape[2], k.shape[2])
+    return cfg
+
+
+def time_launches(fn, steps, warmup):
+    """(wall ms per step, mean kernel ms from per-launch events on the launch stream)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        fn()
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    kern_ms = sum(s.elapsed_time(e) for s, e in zip(starts, stops)) / steps
+    return wall_ms, kern_ms
+
+
+def cpu_baseline(heads=8):
+    """The oracle's fp32 torch attention on the host cores, on `heads` (batch, head) slices of the
+    headline shape (slices are independent, so throughput per slice is representative)."""
+    import torch
+    from oracle import ref_op
+    torch.set_num_threads(os.cpu_count() or 1)
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, heads, S, D, generator=g).half()
+    k = torch.randn(1, heads, S, D, generator=g).half()
+    v = torch.randn(1, heads, S, D, generator=g).half()
+    ref_op.attention_ref(q[:, :1], k[:, :1], v[:, :1])                   # warm-up
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ref_op.attention_ref(q, k, v)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[1]
+    tflops = attn_flops(1, heads, S, S, D, D) / med / 1e12
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = next((l.split(":", 1)[1].strip() for l in f if l.startswith("model name")), "")
+    except OSError:
+        pass
+    return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle attention_ref fp32, {heads} of {B * H} (batch,head) slices of S={S} D={D}, median of 3: {med * 1e3:.0f} ms",
+            "cpu_model": model, "os_cpu_count": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the causal / long-kv / RetNet side measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: the path has no cross-GPU component (batch x head slices are independent); run with --gpus 1")
+        sys.exit(2)
+
+    import torch
+    import attention_autotuner_amd as aat
+    from attention_autotuner_amd.autotuner import Runtime
+
+    if not torch.cuda.is_available():
+        log("bench.py needs a GPU")
+        sys.exit(1)
+    arch = aat.MI355X()
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+
+    def mk(*shape):
+        return torch.randn(*shape, generator=g).half().to(dev)
+
+    q, k, v = mk(B, H, S, D), mk(B, H, S, D), mk(B, H, S, D)
+    o = torch.empty(B, H, S, D, dtype=torch.float16, device=dev)
+    scale = 1.0 / math.sqrt(D)
+
+    cfg = resolve_config(aat, arch, [q, k, v, o], False)
+    rt = Runtime(arch, cfg)
+    log(f"config: {cfg!r}")
+    wall_ms, kern_ms = time_launches(lambda: rt.apply([q, k, v, o], softmax_scale=scale, causal=False), args.steps, args.warmup)
+    flops = attn_flops(B, H, S, S, D, D)
+    value = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+    log(f"attention fwd non-causal: {wall_ms:.4f} ms/step wall, {kern_ms:.4f} ms/launch (events) -> {achieved:.1f} TFLOP/s = {100 * achieved / PEAK_TFLOPS:.1f}% of peak")
+
+    extras = {}
+    if not args.no_extras:
+        try:
+            extras.update(side_measurements(aat, arch, Runtime, mk, max(20, args.steps // 4), max(5, args.warmup // 4)))
+        except Exception as e:                       # side numbers never invalidate the headline
+            log(f"side measurements failed: {e!r}")
+
+    out = {
+        "metric": "attention fwd TFLOP/s (B4 H32 S2048 D128 fp16, non-causal)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": "configs[1]: flash-attention forward q,k,v [4,32,2048,128] fp16 N(0,1), scale 1/sqrt(128), non-causal",
+                   "kernel_config": str(cfg), "pct_of_fp16_mfma_peak": round(100 * value / PEAK_TFLOPS, 2)},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "flashattn_fwd_" + ("regfuse" if cfg.fuse_type == "register" else "smemfuse"),
+                     "launch_ms": round(kern_ms, 5), "algorithmic_flops_per_launch": flops},
+        "extras": extras,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+        log(f"cpu baseline: {out['cpu_baseline']}")
+    print(json.dumps(out), flush=True)
+
+
+def side_measurements(aat, arch, Runtime, mk, steps, warmup):
+    """Causal headline, the long-kv shape and RetNet forward/backward, when their kernels exist."""
+    import torch
+    res = {}
+    q, k, v = mk(B, H, S, D), mk(B, H, S, D), mk(B, H, S, D)
+    o = torch.empty_like(q)
+    cfg = resolve_config(aat, arch, [q, k, v, o], True)
+    rt = Runtime(arch, cfg)
+    _, ms = time_launches(lambda: rt.apply([q, k, v, o], causal=True), steps, warmup)
+    res["attn_causal_b4h32s2048d128"] = {"ms": round(ms, 5), "tflops": round(attn_flops(B, H, S, S, D, D, True) / ms / 1e9, 1), "config": str(cfg)}
+    log(f"attention fwd causal: {ms:.4f} ms -> {res['attn_causal_b4h32s2048d128']['tflops']} TFLOP/s")
+
+    q5, k5, v5 = mk(1, 32, 256, D), mk(1, 32, 16384, D), mk(1, 32, 16384, D)
+    o5 = torch.empty_like(q5)
+    cfg5 = resolve_config(aat, arch, [q5, k5, v5, o5], False)
+    rt5 = Runtime(arch, cfg5)
+    _, ms = time_launches(lambda: rt5.apply([q5, k5, v5, o5]), steps, warmup)
+    bytes5 = 2 * (q5.numel() + k5.numel() + v5.numel() + o5.numel())
+    res["attn_longkv_b1h32q256k16384d128"] = {"ms": round(ms, 5), "tflops": round(attn_flops(1, 32, 256, 16384, D, D) / ms / 1e9, 1),
+                                              "gbps": round(bytes5 / ms / 1e6, 1), "config": str(cfg5)}
+    log(f"attention fwd long-kv: {ms:.4f} ms -> {res['attn_longkv_b1h32q256k16384d128']}")
+    res.update(retnet_measurements(aat, arch, mk, steps, warmup))
+    return res
+
+
+def retnet_measurements(aat, arch, mk, steps, warmup):
+    import torch
+    from attention_autotuner_amd.autotuner import gfx950_space
+    res = {}
+    if not hasattr(gfx950_space, "default_backward_config"):
+        return res
+    from oracle import ref_op
+    b, h, s, dqk, dv = 4, 8, 2048, 256, 512
+    q, k, v, do = mk(b, h, s, dqk), mk(b, h, s, dqk), mk(b, h, s, dv), mk(b, h, s, dv)
+    mask = ref_op.retnet_decay_mask(h, s, s).cuda()
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    fwd_flops = 2.0 * b * h * s * s * (dqk + dv)
+    bwd_flops = 2.0 * b * h * s * s * (3 * dqk + 2 * dv)
+    with torch.no_grad():
+        _, ms_f = time_launches(lambda: aat.RetNetAttnFunc(q, k, v, mask, arch), steps, warmup)
+    res["retnet_fwd_b4h8s2048_dqk256_dv512"] = {"ms": round(ms_f, 5), "tflops": round(fwd_flops / ms_f / 1e9, 1)}
+    log(f"retnet fwd: {ms_f:.4f} ms -> {fwd_flops / ms_f / 1e9:.1f} TFLOP/s")
+
+    def fb():
+        q.grad = k.grad = v.grad = None
+        aat.RetNetAttnFunc(q, k, v, mask, arch).backward(do)
+
+    _, ms_fb = time_launches(fb, steps, warmup)
+    res["retnet_fwd_bwd_b4h8s2048_dqk256_dv512"] = {"ms": round(ms_fb, 5), "tflops": round((fwd_flops + bwd_flops) / ms_fb / 1e9, 1)}
+    log(f"retnet fwd+bwd: {ms_fb:.4f} ms -> {(fwd_flops + bwd_flops) / ms_fb / 1e9:.1f} TFLOP/s (dense-mask FLOPs)")
+    return res
+
+
+if __name__ == "__main__":
+    main()

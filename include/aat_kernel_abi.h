@@ -1,0 +1,98 @@
+/* C ABI of one compiled kernel configuration ("config library").
+ *
+ * The autotuner turns every candidate configuration (tile sizes, wave count, LDS buffering, fuse
+ * type) into its own shared object, exactly as the reference does, and binds it with ctypes.  Each
+ * such library exports the symbols declared below for ONE operator; which operator is selected at
+ * compile time by defining AAT_OP_ATTN, AAT_OP_RET or AAT_OP_RET_BWD before including this header
+ * (the generated wrapper does that, so the compiler checks the definitions against this file).
+ *
+ * Conventions (same as the reference unless stated):
+ *   - all tensors are contiguous row-major device buffers owned by the caller; nothing is allocated,
+ *     freed or retained by the callee;
+ *   - q [B,H,Seq_q,Kd], k [B,H,Seq_k,Kd], v [B,H,Seq_k,D], o/dO [B,H,Seq_q,D] are IEEE fp16;
+ *     mask [H,Seq_q,Seq_k] fp16; r [B,H,Seq_q] fp32; dqaccum [B,H,Seq_q,Kd] fp32, zero on entry;
+ *   - Kd, D and the tile shape are baked into the library (see config_string());
+ *   - Seq_q must be a multiple of the library's Br and Seq_k of its Bc;
+ *   - `profile*` launches the kernel repeatedly (one probe launch, then ceil(100 ms / t) launches) and
+ *     returns the mean time of one launch in milliseconds, or -1 on any error;
+ *   - `kernel_entry*` enqueues one launch and returns without synchronising.
+ *
+ * Differences from the reference, all additive:
+ *   - the two reference-signature entry points keep the reference's argument ORDER, including the
+ *     swapped (Seq_k, Seq_q) of kernel_entry, and its literal behaviour: softmax scale 0.125, no causal
+ *     masking, null stream.  kernel_entry returns 0 on success (the reference always returns 0),
+ *     a positive hipError_t on a launch failure, AAT_ERR_SHAPE for an indivisible shape;
+ *   - the *_ex entry points take (Seq_q, Seq_k) in that order plus a runtime softmax scale, a causal
+ *     flag, an optional workspace and the stream to launch on (a hipStream_t passed as void*);
+ *   - workspace_size() says how many bytes of workspace a problem needs (0 unless the configuration
+ *     splits the kv range); abi_version() and config_string() identify the library.
+ */
+#ifndef AAT_KERNEL_ABI_H
+#define AAT_KERNEL_ABI_H
+
+#include <stddef.h>
+
+#define AAT_ABI_VERSION 1
+#define AAT_ERR_SHAPE (-2)      /* Seq_q / Seq_k not divisible by the tile, or a non-positive size */
+#define AAT_ERR_WORKSPACE (-3)  /* workspace missing or smaller than workspace_size() */
+
+typedef unsigned short aat_half; /* raw IEEE binary16 bits */
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Common to every config library. */
+int abi_version(void);
+const char* config_string(void);
+size_t workspace_size(int B, int H, int Seq_q, int Seq_k);
+
+#if defined(AAT_OP_ATTN)
+/* Flash-attention forward.  Replaces: reference csrc/kernels/attention/regfuse/profile_code.py:30
+ * (profile) and :68 (kernel_entry); csrc/kernels/attention/smemfuse/profile_code.py has the same pair.
+ * Bound by reference python/autotuner/base_tunner.py:96-110 and python/autotuner/runtime.py:74-82. */
+float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k);
+int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_k, int Seq_q);
+float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q,
+                 int Seq_k, float softmax_scale, int causal, void* workspace, size_t workspace_bytes,
+                 void* stream);
+int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q,
+                    int Seq_k, float softmax_scale, int causal, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+#elif defined(AAT_OP_RET)
+/* RetNet parallel forward.  Replaces: reference csrc/kernels/retnet/regfuse/profile_code.py:34 and :72
+ * (and the smemfuse pair).  `causal` != 0 promises that mask is zero above the diagonal so those
+ * tiles may be skipped. */
+float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* o, float* r, int B,
+              int H, int Seq_q, int Seq_k);
+int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* o, float* r, int B,
+                 int H, int Seq_k, int Seq_q);
+float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* o, float* r, int B,
+                 int H, int Seq_q, int Seq_k, int causal, void* workspace, size_t workspace_bytes,
+                 void* stream);
+int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* o, float* r,
+                    int B, int H, int Seq_q, int Seq_k, int causal, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+#elif defined(AAT_OP_RET_BWD)
+/* RetNet parallel backward.  Replaces: reference csrc/kernels/retnet/bwd/profile_code.py:53 and :98.
+ * dqaccum is fp32 scratch the caller has zeroed; dq, dk, dv are fully overwritten. */
+float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
+              aat_half* dq, aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q,
+              int Seq_k);
+int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
+                 aat_half* dq, aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_k,
+                 int Seq_q);
+float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
+                 aat_half* dq, aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q,
+                 int Seq_k, int causal, void* workspace, size_t workspace_bytes, void* stream);
+int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
+                    aat_half* dq, aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q,
+                    int Seq_k, int causal, void* workspace, size_t workspace_bytes, void* stream);
+#endif
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AAT_KERNEL_ABI_H */

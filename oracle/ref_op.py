@@ -83,7 +83,7 @@ def retnet_decay_mask(nheads, seq_q, seq_k, dtype=torch.float16):
     m = torch.arange(seq_k, dtype=torch.float64).view(1, 1, seq_k)
     gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(nheads, dtype=torch.float64)).view(nheads, 1, 1)
     d = torch.where(n >= m, gamma ** (n - m).clamp(min=0), torch.zeros((), dtype=torch.float64))
-    return d.to(torch.float32).to(dtype)
+    return d.to(dtype) if dtype == torch.float64 else d.to(torch.float32).to(dtype)
 
 
 def attention_online_ref(q, k, v, softmax_scale=None, causal=False, block_kv=64):

@@ -1,0 +1,141 @@
+"""GPU parity of the attention forward kernels against the CPU oracle, through the C ABI.
+
+Tolerance: max-abs error <= 2e-3 on fp16 outputs versus the fp32 oracle on the same seeded inputs.
+"""
+import ctypes
+import math
+import os
+
+import pytest
+import torch
+
+import attention_autotuner_amd as aat
+from attention_autotuner_amd.arch import MI355X
+from attention_autotuner_amd.autotuner import AttnConfig, Runtime, codegen, gfx950_space, library
+from attention_autotuner_amd.autotuner.runtime import KernelLaunchError
+from oracle import ref_op
+
+pytestmark = pytest.mark.gpu
+ARCH = MI355X()
+TOL = 2e-3
+
+
+def _inputs(b, h, sq, sk, dqk, dv, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, h, sq, dqk, generator=g).half()
+    k = torch.randn(b, h, sk, dqk, generator=g).half()
+    v = torch.randn(b, h, sk, dv, generator=g).half()
+    return q, k, v
+
+
+def _err(o, ref):
+    return (o.float().cpu() - ref).abs().max().item()
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_config1_plumbing_b2_h8_s512_d64(causal):
+    q, k, v = _inputs(2, 8, 512, 512, 64, 64)
+    o = aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH, causal)
+    assert o.shape == (2, 8, 512, 64) and o.dtype == torch.float16
+    assert _err(o, ref_op.attention_ref(q, k, v, 1 / math.sqrt(64), causal)) <= TOL
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_config2_headline_b4_h32_s2048_d128(causal):
+    q, k, v = _inputs(4, 32, 2048, 2048, 128, 128, seed=1)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    o = aat.flash_attn_func(qc, kc, vc, ARCH, causal)
+    # the oracle on a sample of (batch, head) slices: slices are independent
+    for b, h in ((0, 0), (1, 7), (3, 31)):
+        ref = ref_op.attention_ref(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], None, causal)
+        assert _err(o[b:b + 1, h:h + 1], ref) <= TOL
+    # size-independent properties on the whole problem
+    ones = torch.ones_like(vc)
+    o1 = aat.flash_attn_func(qc, kc, ones, ARCH, causal)
+    assert (o1.float() - 1).abs().max().item() <= 1e-3            # rows of P sum to one
+    o0 = aat.flash_attn_func(qc, kc, vc, ARCH, causal, 0.0)        # scale 0: (prefix) mean of V
+    if causal:
+        want = torch.cumsum(vc.float(), dim=2) / torch.arange(1, 2049, device="cuda").view(1, 1, -1, 1)
+    else:
+        want = vc.float().mean(dim=2, keepdim=True).expand_as(o0)
+    assert (o0.float() - want).abs().max().item() <= TOL
+    again = aat.flash_attn_func(qc, kc, vc, ARCH, causal)
+    assert torch.equal(o, again)                                    # deterministic
+
+
+def test_config5_long_kv_b1_h32_sq256_sk16384_d128():
+    q, k, v = _inputs(1, 32, 256, 16384, 128, 128, seed=2)
+    o = aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH)
+    assert _err(o, ref_op.attention_ref(q, k, v)) <= TOL
+
+
+def test_reference_literal_scale_and_explicit_scale():
+    q, k, v = _inputs(1, 4, 256, 256, 128, 128, seed=3)
+    o = aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH, False, aat.REFERENCE_SOFTMAX_SCALE)
+    assert _err(o, ref_op.attention_ref(q, k, v, 0.125)) <= TOL
+    o = aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH, False, 0.05)
+    assert _err(o, ref_op.attention_ref(q, k, v, 0.05)) <= TOL
+
+
+def test_scaled_inputs_like_the_reference_tuner_demo():
+    # the reference's tuner driver uses k, v = 3 * randn: sharper softmax
+    q, k, v = _inputs(1, 4, 256, 512, 64, 64, seed=4)
+    k, v = (3 * k.float()).half(), (3 * v.float()).half()
+    o = aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH)
+    assert _err(o, ref_op.attention_ref(q, k, v)) <= 3 * TOL      # |v| is 3x larger
+
+
+from attention_autotuner_amd.autotuner.prebuilt import PARITY_DIMS, PARITY_TILES as CONFIGS
+
+
+@pytest.mark.parametrize("dqk,dv", PARITY_DIMS)
+def test_every_configuration_agrees_with_the_oracle(dqk, dv):
+    q, k, v = _inputs(1, 2, 256, 512, dqk, dv, seed=5)
+    refs = {c: ref_op.attention_ref(q, k, v, None, c) for c in (False, True)}
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    ran = 0
+    for br, bc, nt, sq, sv, wpe in CONFIGS:
+        cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+        if not gfx950_space.forward_valid(cfg, ARCH):
+            continue
+        assert os.path.exists(codegen.library_path(cfg)), f"library for {cfg} was not built ahead of time"
+        for causal in (False, True):
+            o = torch.zeros(1, 2, 256, dv, dtype=torch.float16, device="cuda")
+            Runtime(ARCH, cfg).apply([qc, kc, vc, o], causal=causal)
+            assert _err(o, refs[causal]) <= TOL, (cfg, causal)
+        ran += 1
+    assert ran >= 3
+
+
+def test_reference_signature_entry_points():
+    """profile / kernel_entry keep the reference's argument order (kernel_entry swaps the lengths)
+    and its literal behaviour: scale 0.125, non-causal, null stream."""
+    q, k, v = _inputs(1, 2, 256, 512, 128, 128, seed=6)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros(1, 2, 256, 128, dtype=torch.float16, device="cuda")
+    cfg = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
+    lib = library.load(Runtime(ARCH, cfg)._path(), "attn")
+    ptrs = [ctypes.c_void_p(t.data_ptr()) for t in (qc, kc, vc, o)]
+    torch.cuda.synchronize()
+    assert lib.kernel_entry(*ptrs, 1, 2, 512, 256) == 0          # (B, H, Seq_k, Seq_q)
+    torch.cuda.synchronize()
+    assert _err(o, ref_op.attention_ref(q, k, v, 0.125)) <= TOL
+    ms = lib.profile(*ptrs, 1, 2, 256, 512)                       # (B, H, Seq_q, Seq_k)
+    assert 0 < ms < 50
+    assert lib.kernel_entry(*ptrs, 1, 2, 500, 256) == -2          # indivisible: refused, nothing launched
+    assert lib.profile(*ptrs, 1, 2, 256, 500) == -1
+
+
+def test_indivisible_shape_raises():
+    q, k, v = _inputs(1, 1, 128, 96, 64, 64)
+    with pytest.raises((KernelLaunchError, ValueError)):
+        aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH)
+
+
+def test_runs_on_the_current_stream():
+    q, k, v = _inputs(1, 2, 256, 256, 64, 64, seed=7)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        o = aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH)
+    s.synchronize()
+    assert _err(o, ref_op.attention_ref(q, k, v)) <= TOL

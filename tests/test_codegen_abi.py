@@ -1,0 +1,139 @@
+"""Host-side checks that run without a GPU: wrapper text, hipcc compile for gfx950, exported symbols
+versus include/aat_kernel_abi.h, failure handling of the compile driver and of the tuning cache."""
+import ctypes
+import json
+import os
+import re
+
+import pytest
+import torch
+
+from attention_autotuner_amd.arch import MI355X
+from attention_autotuner_amd.autotuner import AttnConfig, AttnTunner, Runtime, codegen, gfx950_space, library, prebuilt
+from attention_autotuner_amd.autotuner import base_tunner
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "aat_kernel_abi.h")
+ARCH = MI355X()
+
+
+def _declared_symbols(op_macro):
+    """Function names include/aat_kernel_abi.h declares for one operator."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    common = text.split("#if defined(AAT_OP_ATTN)")[0]
+    block = re.search(r"defined\(%s\)(.*?)(#elif|#endif)" % op_macro, text, flags=re.S).group(1)
+    names = re.findall(r"\b([a-z_]+)\s*\(", common + block)
+    return sorted(set(n for n in names if n not in ("defined",)))
+
+
+def test_header_declares_the_reference_pair_for_every_operator():
+    for macro in ("AAT_OP_ATTN", "AAT_OP_RET", "AAT_OP_RET_BWD"):
+        names = _declared_symbols(macro)
+        assert names == ["abi_version", "config_string", "kernel_entry", "kernel_entry_ex", "profile", "profile_ex", "workspace_size"]
+
+
+def test_wrapper_text_carries_the_configuration():
+    cfg = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
+    src = codegen.render(cfg)
+    for field in ("Br", "Bc", "Kd", "D", "Nthreads", "num_stages_qk", "num_stages_v"):
+        assert f"constexpr int {field} = {getattr(cfg, field)};" in src
+    assert 'extern "C" float profile(' in src and 'extern "C" int kernel_entry(' in src
+    assert "int Seq_k, int Seq_q)" in src.split('extern "C" int kernel_entry(')[1].split("{")[0]   # reference order
+    assert "int Seq_q, int Seq_k)" in src.split('extern "C" float profile(')[1].split("{")[0]
+    cmd = codegen.hipcc_command("a.hip", "a.so", ARCH)
+    assert "--offload-arch=gfx950" in cmd and "-packed-fp32-ops" in cmd
+
+
+def test_shipping_set_is_built_and_exports_the_abi():
+    cfgs = prebuilt.shipping_set(ARCH)
+    assert cfgs
+    macro = {"attn": "AAT_OP_ATTN", "ret": "AAT_OP_RET", "ret_bwd": "AAT_OP_RET_BWD"}
+    for cfg in cfgs:
+        path = codegen.compile_config(cfg, ARCH, timeout=600)          # already built by build(); builds if not
+        assert path and os.path.exists(path), cfg
+        raw = ctypes.CDLL(path)
+        for name in _declared_symbols(macro[cfg.operation]):
+            assert hasattr(raw, name), (cfg, name)
+        lib = library.load(path, cfg.operation)
+        assert lib.abi_version() == 1
+        assert lib.config_string().decode() == f"{cfg.operation}:{cfg}"
+        if getattr(cfg, "kv_splits", 1) == 1:
+            assert lib.workspace_size(1, 1, 256, 256) == 0
+
+
+def test_failed_compile_is_skipped_not_fatal(tmp_path):
+    bad = AttnConfig(96, 64, 128, 128, 128, 64, 1, 1, 256, True).set_fuse_type("register")   # 96 rows / 4 waves: static_assert
+    assert codegen.compile_config(bad, ARCH, str(tmp_path), timeout=120) is None
+    logs = [f for f in os.listdir(tmp_path / "attn") if f.endswith(".log")]
+    assert logs and "static assertion" in open(tmp_path / "attn" / logs[0]).read()
+    with pytest.raises(Exception):
+        Runtime(ARCH, bad, tmp_dir=str(tmp_path))
+    good = gfx950_space.default_forward_config("attn", 64, 64, ARCH)
+    res = codegen.compile_parallel([bad, good], ARCH, str(tmp_path), timeout=300)
+    assert res[0] is None and res[1] and os.path.exists(res[1])
+
+
+def test_compile_timeout_yields_none(tmp_path):
+    cfg = gfx950_space.default_forward_config("attn", 64, 64, ARCH)
+    assert codegen.compile_config(cfg, ARCH, str(tmp_path), timeout=0.05) is None
+    assert not [f for f in os.listdir(tmp_path / "attn") if f.endswith(".so")]
+
+
+def _meta(dqk=128, dv=128, sq=2048, sk=2048):
+    return [torch.empty(4, 32, sq, dqk, dtype=torch.float16, device="meta"),
+            torch.empty(4, 32, sk, dqk, dtype=torch.float16, device="meta"),
+            torch.empty(4, 32, sk, dv, dtype=torch.float16, device="meta")]
+
+
+def test_cache_roundtrip_corruption_and_key(tmp_path, monkeypatch):
+    base_tunner._memo.clear()
+    t = AttnTunner(ARCH, _meta(), causal=True)
+    t.cache_path = str(tmp_path)
+    assert t.check_cache() is None
+    cfg = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
+    t._write_cache(cfg)
+    base_tunner._memo.clear()
+    assert t.check_cache() == cfg
+    name = os.path.basename(t._cache_file())
+    assert name == "best_config_attention_MI355X_128_128_b4h32q2048k2048_c1.json"
+    # a different problem (non-causal, other lengths) does not see that entry
+    t2 = AttnTunner(ARCH, _meta(sq=256, sk=16384), causal=False)
+    t2.cache_path = str(tmp_path)
+    assert t2.check_cache() is None
+    # the reference's file name is honoured as a fallback
+    with open(tmp_path / "best_config_attention_128_128.json", "w") as f:
+        json.dump(cfg.to_dict(), f)
+    assert t2.check_cache() == cfg
+    # corrupt files are ignored
+    base_tunner._memo.clear()
+    with open(t._cache_file(), "w") as f:
+        f.write("{not json")
+    os.remove(tmp_path / "best_config_attention_128_128.json")
+    assert t.check_cache() is None
+    # a cached tile that does not divide the problem is ignored
+    t3 = AttnTunner(ARCH, _meta(sq=64, sk=2048), causal=True)
+    t3.cache_path = str(tmp_path)
+    with open(t3._cache_file(), "w") as f:
+        json.dump(cfg.to_dict(), f)
+    assert cfg.Br == 128 and t3.check_cache() is None
+
+
+def test_validity_model_rejects_over_lds_and_over_register():
+    over_lds = AttnConfig(128, 128, 256, 512, 256, 128, 2, 2, 256, True, waves_per_eu=1).set_fuse_type("register")
+    assert gfx950_space.forward_lds_bytes(over_lds) > ARCH.smem_cap
+    assert not gfx950_space.forward_valid(over_lds, ARCH)
+    over_reg = AttnConfig(128, 64, 256, 512, 256, 64, 1, 1, 128, True, waves_per_eu=2).set_fuse_type("register")
+    assert not gfx950_space.forward_valid(over_reg, ARCH)
+    ok = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
+    assert gfx950_space.forward_valid(ok, ARCH)
+    assert gfx950_space.forward_lds_bytes(ok) == 2 * 64 * 128 * 2 * 2
+
+
+def test_ops_refuse_cpu_tensors():
+    import attention_autotuner_amd as aat
+    q = torch.zeros(1, 1, 128, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        aat.flash_attn_func(q, q, q, ARCH)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        aat.RetNetAttnFunc(q, q, q, torch.zeros(1, 128, 128, dtype=torch.float16), ARCH)

@@ -1,0 +1,192 @@
+"""Pins oracle/ref_op.py: library routines, fp64 brute force, closed forms, autograd, gradcheck.
+
+Each check is chosen so that a plausible slip in the restatement (dropped scale, mask applied after
+the abs-sum, missing clamp, transposed operand, r not detached) fails at least one of them.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import brute, ref_op
+
+
+def _rand(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).half()
+
+
+# ---------------------------------------------------------------------------------- attention
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("sq,sk", [(32, 32), (16, 48)])
+def test_attention_matches_torch_sdpa(causal, sq, sk):
+    if causal and sq != sk:
+        pytest.skip("torch's is_causal aligns top-left; bottom-right alignment is checked by brute force")
+    q, k, v = _rand(2, 3, sq, 64, seed=1), _rand(2, 3, sk, 64, seed=2), _rand(2, 3, sk, 128, seed=3)
+    for scale in (0.125, 1 / math.sqrt(64), 0.3):
+        want = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), scale=scale, is_causal=causal)
+        got = ref_op.attention_ref(q, k, v, softmax_scale=scale, causal=causal)
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("sq,sk", [(8, 8), (4, 12), (12, 4)])
+def test_attention_matches_fp64_brute_force(causal, sq, sk):
+    q, k, v = _rand(1, 2, sq, 64, seed=4), _rand(1, 2, sk, 64, seed=5), _rand(1, 2, sk, 64, seed=6)
+    want = brute.attention_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), 0.2, causal)
+    got = ref_op.attention_ref(q, k, v, softmax_scale=0.2, causal=causal).numpy()
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
+
+
+def test_attention_closed_forms():
+    q, k, v = _rand(1, 2, 16, 64, seed=7), _rand(1, 2, 16, 64, seed=8), _rand(1, 2, 16, 64, seed=9)
+    ones = torch.ones_like(v)
+    torch.testing.assert_close(ref_op.attention_ref(q, k, ones), ones.float())                      # rows of P sum to 1
+    mean_v = v.float().mean(dim=-2, keepdim=True).expand(-1, -1, 16, -1)
+    torch.testing.assert_close(ref_op.attention_ref(q, k, v, softmax_scale=0.0), mean_v)            # scale 0 -> mean
+    same_k = k[..., :1, :].expand_as(k)
+    torch.testing.assert_close(ref_op.attention_ref(q, same_k, v), mean_v, rtol=1e-5, atol=1e-5)    # identical keys -> mean
+    prefix = torch.cumsum(v.float(), dim=-2) / torch.arange(1, 17).view(1, 1, 16, 1)
+    torch.testing.assert_close(ref_op.attention_ref(q, k, v, softmax_scale=0.0, causal=True), prefix)
+    torch.testing.assert_close(ref_op.attention_ref(q, k, v, causal=True)[..., 0, :], v.float()[..., 0, :])
+    perm = torch.randperm(16, generator=torch.Generator().manual_seed(0))                           # kv order is irrelevant
+    torch.testing.assert_close(ref_op.attention_ref(q, k[..., perm, :], v[..., perm, :]), ref_op.attention_ref(q, k, v))
+    eye = torch.eye(16).expand(1, 2, 16, 16).half()                                                 # one-hot V returns P
+    p = ref_op.attention_ref(q, k, eye, softmax_scale=0.125)
+    want = torch.softmax(q.float() @ k.float().transpose(-1, -2) * 0.125, dim=-1)
+    torch.testing.assert_close(p, want)
+    assert ref_op.REFERENCE_SOFTMAX_SCALE == 0.125
+    torch.testing.assert_close(ref_op.attention_ref(q, k, v), ref_op.attention_ref(q, k, v, softmax_scale=0.125))  # d=64
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_online_and_split_forms_agree(causal):
+    q, k, v = _rand(1, 2, 64, 64, seed=10), _rand(1, 2, 128, 64, seed=11), _rand(1, 2, 128, 64, seed=12)
+    full = ref_op.attention_ref(q, k, v, causal=causal)
+    online = ref_op.attention_online_ref(q, k, v, causal=causal, block_kv=32)
+    assert (full - online).abs().max() < 2e-3       # only P's fp16 rounding separates them
+    if not causal:
+        torch.testing.assert_close(ref_op.attention_split_merge_ref(q, k, v, n_splits=4), full, rtol=1e-5, atol=1e-5)
+
+
+def test_attention_lse():
+    q, k, v = _rand(1, 1, 8, 64, seed=13), _rand(1, 1, 8, 64, seed=14), _rand(1, 1, 8, 64, seed=15)
+    _, lse = ref_op.attention_ref(q, k, v, softmax_scale=0.125, return_lse=True)
+    want = torch.log(torch.exp(q.float() @ k.float().transpose(-1, -2) * 0.125).sum(-1))
+    torch.testing.assert_close(lse, want)
+
+
+# ---------------------------------------------------------------------------------- RetNet forward
+def test_decay_mask_closed_form():
+    m = ref_op.retnet_decay_mask(3, 8, 8, dtype=torch.float32)
+    for h in range(3):
+        g = 1 - 2.0 ** (-5 - h)
+        for n in range(8):
+            for j in range(8):
+                want = g ** (n - j) if n >= j else 0.0
+                assert abs(m[h, n, j].item() - want) < 1e-6
+    m16 = ref_op.retnet_decay_mask(2, 2048, 2048)
+    assert m16.dtype == torch.float16 and m16[0, 2047, 0] == 0 and m16[0, 5, 5] == 1       # fp16 underflow far from the diagonal
+
+
+def test_retnet_matches_fp64_brute_force():
+    q, k, v = _rand(2, 2, 8, 64, seed=20), _rand(2, 2, 12, 64, seed=21), _rand(2, 2, 12, 128, seed=22)
+    mask = _rand(2, 8, 12, seed=23)
+    o, r = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    bo, br = brute.retnet_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), mask.float().numpy())
+    np.testing.assert_allclose(o.numpy(), bo, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(r.numpy(), br, rtol=2e-5, atol=2e-5)
+
+
+def test_retnet_closed_forms():
+    q, k, v = _rand(1, 2, 16, 64, seed=24), _rand(1, 2, 16, 64, seed=25), _rand(1, 2, 16, 64, seed=26)
+    zero = torch.zeros(2, 16, 16).half()
+    o, r = ref_op.retnet_ref(q, k, v, zero, return_r=True)
+    assert o.abs().max() == 0 and (r == 1).all()                                       # M = 0
+    tiny_q = (q.float() * 1e-3).half()
+    ones = torch.ones(2, 16, 16).half()
+    o, r = ref_op.retnet_ref(tiny_q, k, v, ones, return_r=True)
+    assert (r == 1).all()                                                              # clamp active -> plain matmuls
+    torch.testing.assert_close(o, (tiny_q.float() @ k.float().transpose(-1, -2)) @ v.float())
+    mask = ref_op.retnet_decay_mask(2, 16, 16)
+    o1, r1 = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    assert (r1 > 1).all()
+    o2 = ref_op.retnet_ref((q.float() * 2).half(), k, v, mask)                          # r > 1: scale invariance in q
+    torch.testing.assert_close(o1, o2, rtol=1e-5, atol=1e-5)
+    s = (q.float() @ k.float().transpose(-1, -2)) * mask.float()
+    torch.testing.assert_close(r1, s.abs().sum(-1).clamp(min=1.0))
+    torch.testing.assert_close((s / r1.unsqueeze(-1)).abs().sum(-1), torch.ones_like(r1))
+    # numerator equals the recurrent form  S_n = gamma S_{n-1} + k_n^T v_n,  num_n = q_n S_n
+    # (unrounded decay mask here: the recurrence uses the exact gamma)
+    s = (q.double() @ k.double().transpose(-1, -2)) * ref_op.retnet_decay_mask(2, 16, 16, dtype=torch.float64)
+    for h in range(2):
+        g = 1 - 2.0 ** (-5 - h)
+        state = torch.zeros(64, 64, dtype=torch.float64)
+        for n in range(16):
+            state = g * state + k[0, h, n].double().unsqueeze(1) * v[0, h, n].double().unsqueeze(0)
+            num = q[0, h, n].double() @ state
+            want = (s[0, h, n].double() @ v[0, h].double())
+            torch.testing.assert_close(num, want, rtol=1e-6, atol=1e-6)
+
+
+def test_retnet_online_form_agrees():
+    q, k, v = _rand(1, 2, 32, 64, seed=27), _rand(1, 2, 128, 64, seed=28), _rand(1, 2, 128, 64, seed=29)
+    mask = _rand(2, 32, 128, seed=30, scale=0.5)
+    o, r = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    oo, ro = ref_op.retnet_online_ref(q, k, v, mask, block_kv=32)
+    torch.testing.assert_close(ro, r, rtol=1e-5, atol=1e-5)
+    assert (o - oo).abs().max() < 2e-3
+
+
+# ---------------------------------------------------------------------------------- RetNet backward
+def _autograd_grads(q, k, v, mask, do, dtype=torch.float32):
+    qq, kk, vv = (t.detach().to(dtype).requires_grad_(True) for t in (q, k, v))
+    s = (qq @ kk.transpose(-1, -2)) * mask.to(dtype)
+    r = s.detach().abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
+    o = (s / r) @ vv
+    o.backward(do.to(dtype))
+    return qq.grad, kk.grad, vv.grad
+
+
+def test_retnet_bwd_matches_autograd_and_brute_force():
+    q, k, v = _rand(2, 2, 8, 64, seed=31), _rand(2, 2, 12, 64, seed=32), _rand(2, 2, 12, 128, seed=33)
+    mask, do = _rand(2, 8, 12, seed=34), _rand(2, 2, 8, 128, seed=35)
+    got = ref_op.retnet_bwd_ref(q, k, v, mask, do)
+    want = _autograd_grads(q, k, v, mask, do)
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g, w, rtol=1e-4, atol=1e-4)
+    b = brute.retnet_bwd(*(t.float().numpy() for t in (q, k, v, mask, do)))
+    for g, w in zip(got, b):
+        np.testing.assert_allclose(g.numpy(), w, rtol=1e-4, atol=1e-4)
+
+
+def test_retnet_bwd_gradcheck_fp64():
+    g = torch.Generator().manual_seed(36)
+    q, k, v = (torch.randn(1, 1, 4, 6, generator=g, dtype=torch.float64) for _ in range(3))
+    mask = torch.randn(1, 4, 4, generator=g, dtype=torch.float64)
+    do = torch.randn(1, 1, 4, 6, generator=g, dtype=torch.float64)
+    r = ((q @ k.transpose(-1, -2)) * mask).abs().sum(-1, keepdim=True).clamp(min=1.0)
+
+    def f(qq, kk, vv):                         # r frozen, as the reference detaches it
+        return (((qq @ kk.transpose(-1, -2)) * mask) / r) @ vv
+
+    assert torch.autograd.gradcheck(f, tuple(t.clone().requires_grad_(True) for t in (q, k, v)), eps=1e-6, atol=1e-6)
+    want = torch.autograd.grad(f(*(t.requires_grad_(True) for t in (q, k, v))), (q, k, v), do)
+    got = ref_op.retnet_bwd_ref(q, k, v, mask, do)
+    for a, b in zip(got, want):
+        torch.testing.assert_close(a, b.float(), rtol=1e-4, atol=1e-4)
+
+
+def test_retnet_bwd_linearity_and_zero_mask():
+    q, k, v = _rand(1, 2, 8, 64, seed=37), _rand(1, 2, 8, 64, seed=38), _rand(1, 2, 8, 64, seed=39)
+    mask = _rand(2, 8, 8, seed=40)
+    d1, d2 = _rand(1, 2, 8, 64, seed=41), _rand(1, 2, 8, 64, seed=42)
+    g1 = ref_op.retnet_bwd_ref(q, k, v, mask, d1.float())
+    g2 = ref_op.retnet_bwd_ref(q, k, v, mask, d2.float())
+    g12 = ref_op.retnet_bwd_ref(q, k, v, mask, 2 * d1.float() - 3 * d2.float())
+    for a, b, c in zip(g1, g2, g12):
+        torch.testing.assert_close(2 * a - 3 * b, c, rtol=1e-4, atol=1e-4)
+    for g in ref_op.retnet_bwd_ref(q, k, v, torch.zeros_like(mask), d1):
+        assert g.abs().max() == 0
