@@ -16,6 +16,7 @@
 #pragma once
 #include "../../utils/cdna4.h"
 #include "../../utils/softmax.h"
+#include <type_traits>
 
 namespace aat {
 
@@ -128,7 +129,10 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     if constexpr (NSV == 2) vdma.issue(vg, vbuf, wave_base);
   }
 
-  for (int j = 0; j < n_tiles; ++j) {
+  // One kv tile.  MASKED is set for the tiles the causal diagonal crosses; all other tiles run the
+  // plain path, so the mask costs nothing where it cannot apply.
+  auto kv_tile = [&](const int j, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
     char* const kcur = kbuf + (NSK == 2 ? (j & 1) * T::kKBytes : 0);
     char* const vcur = vbuf + (NSV == 2 ? (j & 1) * T::kVBytes : 0);
     const bool more = (j + 1 < n_tiles);
@@ -162,33 +166,31 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     h8 pf[RT][NT][2];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      if (causal) {
-        const int kv0 = j * Bc;
-        const int q_first = q0 + wave * WM + rt * 32;
-        if (kv0 + Bc - 1 > q_first + diag) causal_mask<NT>(sacc[rt], kv0, q_first + n + diag, h);
+      const int q_lim = q0 + wave * WM + rt * 32 + n + diag;             // last kv index this row may see
+      if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim, h);
+      // Lazy running max: the reference point m_run of the exponent is moved (and O, l rescaled) only
+      // when some row of the wave has grown past it by more than kLazyLog2 in the log2 domain.  Until
+      // then P may exceed 1 by at most 2^kLazyLog2, which fp16 P and fp32 l, O absorb without loss;
+      // the final O / l is unchanged because numerator and denominator share the reference point.
+      const float m_tile = pair_max(lane_max<NT>(sacc[rt]));
+      const bool grow = (m_tile - m_run[rt]) * c2 > kLazyLog2;          // false for -inf - -inf
+      if (__builtin_amdgcn_ballot_w64(grow) != 0) {                      // wave-uniform branch
+        const float m_new = fmaxf(m_run[rt], m_tile);
+        const SoftmaxStep st = softmax_step(m_run[rt], m_new, c2);
+        m_run[rt] = m_new;
+        l_run[rt] *= st.alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int vv = 0; vv < 16; ++vv) oacc[rt][dt][vv] *= st.alpha;
       }
-      const float m_new = fmaxf(m_run[rt], pair_max(lane_max<NT>(sacc[rt])));
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2((m_run[rt] - m_use) * c2);
-      const float mc = m_use * c2;
-      m_run[rt] = m_new;
-      float lsum = 0.f;
+      const float mc = (m_run[rt] == -INFINITY ? 0.f : m_run[rt]) * c2;
+      l_run[rt] += exp_tile<NT, MASKED>(sacc[rt], c2, mc, j * Bc, q_lim, h);   // per-lane partial sum
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-        for (int vv = 0; vv < 16; ++vv) {
-          const float p = fast_exp2(__builtin_fmaf(sacc[rt][nt][vv], c2, -mc));
-          sacc[rt][nt][vv] = p;
-          lsum += p;
-        }
         pf[rt][nt][0] = pack8_rne(sacc[rt][nt], 0);
         pf[rt][nt][1] = pack8_rne(sacc[rt][nt], 8);
       }
-      l_run[rt] = l_run[rt] * alpha + lsum;      // per-lane partial; the two halves are added at the end
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int vv = 0; vv < 16; ++vv) oacc[rt][dt][vv] *= alpha;
     }
 
     // (B) with one buffer: V_j must have landed / K buffer must be free before K_{j+1} is fetched.
@@ -216,7 +218,16 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
         }
       }
     }
+  };
+
+  // Tiles [0, n_full) are visible to every row of the block; [n_full, n_tiles) touch the diagonal.
+  int n_full = n_tiles;
+  if (causal) {
+    const int lim = (q0 + diag + 1) / Bc;
+    n_full = lim < 0 ? 0 : (lim < n_tiles ? lim : n_tiles);
   }
+  for (int j = 0; j < n_full; ++j) kv_tile(j, std::false_type{});
+  for (int j = n_full; j < n_tiles; ++j) kv_tile(j, std::true_type{});
 
   // ---- epilogue: normalise, round, transpose through LDS, coalesced store ----------------------
   wait_vmcnt<0>();
