@@ -23,7 +23,7 @@ DEFAULT_BUILD_DIR = os.environ.get("AAT_BUILD_DIR", os.path.join(_PKG, "build"))
 
 # -packed-fp32-ops is switched OFF on purpose: hipcc would otherwise fuse scalar fp32 math into
 # v_pk_*_f32 instructions.
-HIPCC_FLAGS = ["-std=c++17", "-O3", "-fno-math-errno", "-ffp-contract=fast", "-fPIC", "-shared", "-w",
+HIPCC_FLAGS = ["-std=c++17", "-O3", "-fno-math-errno", "-ffp-contract=fast", "-fno-honor-nans", "-fPIC", "-shared", "-w",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 

@@ -17,7 +17,7 @@ class AttnConfig(BaseConfig):
 
     def __init__(self, Br, Bc, Kd, D, BlockKSmem=256, BlockKSmem2=64, num_stages_qk=1, num_stages_v=1,
                  Nthreads=256, unrollLastIter=True, warps_mma1_n=None, warps_mma_n=None,
-                 waves_per_eu=1, kv_splits=1):
+                 waves_per_eu=1, kv_splits=1, sw_pipeline=0):
         super().__init__(Br, Bc, Kd, D, BlockKSmem, num_stages_qk, Nthreads, unrollLastIter)
         self.BlockKSmem2 = BlockKSmem2
         self.num_stages_v = num_stages_v
@@ -27,3 +27,4 @@ class AttnConfig(BaseConfig):
             self.warps_mma_n = warps_mma_n
         self.waves_per_eu = waves_per_eu
         self.kv_splits = kv_splits
+        self.sw_pipeline = int(sw_pipeline)

@@ -6,8 +6,10 @@ stored in the tuning cache.  Field names, ``repr`` (one line of a tuning log) an
 compiled library is filed under) follow reference python/autotuner/configs/base_config.py:30-76 and its
 subclasses, so logs and cache files written by the reference remain readable.
 
-New on MI355X: ``waves_per_eu`` (resident waves per SIMD the kernel is compiled for) and
-``kv_splits`` (number of kv-range partitions for long-kv / few-row problems).
+New on MI355X: ``waves_per_eu`` (resident waves per SIMD the kernel is compiled for),
+``sw_pipeline`` (software-pipelined schedule: the next tile's first contraction is issued between the
+current tile's exponentials; needs two K and two V buffers) and ``kv_splits`` (number of kv-range
+partitions for long-kv / few-row problems).
 """
 import os
 
@@ -53,6 +55,7 @@ class BaseConfig:
         self.warps_mma_n = split2[1] if split2 else None
         self.fuse_type = "None"
         self.waves_per_eu = 1
+        self.sw_pipeline = 0
         self.kv_splits = 1
         self.operation = type(self).operation
         self.template_dir = os.path.join(_KERNEL_ROOT, type(self).kernel_subdir) if type(self).kernel_subdir else None
@@ -71,6 +74,8 @@ class BaseConfig:
         out = []
         if getattr(self, "waves_per_eu", 1) != 1:
             out.append(f"w{self.waves_per_eu}")
+        if getattr(self, "sw_pipeline", 0):
+            out.append("p1")
         if getattr(self, "kv_splits", 1) != 1:
             out.append(f"s{self.kv_splits}")
         return out
@@ -81,7 +86,8 @@ class BaseConfig:
             body += f",warps_mma1_n={self.warps_mma1_n},warp_mma_n={self.warps_mma_n}"
         extras = self._extras()
         if extras:
-            body += ", " + ", ".join(f"{k}={getattr(self, k)}" for k in ("waves_per_eu", "kv_splits") if getattr(self, k, 1) != 1)
+            body += ", " + ", ".join(f"{k}={getattr(self, k)}" for k, d in (("waves_per_eu", 1), ("sw_pipeline", 0), ("kv_splits", 1))
+                                     if getattr(self, k, d) != d)
         return f"Config({body})"
 
     def __str__(self):
@@ -104,6 +110,7 @@ class BaseConfig:
     def from_dict(cls, dd):
         cfg = cls.__new__(cls)
         cfg.waves_per_eu = 1
+        cfg.sw_pipeline = 0
         cfg.kv_splits = 1
         vars(cfg).update({k: v for k, v in dd.items() if k != "template_dir"})
         cfg.operation = cls.operation

@@ -56,6 +56,8 @@ def forward_reg_estimate(cfg):
     else:
         # shared fuse: the waves split D between them for the second contraction
         o_regs = (cfg.Br // MFMA_M) * (cfg.D // 32) * 16 // _waves(cfg)
+    if getattr(cfg, "sw_pipeline", 0):
+        s_regs *= 2                                   # current and next score tile are both live
     return q_regs + s_regs + p_regs + o_regs + 48
 
 
@@ -67,6 +69,8 @@ def forward_valid(cfg, arch):
     if _waves(cfg) > 4 * cfg.waves_per_eu:           # the block itself needs that many waves per SIMD
         return False
     if not dma_divisible(cfg):
+        return False
+    if getattr(cfg, "sw_pipeline", 0) and not (cfg.num_stages_qk == 2 and cfg.num_stages_v == 2 and cfg.fuse_type == "register"):
         return False
     if forward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
         return False
@@ -84,6 +88,9 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
                     else:
                         cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, 1, st_v, nthreads, True, waves_per_eu=wpe)
                     out.append(cfg.set_fuse_type(fuse))
+                    if op == "attn" and fuse == "register" and (st_qk, st_v) == (2, 2):
+                        piped = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 2, 2, nthreads, True, waves_per_eu=wpe, sw_pipeline=1)
+                        out.append(piped.set_fuse_type(fuse))
     return out
 
 

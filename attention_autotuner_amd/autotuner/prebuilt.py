@@ -41,6 +41,10 @@ def extra_configs(arch=None):
             cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
             if gfx950_space.forward_valid(cfg, arch):
                 out.append(cfg)
+            if (sq, sv) == (2, 2):
+                piped = AttnConfig(br, bc, dqk, dv, dqk, bc, 2, 2, nt, True, waves_per_eu=wpe, sw_pipeline=1).set_fuse_type("register")
+                if gfx950_space.forward_valid(piped, arch):
+                    out.append(piped)
     return out
 
 

@@ -20,11 +20,12 @@ constexpr int Nthreads = {Nthreads};
 constexpr int num_stages_qk = {num_stages_qk};   // LDS buffers for the K tile
 constexpr int num_stages_v = {num_stages_v};     // LDS buffers for the V tile
 constexpr int waves_per_eu = {waves_per_eu};
+constexpr bool sw_pipeline = {sw_pipeline};      // next tile's QK^T MFMAs interleaved with this tile's exponentials
 constexpr float kReferenceScale = 0.125f;        // what the reference kernels hard-code
 
 using Traits = aat::AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v>;
 constexpr int shared_mem = Traits::kSmemBytes;
-const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu>;
+const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline>;
 
 hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k,
                   float softmax_scale, int causal, hipStream_t stream) {{

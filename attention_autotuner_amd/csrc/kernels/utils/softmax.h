@@ -72,3 +72,55 @@ AAT_DEV float exp_tile(f16v (&s)[NT], float c2, float mc, int kv_base, int q_lim
 }
 
 }  // namespace aat
+
+namespace aat {
+
+// Lazy running max for one 32-row group (see kLazyLog2): moves the exponent's reference point m_run
+// and rescales l_run and the O accumulators only when some row of the wave outgrew it.  Returns
+// mc = m_run * c2, the term subtracted inside the exponent for this tile.
+template <int NT, int DT>
+AAT_DEV float lazy_max_step(const f16v (&s)[NT], float& m_run, float& l_run, f16v (&oacc)[DT], float c2) {
+  const float m_tile = pair_max(lane_max<NT>(s));
+  const bool grow = (m_tile - m_run) * c2 > kLazyLog2;             // false for -inf - -inf
+  if (__builtin_amdgcn_ballot_w64(grow) != 0) {                     // wave-uniform branch
+    const float m_new = fmaxf(m_run, m_tile);
+    const SoftmaxStep st = softmax_step(m_run, m_new, c2);
+    m_run = m_new;
+    l_run *= st.alpha;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) oacc[dt][v] *= st.alpha;
+  }
+  return (m_run == -INFINITY ? 0.f : m_run) * c2;
+}
+
+// exp of `count` consecutive entries (flattened index e = 16*tile + v) of a row group, in place;
+// returns their sum.  Used to spread the exponentials between the MFMAs of the next score tile.
+template <int NT, bool MASKED>
+AAT_DEV float exp_range(f16v (&s)[NT], int e0, int count, float c2, float mc, int kv_base, int q_lim, int h) {
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < count; ++i) {
+    const int e = e0 + i;
+    if (e < NT * 16) {
+      const int t = e >> 4, v = e & 15;
+      float p;
+      if (MASKED && kv_base + 32 * t + c_row(v, h) > q_lim) p = 0.f;
+      else p = fast_exp2(__builtin_fmaf(MASKED ? fmaxf(s[t][v], -3.0e38f) : s[t][v], c2, -mc));
+      s[t][v] = p;
+      sum += p;
+    }
+  }
+  return sum;
+}
+
+template <int NT> AAT_DEV void pack_p(h8 (&pf)[NT][2], const f16v (&s)[NT]) {
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    pf[t][0] = pack8_rne(s[t], 0);
+    pf[t][1] = pack8_rne(s[t], 8);
+  }
+}
+
+}  // namespace aat

@@ -1,0 +1,116 @@
+// Wave-level tile operations shared by the forward kernels (attention and RetNet): operand fetch in
+// MFMA layouts, the two contractions S^T = K Q^T and O^T += V^T P^T, and the output epilogue.
+// Counterpart of reference csrc/kernels/utils/matmul.h:10-267 (smem->register + MMA pipelines), built on the
+// gfx950 layouts described in cdna4.h.
+#pragma once
+#include "cdna4.h"
+
+namespace aat {
+
+// Q rows of this wave as MFMA B operands, straight from global memory.
+// qrow points at element [first row of the wave + n][8*h] of a row-major [*, Kd] matrix.
+template <int RT, int KS, int Kd>
+AAT_DEV void load_q_frags(h8 (&qf)[RT][KS], const half_t* qrow) {
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[rt][ks] = *reinterpret_cast<const h8*>(qrow + (size_t)rt * 32 * Kd + 16 * ks);
+}
+
+// Byte offsets, inside a Rows16-swizzled [rows][Kd] tile, of this lane's A-operand chunks for tile row n.
+template <int KS, int NCK>
+AAT_DEV void k_frag_offsets(int (&koff)[KS], int n, int h) {
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = lds_chunk_off<NCK, Swz::Rows16>(n, 2 * ks + h);
+}
+
+// Byte offsets, inside a Rows4-swizzled [rows][D] tile, of the address this lane presents to the
+// transposing read for d-tile dt (kv rows 4h .. 4h+3 of a 16-row step; add 8 rows for the second half).
+template <int DT, int NCV>
+AAT_DEV void v_frag_offsets(int (&voff)[DT], int lane) {
+  const int h = lane >> 5, s16 = lane & 15;
+  const int row = 4 * h + (s16 >> 2);
+  const int vcol = 16 * ((lane >> 4) & 1) + 4 * (s16 & 3);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    voff[dt] = lds_chunk_off<NCV, Swz::Rows4>(row, 4 * dt + (vcol >> 3)) + (vcol & 7) * 2;
+}
+
+// One MFMA step of S^T = K Q^T: score tile nt, k-step ks.
+template <int RT, int NT, int KS, int NCK>
+AAT_DEV void qk_step(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const char* ktile, const int (&koff)[KS],
+                     int nt, int ks) {
+  const h8 kf = lds_read_h8(ktile + nt * 32 * NCK * 16 + koff[ks]);
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) sacc[rt][nt] = mfma_32x32x16(kf, qf[rt][ks], sacc[rt][nt]);
+}
+
+template <int RT, int NT, int KS, int NCK>
+AAT_DEV void qk_gemm(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const char* ktile, const int (&koff)[KS]) {
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) sacc[rt][nt] = zero16();
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qk_step<RT, NT, KS, NCK>(sacc, qf, ktile, koff, nt, ks);
+}
+
+// O^T += V^T P^T over one kv tile.  pf[rt][nt][s] is the fp16 P operand for kv rows 32*nt + 16*s ..+15.
+template <int RT, int NT, int DT, int NCV>
+AAT_DEV void pv_gemm(f16v (&oacc)[RT][DT], const h8 (&pf)[RT][NT][2], const char* vtile, const int (&voff)[DT]) {
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const char* vrow = vtile + (32 * nt + 16 * s) * NCV * 16;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const h4 lo = lds_read_tr_h4(vrow + voff[dt]);
+        const h4 hi = lds_read_tr_h4(vrow + 8 * NCV * 16 + voff[dt]);
+        const h8 vf = cat_h4(lo, hi);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][nt][s], oacc[rt][dt]);
+      }
+    }
+  }
+}
+
+// Epilogue: scale the wave's O^T accumulators per row, round to fp16 (RNE), transpose through a
+// wave-private LDS staging area and store rows with 16-byte coalesced writes.
+// ostage: wave-private LDS, WM rows of O_STRIDE bytes.  og: global pointer to the wave's first output row.
+template <int RT, int DT, int D, int O_STRIDE>
+AAT_DEV void store_o_tile(const f16v (&oacc)[RT][DT], const float (&row_scale)[RT], char* ostage, half_t* og,
+                          int lane) {
+  constexpr int NCV = D / 8, WM = RT * 32;
+  const int n = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const float sc = row_scale[rt];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const h2 a = pack_rne(oacc[rt][dt][4 * g] * sc, oacc[rt][dt][4 * g + 1] * sc);
+        const h2 b = pack_rne(oacc[rt][dt][4 * g + 2] * sc, oacc[rt][dt][4 * g + 3] * sc);
+        h4 w;
+        w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
+        const int d0 = 32 * dt + 8 * g + 4 * h;
+        *reinterpret_cast<h4*>(ostage + (rt * 32 + n) * O_STRIDE + d0 * 2) = w;
+      }
+    }
+  }
+  wait_lgkm0();                                   // the staging region is private to this wave
+  constexpr int kChunks = WM * NCV;
+#pragma unroll
+  for (int t = 0; t < kChunks / 64; ++t) {
+    const int idx = t * 64 + lane;
+    const int row = idx / NCV, c = idx % NCV;
+    const u4v val = *reinterpret_cast<const u4v*>(ostage + row * O_STRIDE + c * 16);
+    *reinterpret_cast<u4v*>(reinterpret_cast<char*>(og) + ((size_t)row * NCV + c) * 16) = val;
+  }
+}
+
+}  // namespace aat

@@ -96,8 +96,9 @@ def test_every_configuration_agrees_with_the_oracle(dqk, dv):
     refs = {c: ref_op.attention_ref(q, k, v, None, c) for c in (False, True)}
     qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
     ran = 0
-    for br, bc, nt, sq, sv, wpe in CONFIGS:
-        cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+    variants = [(t, 0) for t in CONFIGS] + [(t, 1) for t in CONFIGS if t[3:5] == (2, 2)]
+    for (br, bc, nt, sq, sv, wpe), pipe in variants:
+        cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe, sw_pipeline=pipe).set_fuse_type("register")
         if not gfx950_space.forward_valid(cfg, ARCH):
             continue
         assert os.path.exists(codegen.library_path(cfg)), f"library for {cfg} was not built ahead of time"
