@@ -50,7 +50,7 @@ def forward_reg_estimate(cfg):
     rt = rows_per_wave(cfg) // MFMA_M
     q_regs = rt * (cfg.Kd // 16) * 4
     s_regs = rt * (cfg.Bc // 32) * 16
-    p_regs = rt * (cfg.Bc // 32) * 8
+    p_regs = rt * (cfg.Bc // 32) * 4            # fp16 P, built while the fp32 scores retire
     if cfg.fuse_type == "register":
         o_regs = rt * (cfg.D // 32) * 16
     else:
@@ -58,7 +58,7 @@ def forward_reg_estimate(cfg):
         o_regs = (cfg.Br // MFMA_M) * (cfg.D // 32) * 16 // _waves(cfg)
     if getattr(cfg, "sw_pipeline", 0):
         s_regs *= 2                                   # current and next score tile are both live
-    return q_regs + s_regs + p_regs + o_regs + 48
+    return q_regs + s_regs + p_regs + o_regs + 32
 
 
 def forward_valid(cfg, arch):
@@ -70,8 +70,13 @@ def forward_valid(cfg, arch):
         return False
     if not dma_divisible(cfg):
         return False
-    if getattr(cfg, "sw_pipeline", 0) and not (cfg.num_stages_qk == 2 and cfg.num_stages_v == 2 and cfg.fuse_type == "register"):
-        return False
+    if getattr(cfg, "sw_pipeline", 0):
+        # needs 2+2 buffers and K copies made of whole 32-row units
+        rows_per_dma = cfg.Nthreads * 8 // cfg.Kd if (cfg.Nthreads * 8) % cfg.Kd == 0 else 0
+        if not (cfg.num_stages_qk == 2 and cfg.num_stages_v == 2 and cfg.fuse_type == "register"):
+            return False
+        if rows_per_dma == 0 or rows_per_dma > 32 or 32 % rows_per_dma:
+            return False
     if forward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
         return False
     return forward_reg_estimate(cfg) <= arch.register_per_thread // cfg.waves_per_eu
@@ -81,7 +86,7 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
     out = []
     for nthreads in THREADS:
         for st_qk, st_v in STAGES:
-            for wpe in (1, 2):
+            for wpe in (1, 2, 3):
                 for fuse in fuse_types:
                     if op == "attn":
                         cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, waves_per_eu=wpe)
@@ -96,7 +101,7 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
 
 def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
     """A configuration that is valid for every supported head size; used before/without tuning."""
-    prefs = [(128, 64, 256, 2, 2, 2), (128, 64, 256, 1, 1, 2), (128, 64, 256, 1, 1, 1), (128, 32, 256, 1, 1, 1),
+    prefs = [(256, 64, 512, 2, 2, 2), (128, 64, 256, 2, 2, 2), (128, 64, 256, 1, 1, 2), (128, 64, 256, 1, 1, 1), (128, 32, 256, 1, 1, 1),
              (64, 32, 128, 1, 1, 1)]
     for br, bc, nt, sq, sv, wpe in prefs:
         if (seq_q and seq_q % br) or (seq_k and seq_k % bc):

@@ -26,7 +26,7 @@ DEFAULT_PROBLEMS = [
 PARITY_TILES = [
     (128, 64, 256, 2, 2, 2), (128, 64, 256, 1, 1, 2), (128, 64, 256, 2, 1, 1), (128, 64, 256, 1, 2, 1),
     (128, 32, 256, 2, 2, 2), (128, 128, 256, 1, 1, 1), (64, 64, 128, 2, 2, 2), (128, 64, 128, 1, 1, 1),
-    (256, 64, 512, 2, 2, 2),
+    (256, 64, 512, 2, 2, 2), (128, 32, 256, 2, 2, 3), (128, 64, 256, 1, 1, 3),
 ]
 PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
 
@@ -65,7 +65,8 @@ def shipping_set(arch=None):
     cfgs = []
     for op, dqk, dv in DEFAULT_PROBLEMS:
         if op in ("attn", "ret"):
-            cfgs.append(gfx950_space.default_forward_config(op, dqk, dv, arch))
+            for seq in (None, 128, 64):          # defaults differ with what the sequence length divides by
+                cfgs.append(gfx950_space.default_forward_config(op, dqk, dv, arch, seq, seq))
     cfgs += extra_configs(arch)
     cfgs += cached_configs()
     seen, unique = set(), []

@@ -25,16 +25,19 @@ constexpr float kReferenceScale = 0.125f;        // what the reference kernels h
 
 using Traits = aat::AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v>;
 constexpr int shared_mem = Traits::kSmemBytes;
-const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline>;
+const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, false>;
+const auto kernel_causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, true>;
 
 hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k,
                   float softmax_scale, int causal, hipStream_t stream) {{
   static const hipError_t lds_ok = aat::allow_lds(kernel, shared_mem);
+  static const hipError_t lds_ok_causal = aat::allow_lds(kernel_causal, shared_mem);
   if (lds_ok != hipSuccess) return lds_ok;
-  kernel<<<dim3(B * H * (Seq_q / Br)), dim3(Nthreads), shared_mem, stream>>>(
+  if (lds_ok_causal != hipSuccess) return lds_ok_causal;
+  (causal ? kernel_causal : kernel)<<<dim3(B * H * (Seq_q / Br)), dim3(Nthreads), shared_mem, stream>>>(
       reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
       reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<aat::half_t*>(o), nullptr, H, Seq_k, Seq_q,
-      softmax_scale, causal);
+      softmax_scale);
   return hipGetLastError();
 }}
 }}  // namespace

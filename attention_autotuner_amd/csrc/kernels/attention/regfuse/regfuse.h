@@ -11,9 +11,10 @@
 //  * Q never touches LDS: it is loaded once, straight into MFMA B-operand registers;
 //  * K and V tiles reach LDS by LDS-DMA (global_load_lds_dwordx4), XOR-swizzled, 1 or 2 buffers each;
 //  * V^T operands come from ds_read_b64_tr_b16;
-//  * the running max is lazy (softmax.h) and, in the pipelined schedule, the MFMAs of the NEXT score
-//    tile are issued between the exponentials of the current one so matrix and vector pipes overlap
-//    inside one wave;
+//  * the running max is lazy (softmax.h);
+//  * two schedules: the plain one walks Bc-wide tiles (scores, softmax, PV, in that order); the
+//    pipelined one works in 32-row units and issues the MFMAs of the NEXT unit's scores between the
+//    exponentials of the current unit, so the matrix and vector pipes overlap inside one wave;
 //  * softmax scale and causal masking are runtime arguments (the reference hard-codes 0.125 at :50 and
 //    has the causal bound commented out at :59-61).
 #pragma once
@@ -23,6 +24,10 @@
 #include "../../utils/softmax.h"
 #include "../../utils/tile_ops.h"
 
+#ifndef AAT_PF
+#define AAT_PF 2
+#endif
+
 namespace aat {
 
 template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV>
@@ -30,7 +35,7 @@ struct AttnFwdRegfuse {
   static constexpr int NW = Nthreads / kWave;   // waves per block
   static constexpr int WM = Br / NW;            // query rows per wave
   static constexpr int RT = WM / 32;            // 32-row groups per wave
-  static constexpr int NT = Bc / 32;            // score tiles along kv
+  static constexpr int NT = Bc / 32;            // score tiles (units) along kv
   static constexpr int KS = Kd / 16;            // MFMA k-steps of S^T = K Q^T
   static constexpr int DT = D / 32;             // output tiles along d
   static constexpr int NCK = Kd / 8, NCV = D / 8;
@@ -41,23 +46,54 @@ struct AttnFwdRegfuse {
   using KDma = TileDma<Bc, NCK, Nthreads, Swz::Rows16>;
   using VDma = TileDma<Bc, NCV, Nthreads, Swz::Rows4>;
   static constexpr int kKBytes = Bc * Kd * 2, kVBytes = Bc * D * 2;
+  static constexpr int kUnitK = 32 * Kd * 2, kUnitV = 32 * D * 2;   // bytes of one 32-row unit
   static constexpr int kOStride = D * 2 + 16;   // epilogue staging row stride (bytes)
   static constexpr int kMainBytes = NSK * kKBytes + NSV * kVBytes;
   static constexpr int kEpiBytes = Br * kOStride;
   static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
+  // The pipelined schedule copies K in whole 32-row units.
+  static constexpr bool kPipeOk = NSK == 2 && NSV == 2 && KDma::kRegular && KDma::kRowsPerIter <= 32 &&
+                                  32 % KDma::kRowsPerIter == 0;
+  static constexpr int kKInstrPerUnit = KDma::kRegular ? 32 / (KDma::kRowsPerIter > 32 ? 32 : KDma::kRowsPerIter) : 0;
 };
 
+// Walk the kv tiles of a block two at a time (buffer parity 0, then 1).  Tiles [0, n_full) run the
+// unmasked body; with CAUSAL the rest run the masked body.  n_full is even, so both loops start on
+// parity 0 and every tile body is instantiated exactly once per (parity, masked) pair.
+template <bool CAUSAL, class F> AAT_DEV void run_tiles(F& tile, int n_full, int n_tiles) {
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  const int n_plain = CAUSAL ? n_full : n_tiles;
+  for (int j = 0; j < n_plain; j += 2) {
+    tile(j, P0{}, std::false_type{});
+    if (j + 1 < n_plain) tile(j + 1, P1{}, std::false_type{});
+  }
+  if constexpr (CAUSAL) {
+    for (int j = n_full; j < n_tiles; j += 2) {
+      tile(j, P0{}, std::true_type{});
+      if (j + 1 < n_tiles) tile(j + 1, P1{}, std::true_type{});
+    }
+  }
+}
+
 // lse may be null.  When non-null it receives the natural-log-sum-exp of the scaled scores per row.
-// PIPE selects the software-pipelined schedule (needs two K and two V buffers).
-template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int WPE = 1, bool PIPE = false>
+// PIPE selects the software-pipelined schedule (needs two K and two V buffers).  CAUSAL is a
+// compile-time switch so that the non-causal kernel carries no masking code at all; in the causal
+// kernel the tiles the diagonal cannot touch still run the unmasked tile body.
+template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int WPE = 1, bool PIPE = false,
+          bool CAUSAL = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k,
                       const half_t* __restrict__ v, half_t* __restrict__ o, float* __restrict__ lse,
-                      int H, int seq_k, int seq_q, float softmax_scale, int causal) {
+                      int H, int seq_k, int seq_q, float softmax_scale) {
   using T = AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, WM = T::WM;
-  static_assert(!PIPE || (NSK == 2 && NSV == 2), "the pipelined schedule reads K one tile ahead");
+  constexpr int PF = AAT_PF;                     // operand prefetch distance, in MFMA steps
+  static_assert(!PIPE || T::kPipeOk, "the pipelined schedule needs 2+2 buffers and unit-aligned K copies");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+#ifdef AAT_CLOCK_PROBE
+  const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
+#endif
   char* const kbuf = smem;
   char* const vbuf = smem + NSK * T::kKBytes;
 
@@ -70,17 +106,18 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = tile / Tr;
   int rb = tile % Tr;
-  if (causal) rb = Tr - 1 - rb;                 // long rows first
+  if constexpr (CAUSAL) rb = Tr - 1 - rb;       // long rows first
   const int q0 = rb * Br;
   const int diag = seq_k - seq_q;               // kv index allowed for query i is <= i + diag
   int n_tiles = seq_k / Bc;
   int n_full = n_tiles;                         // tiles [0, n_full) are visible to every row of the block
-  if (causal) {
+  if constexpr (CAUSAL) {
     const int last = q0 + Br - 1 + diag;        // last visible kv index for this block
     const int lim = last < 0 ? 0 : last / Bc + 1;
     n_tiles = lim < n_tiles ? lim : n_tiles;
     const int full = (q0 + diag + 1) / Bc;
     n_full = full < 0 ? 0 : (full < n_tiles ? full : n_tiles);
+    n_full &= ~1;                               // keep the masked loop on an even tile: buffer parity 0
   }
 
   const char* kg = reinterpret_cast<const char*>(k + (size_t)bh * seq_k * Kd);
@@ -88,15 +125,22 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
 
   typename T::KDma kdma;
   typename T::VDma vdma;
-  kdma.init(tid, Kd * 2);
-  vdma.init(tid, D * 2);
+  kdma.init(tid);
+  vdma.init(tid);
   const int wave_base = wave * 64;
 
   h8 qf[RT][KS];
   load_q_frags<RT, KS, Kd>(qf, q + ((size_t)bh * seq_q + q0 + wave * WM + n) * Kd + 8 * h);
-  int koff[KS], voff[DT];
-  k_frag_offsets<KS, NCK>(koff, n, h);
-  v_frag_offsets<DT, NCV>(voff, lane);
+  uint32_t kaddr[KS], vaddr[DT];                 // this lane's operand addresses inside buffer 0
+  {
+    int koff[KS], voff[DT];
+    k_frag_offsets<KS, NCK>(koff, n, h);
+    v_frag_offsets<DT, NCV>(voff, lane);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = lds_addr(kbuf + koff[ks]);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vaddr[dt] = lds_addr(vbuf + voff[dt]);
+  }
 
   f16v oacc[RT][DT];
   float m_run[RT], l_run[RT];
@@ -116,10 +160,12 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
       kdma.issue(kg, kbuf, wave_base);
       if constexpr (NSV == 2) vdma.issue(vg, vbuf, wave_base);
     }
-    auto kv_tile = [&](const int j, auto masked_tag) {
-      constexpr bool MASKED = decltype(masked_tag)::value;
-      char* const kcur = kbuf + (NSK == 2 ? (j & 1) * T::kKBytes : 0);
-      char* const vcur = vbuf + (NSV == 2 ? (j & 1) * T::kVBytes : 0);
+    // `parity_tag` carries j & 1 as a compile-time value so that every LDS address of the tile is a
+    // per-lane constant plus an immediate.
+    auto kv_tile = [&](const int j, auto parity_tag, auto masked_tag) {
+      constexpr int PAR = decltype(parity_tag)::value;
+      constexpr bool MASKED = decltype(masked_tag)::value;   // the causal diagonal may cross this tile
+      char* const vcur = vbuf + (NSV == 2 ? PAR * T::kVBytes : 0);
       const bool more = (j + 1 < n_tiles);
 
       // (A) K_j (and with two V buffers V_j) has landed; every wave is past iteration j-1.
@@ -127,21 +173,19 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
       block_sync();
       if constexpr (NSV == 1) vdma.issue(vg + (size_t)j * T::kVBytes, vcur, wave_base);
       if (more) {
-        if constexpr (NSK == 2) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf + ((j + 1) & 1) * T::kKBytes, wave_base);
-        if constexpr (NSV == 2) vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + ((j + 1) & 1) * T::kVBytes, wave_base);
+        if constexpr (NSK == 2) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf + (PAR ^ 1) * T::kKBytes, wave_base);
+        if constexpr (NSV == 2) vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + (PAR ^ 1) * T::kVBytes, wave_base);
       }
 
       f16v sacc[RT][NT];
-      qk_gemm<RT, NT, KS, NCK>(sacc, qf, kcur, koff);
+      qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
 
-      h8 pf[RT][NT][2];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
-        const int q_lim = q_lim0 + rt * 32;
-        if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim, h);
+        if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
         const float mc = lazy_max_step<NT, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
-        l_run[rt] += exp_tile<NT, MASKED>(sacc[rt], c2, mc, j * Bc, q_lim, h);   // per-lane partial sum
-        pack_p<NT>(pf[rt], sacc[rt]);
+        exp_tile<NT>(sacc[rt], c2, mc);
+        if constexpr (MASKED) zero_masked<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
       }
 
       // (B) with one buffer: V_j must have landed / K buffer must be free before K_{j+1} is fetched.
@@ -152,75 +196,85 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
           if (more) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf, wave_base);
         }
       }
-      pv_gemm<RT, NT, DT, NCV>(oacc, pf, vcur, voff);
+      h8 pf[RT][NT][2];
+      pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) pack_p_group<NT>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
+      });
     };
-    for (int j = 0; j < n_full; ++j) kv_tile(j, std::false_type{});
-    for (int j = n_full; j < n_tiles; ++j) kv_tile(j, std::true_type{});
+    run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
   } else {
     // ============================ pipelined schedule =============================================
-    // Iteration j holds S_j in registers (computed one iteration earlier) and does
-    //   [ S_{j+1} = K_{j+1} Q^T  interleaved with  P_j = exp(S_j - m) ] ; O += V_j^T P_j.
-    // Buffers: K_{j+1} is read while K_{j+2} is fetched into the other K buffer; V_j is read while
-    // V_{j+1} is fetched.  One barrier per iteration.
-    f16v scur[RT][NT];
+    // The unit of work is 32 kv rows.  While unit u is exponentiated, the MFMAs of unit u+1's scores
+    // run underneath; then O += V_u^T P_u runs with the fp16 packing of P_u underneath.  Two score
+    // tiles are live (current, next).
+    //
+    // K is copied in Bc-row tiles that are SHIFTED by one unit against the V tiles: K copy j holds kv
+    // rows [j*Bc + 32, (j+1)*Bc + 32), exactly the units whose scores are computed during iteration j
+    // (units 1..NT-1 of tile j and unit 0 of tile j+1).  So iteration j reads K buffer j&1 only, while
+    // copy j+1 streams into the other one; V tile j is read from V buffer j&1 while V_{j+1} streams
+    // in.  One barrier per Bc rows.  Rows [0, 32) are fetched on their own in the prologue.
+    constexpr int KI = T::kKInstrPerUnit;        // DMA instructions per 32 rows of K
+    f16v sbuf[2][RT][1];
+    auto issue_k_copy = [&](int jj, char* dst) { // K copy jj; the last one stops at the end of the range
+      const char* src = kg + (size_t)jj * T::kKBytes + T::kUnitK;
+      if (jj + 1 < n_tiles) kdma.issue(src, dst, wave_base);
+      else kdma.template issue_part<0, (NT - 1) * KI>(src, dst, wave_base);
+    };
     if (n_tiles > 0) {
-      kdma.issue(kg, kbuf, wave_base);
+      kdma.template issue_part<0, KI>(kg, kbuf + T::kKBytes + (NT - 1) * T::kUnitK, wave_base);   // rows [0, 32)
+      issue_k_copy(0, kbuf);
       vdma.issue(vg, vbuf, wave_base);
-      if (n_tiles > 1) kdma.issue(kg + T::kKBytes, kbuf + T::kKBytes, wave_base);
       wait_vmcnt<0>();
       block_sync();
-      qk_gemm<RT, NT, KS, NCK>(scur, qf, kbuf, koff);
+      qk_gemm_steps<RT, 1, KS, NCK, PF>(sbuf[0], qf, kaddr, T::kKBytes + (NT - 1) * T::kUnitK, [](int) {});
     }
-    auto kv_tile = [&](const int j, auto masked_tag) {
+    auto kv_tile = [&](const int j, auto parity_tag, auto masked_tag) {
+      constexpr int PAR = decltype(parity_tag)::value;
       constexpr bool MASKED = decltype(masked_tag)::value;
-      char* const knext = kbuf + ((j + 1) & 1) * T::kKBytes;
-      char* const vcur = vbuf + (j & 1) * T::kVBytes;
-      // K_{j+1} and V_j have landed; every wave finished S_j (frees K buffer j&1) and O += V_{j-1} P.
+      const bool last_tile = (j + 1 >= n_tiles);
+      // K copy j and V_j have landed; every wave finished iteration j-1 (frees the other buffers).
       wait_vmcnt<0>();
       block_sync();
-      if (j + 2 < n_tiles) kdma.issue(kg + (size_t)(j + 2) * T::kKBytes, kbuf + (j & 1) * T::kKBytes, wave_base);
-      if (j + 1 < n_tiles) vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + ((j + 1) & 1) * T::kVBytes, wave_base);
-
-      float mc[RT];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if constexpr (MASKED) causal_mask<NT>(scur[rt], j * Bc, q_lim0 + rt * 32, h);
-        mc[rt] = lazy_max_step<NT, DT>(scur[rt], m_run[rt], l_run[rt], oacc[rt], c2);
+      if (!last_tile) {
+        issue_k_copy(j + 1, kbuf + (PAR ^ 1) * T::kKBytes);
+        vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + (PAR ^ 1) * T::kVBytes, wave_base);
       }
-
-      f16v snext[RT][NT];
-      h8 pf[RT][NT][2];
-      if (j + 1 < n_tiles) {
-        constexpr int kSteps = NT * KS;                              // MFMA groups of the next tile
-        constexpr int kPerStep = (NT * 16 + kSteps - 1) / kSteps;    // exponentials per group and row group
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+      for (int t = 0; t < NT; ++t) {
+        const int cur = (PAR * NT + t) & 1;                        // which score buffer holds unit (j, t)
+        auto& scur = sbuf[cur];
+        auto& snext = sbuf[cur ^ 1];
+        const int kv0 = j * Bc + 32 * t;
+        float mc[RT];
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) snext[rt][nt] = zero16();
-#pragma unroll
-        for (int step = 0; step < kSteps; ++step) {
-          qk_step<RT, NT, KS, NCK>(snext, qf, knext, koff, step / KS, step % KS);
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            l_run[rt] += exp_range<NT, MASKED>(scur[rt], step * kPerStep, kPerStep, c2, mc[rt], j * Bc, q_lim0 + rt * 32, h);
+        for (int rt = 0; rt < RT; ++rt) {
+          if constexpr (MASKED) causal_mask<1>(scur[rt], kv0, q_lim0 + rt * 32, h);
+          mc[rt] = lazy_max_step<1, DT>(scur[rt], m_run[rt], l_run[rt], oacc[rt], c2);
         }
-      } else {
+        constexpr int kPerStep = (16 + KS - 1) / KS;               // exponentials per MFMA step
+        if (t + 1 < NT || !last_tile) {
+          // scores of the next unit: slot t of K buffer PAR
+          qk_gemm_steps<RT, 1, KS, NCK, PF>(snext, qf, kaddr, PAR * T::kKBytes + t * T::kUnitK, [&](int step) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-          l_run[rt] += exp_tile<NT, MASKED>(scur[rt], c2, mc[rt], j * Bc, q_lim0 + rt * 32, h);
-      }
+            for (int rt = 0; rt < RT; ++rt) exp_range<1>(scur[rt], step * kPerStep, kPerStep, c2, mc[rt]);
+          });
+        } else {
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) pack_p<NT>(pf[rt], scur[rt]);
-      pv_gemm<RT, NT, DT, NCV>(oacc, pf, vcur, voff);
-      if (j + 1 < n_tiles) {
+          for (int rt = 0; rt < RT; ++rt) exp_tile<1>(scur[rt], c2, mc[rt]);
+        }
+        if constexpr (MASKED) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+          for (int rt = 0; rt < RT; ++rt) zero_masked<1>(scur[rt], kv0, q_lim0 + rt * 32, h);
+        }
+        h8 pf[RT][1][2];
+        pv_gemm_steps<RT, 1, DT, NCV, PF>(oacc, pf, vaddr, PAR * T::kVBytes + t * T::kUnitV, [&](int g) {
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt) scur[rt][nt] = snext[rt][nt];
+          for (int rt = 0; rt < RT; ++rt) pack_p_group<1>(pf[rt], scur[rt], g, l_run[rt]);
+        });
       }
     };
-    for (int j = 0; j < n_full; ++j) kv_tile(j, std::false_type{});
-    for (int j = n_full; j < n_tiles; ++j) kv_tile(j, std::true_type{});
+    run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
   }
 
   // ---- epilogue: normalise, round, transpose through LDS, coalesced store ----------------------
@@ -238,6 +292,12 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   }
   store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + wave * WM * T::kOStride,
                                        o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+#ifdef AAT_CLOCK_PROBE
+  if (lse != nullptr && tid == 0 && (blockIdx.x % 64) == 0) {
+    lse[2 * (blockIdx.x / 64)] = (float)(clock64() - probe_c0);
+    lse[2 * (blockIdx.x / 64) + 1] = (float)(wall_clock64() - probe_w0);
+  }
+#endif
 }
 
 }  // namespace aat

@@ -107,28 +107,50 @@ template <int NC, Swz MODE> AAT_DEV constexpr int swz(int row, int c) {
   else return swz_rows4<NC>(row, c);
 }
 
+constexpr int cgcd(int a, int b) { return b == 0 ? a : cgcd(b, a % b); }
+
+// The source address of every copy is split into a wave-uniform part (tile pointer + a compile-time
+// multiple of the row pitch, kept in SGPRs) and one 32-bit per-lane offset, so a tile copy costs one
+// or two VGPRs of addressing instead of a 64-bit pointer per instruction.  That works when the block's
+// threads cover whole rows per instruction (NT % NC == 0): then a thread keeps its chunk column and
+// only the swizzle term can change from one instruction to the next, with a short period.
 template <int ROWS, int NC, int NT, Swz MODE>
 struct TileDma {
   static constexpr int kChunks = ROWS * NC;
   static_assert(kChunks % NT == 0, "tile chunks must divide evenly over the block's threads");
   static constexpr int kIters = kChunks / NT;          // LDS-DMA instructions per thread per tile
   static constexpr int kBytes = kChunks * 16;
-  int goff[kIters];                                    // byte offset of this thread's source chunk inside a tile
+  static constexpr int kRowBytes = NC * 16;
+  static constexpr bool kRegular = (NT % NC == 0);
+  static constexpr int kRowsPerIter = kRegular ? NT / NC : 1;
+  static constexpr int kPeriod = (MODE == Swz::Rows16) ? 16 : 4;   // rows after which the swizzle repeats
+  static constexpr int kDistinctRaw = kPeriod / cgcd(kRowsPerIter, kPeriod);
+  static constexpr int kDistinct = !kRegular ? kIters : (kDistinctRaw < kIters ? kDistinctRaw : kIters);
+  uint32_t loff[kDistinct];                            // per-lane byte offsets inside a tile
 
-  AAT_DEV void init(int tid, int row_stride_bytes) {
+  AAT_DEV void init(int tid) {
 #pragma unroll
-    for (int i = 0; i < kIters; ++i) {
+    for (int i = 0; i < kDistinct; ++i) {
       const int s = i * NT + tid;
       const int row = s / NC, cs = s % NC;
-      goff[i] = row * row_stride_bytes + swz<NC, MODE>(row, cs) * 16;
+      const int row0 = kRegular ? tid / NC : row;      // the uniform part carries i * kRowsPerIter rows
+      loff[i] = (uint32_t)(row0 * kRowBytes + swz<NC, MODE>(row, cs) * 16);
     }
   }
-  // Issue the copy of one tile.  `g` points at the tile's first row in global memory, `lds` at the
-  // destination buffer (block-uniform); wave_base = 64 * wave index (wave-uniform).
-  AAT_DEV void issue(const char* g, char* lds, int wave_base) const {
+  // Issue the copy of one tile.  `g` points at the tile's first row in global memory (wave-uniform),
+  // `lds` at the destination buffer (block-uniform); wave_base = 64 * wave index (wave-uniform).
+  AAT_DEV void issue(const char* g, char* lds, int wave_base) const { issue_part<0, kIters>(g, lds, wave_base); }
+
+  // Instructions [I0, I1) only.  With kRegular, instruction i covers tile rows
+  // [i*kRowsPerIter, (i+1)*kRowsPerIter), so this copies a contiguous range of rows.
+  template <int I0, int I1>
+  AAT_DEV void issue_part(const char* g, char* lds, int wave_base) const {
 #pragma unroll
-    for (int i = 0; i < kIters; ++i) {
-      __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(g + goff[i]),
+    for (int i = I0; i < I1; ++i) {
+      uint64_t base = (uint64_t)(uintptr_t)(kRegular ? g + (size_t)i * kRowsPerIter * kRowBytes : g);
+      asm volatile("" : "+s"(base));                   // keep the uniform part in SGPRs (saddr form)
+      const uint32_t lane_off = loff[kRegular ? i % kDistinct : i];
+      __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)(base + lane_off),
                                        (AAT_AS3 void*)(lds + (i * NT + wave_base) * 16), 16, 0, 0);
     }
   }

@@ -1,8 +1,7 @@
-// Row-wise pieces of the online softmax and of the RetNet abs-sum normalisation, written for the
-// transposed score layout (one lane = one query row, see cdna4.h).  These replace the warp-shuffle
-// butterflies of the reference (reference: csrc/kernels/utils/reduce.h:16-100, elementwise.h:5-41):
-// here a row lives in 16*NT registers of two lanes, so a reduction is a register loop plus one
-// exchange with lane^32.
+// Row-wise pieces of the online softmax, written for the transposed score layout (one lane = one
+// query row, see cdna4.h).  These replace the warp-shuffle butterflies of the reference
+// (reference: csrc/kernels/utils/reduce.h:16-100): here a row lives in 16*NT registers of two lanes, so a
+// reduction is a register loop plus one exchange with lane^32.
 #pragma once
 #include "cdna4.h"
 
@@ -36,6 +35,20 @@ template <int NT> AAT_DEV void causal_mask(f16v (&s)[NT], int kv_base, int q_lim
   }
 }
 
+// Zero the P entries above the causal diagonal (same predicate as causal_mask).  exp2 of a masked
+// score is already 0 for any positive scale; this pass makes the result exact for scale 0 as well,
+// where -inf * 0 would otherwise leave a NaN.
+template <int NT> AAT_DEV void zero_masked(f16v (&p)[NT], int kv_base, int q_lim, int h) {
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int kv = kv_base + 32 * t + c_row(v, h);
+      if (kv > q_lim) p[t][v] = 0.f;
+    }
+  }
+}
+
 // One step of the running-max recurrence.  m_old / m_new are UNSCALED row maxima (-inf before the
 // first visible kv), c2 = softmax_scale * log2(e).  alpha rescales the running sum and output,
 // mc is the term subtracted inside the exponent.  Written so that -inf never meets a multiply:
@@ -52,32 +65,11 @@ AAT_DEV SoftmaxStep softmax_step(float m_old, float m_new, float c2) {
   return st;
 }
 
-// s <- exp2(s*c2 - mc) in place; returns the lane's partial row sum.  MASKED zeroes the entries above
-// the causal diagonal explicitly (exact for any scale, including 0) and is used on diagonal tiles only.
-template <int NT, bool MASKED>
-AAT_DEV float exp_tile(f16v (&s)[NT], float c2, float mc, int kv_base, int q_lim, int h) {
-  float lsum = 0.f;
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      float p;
-      if (MASKED && kv_base + 32 * t + c_row(v, h) > q_lim) p = 0.f;
-      else p = fast_exp2(__builtin_fmaf(MASKED ? fmaxf(s[t][v], -3.0e38f) : s[t][v], c2, -mc));
-      s[t][v] = p;
-      lsum += p;
-    }
-  }
-  return lsum;
-}
-
-}  // namespace aat
-
-namespace aat {
-
-// Lazy running max for one 32-row group (see kLazyLog2): moves the exponent's reference point m_run
-// and rescales l_run and the O accumulators only when some row of the wave outgrew it.  Returns
-// mc = m_run * c2, the term subtracted inside the exponent for this tile.
+// Lazy running max for one 32-row group: moves the exponent's reference point m_run and rescales
+// l_run and the O accumulators only when some row of the wave has grown past it by more than
+// kLazyLog2 in the log2 domain.  Until then P may exceed 1 by at most 2^kLazyLog2, which fp16 P and
+// fp32 l, O absorb without loss; the final O / l is unchanged because numerator and denominator share
+// the reference point.  Returns mc = m_run * c2, the term subtracted inside the exponent.
 template <int NT, int DT>
 AAT_DEV float lazy_max_step(const f16v (&s)[NT], float& m_run, float& l_run, f16v (&oacc)[DT], float c2) {
   const float m_tile = pair_max(lane_max<NT>(s));
@@ -95,32 +87,40 @@ AAT_DEV float lazy_max_step(const f16v (&s)[NT], float& m_run, float& l_run, f16
   return (m_run == -INFINITY ? 0.f : m_run) * c2;
 }
 
-// exp of `count` consecutive entries (flattened index e = 16*tile + v) of a row group, in place;
-// returns their sum.  Used to spread the exponentials between the MFMAs of the next score tile.
-template <int NT, bool MASKED>
-AAT_DEV float exp_range(f16v (&s)[NT], int e0, int count, float c2, float mc, int kv_base, int q_lim, int h) {
-  float sum = 0.f;
+// s <- exp2(s*c2 - mc) in place (masked entries hold -inf and come out as 0 for any positive scale).
+template <int NT> AAT_DEV void exp_tile(f16v (&s)[NT], float c2, float mc) {
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[t][v] = fast_exp2(__builtin_fmaf(s[t][v], c2, -mc));
+}
+
+// exp of `count` consecutive entries (flattened index e = 16*tile + v) of a row group, in place.
+// Used to spread the exponentials between the MFMAs of the next score tile.
+template <int NT> AAT_DEV void exp_range(f16v (&s)[NT], int e0, int count, float c2, float mc) {
 #pragma unroll
   for (int i = 0; i < count; ++i) {
     const int e = e0 + i;
-    if (e < NT * 16) {
-      const int t = e >> 4, v = e & 15;
-      float p;
-      if (MASKED && kv_base + 32 * t + c_row(v, h) > q_lim) p = 0.f;
-      else p = fast_exp2(__builtin_fmaf(MASKED ? fmaxf(s[t][v], -3.0e38f) : s[t][v], c2, -mc));
-      s[t][v] = p;
-      sum += p;
-    }
+    if (e < NT * 16) s[e >> 4][e & 15] = fast_exp2(__builtin_fmaf(s[e >> 4][e & 15], c2, -mc));
   }
-  return sum;
 }
 
-template <int NT> AAT_DEV void pack_p(h8 (&pf)[NT][2], const f16v (&s)[NT]) {
+// Round 16 kv rows (group g: score tile g/2, registers 8*(g%2) .. +7) of P to one fp16 MFMA operand and
+// add their sum to `sum`.  The sum is taken over the ROUNDED values (v_dot2_f32_f16 against ones, fp32
+// accumulate), i.e. over exactly the weights the second contraction applies, at half the instruction
+// count of fp32 adds.
+template <int NT> AAT_DEV void pack_p_group(h8 (&pf)[NT][2], const f16v (&s)[NT], int g, float& sum) {
+  const h2 ones = {(half_t)1.f, (half_t)1.f};
+  const int t = g >> 1, half = g & 1;
+  h8 r;
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    pf[t][0] = pack8_rne(s[t], 0);
-    pf[t][1] = pack8_rne(s[t], 8);
+  for (int i = 0; i < 4; ++i) {
+    const h2 pr = pack_rne(s[t][8 * half + 2 * i], s[t][8 * half + 2 * i + 1]);
+    r[2 * i] = pr[0];
+    r[2 * i + 1] = pr[1];
+    sum = __builtin_amdgcn_fdot2(pr, ones, sum, false);
   }
+  pf[t][half] = r;
 }
 
 }  // namespace aat

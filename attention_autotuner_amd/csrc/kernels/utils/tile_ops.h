@@ -78,6 +78,95 @@ AAT_DEV void pv_gemm(f16v (&oacc)[RT][DT], const h8 (&pf)[RT][NT][2], const char
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Explicitly scheduled variants.  The compiler's own ordering of ds_read / MFMA / VALU leaves the
+// first MFMA chain waiting on every LDS read and clusters vector work away from the matrix work, so
+// the two contractions below are written as a sequence of steps -- prefetch the operand PF steps
+// ahead, one MFMA group, a slice of caller-supplied vector work -- with a scheduling barrier after
+// each step that pins that order.
+
+// LDS byte address (32-bit) of a generic pointer into the dynamic LDS segment, made opaque so the
+// compiler keeps the sum base+offset in a register instead of re-adding the segment base at every use.
+AAT_DEV uint32_t lds_addr(const char* p) {
+  uint32_t a = (uint32_t)(uintptr_t)(AAT_AS3 const char*)p;
+  asm volatile("" : "+v"(a));
+  return a;
+}
+AAT_DEV h8 lds_read_h8_at(uint32_t addr) { return *reinterpret_cast<AAT_AS3 const h8*>((uintptr_t)addr); }
+AAT_DEV h4 lds_read_tr_h4_at(uint32_t addr) {
+  fp16x4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4f16((AAT_AS3 fp16x4_t*)(uintptr_t)addr);
+  h4 o;
+  __builtin_memcpy(&o, &r, 8);
+  return o;
+}
+#ifdef AAT_NOFENCE
+AAT_DEV void sched_fence() {}
+#else
+AAT_DEV void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+#endif
+
+// S^T = K Q^T over one kv tile.  kaddr[ks] = LDS address of this lane's chunk for k-step ks in score
+// tile 0 of the K buffer (tile nt adds nt*32 rows).  side(step) runs after the MFMA group of each step.
+template <int RT, int NT, int KS, int NCK, int PF, class Side>
+AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const uint32_t (&kaddr)[KS],
+                           int buf_off, Side&& side) {
+  constexpr int S = NT * KS;
+  constexpr int kTileStride = 32 * NCK * 16;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) sacc[rt][nt] = zero16();
+  h8 ring[PF];
+#pragma unroll
+  for (int i = 0; i < PF && i < S; ++i) ring[i] = lds_read_h8_at(kaddr[i % KS] + buf_off + (i / KS) * kTileStride);
+  sched_fence();
+#pragma unroll
+  for (int step = 0; step < S; ++step) {
+    const h8 cur = ring[step % PF];
+    if (step + PF < S) {
+      const int nx = step + PF;
+      ring[step % PF] = lds_read_h8_at(kaddr[nx % KS] + buf_off + (nx / KS) * kTileStride);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) sacc[rt][step / KS] = mfma_32x32x16(cur, qf[rt][step % KS], sacc[rt][step / KS]);
+    side(step);
+    sched_fence();
+  }
+}
+
+// O^T += V^T P^T over one kv tile.  vaddr[dt] = LDS address this lane presents to the transposing read
+// for d-tile dt, kv rows 0..3 (+4h) of the V buffer.  pack(g) must fill pf[*][g/2][g%2] (the P operand of
+// kv rows 16g .. 16g+15); it is called one group ahead of use, between MFMAs.
+template <int RT, int NT, int DT, int NCV, int PF, class Pack>
+AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint32_t (&vaddr)[DT], int buf_off,
+                           Pack&& pack) {
+  constexpr int G = NT * 2;              // groups of 16 kv rows
+  constexpr int S = G * DT;
+  constexpr int kRow16 = 16 * NCV * 16, kRow8 = 8 * NCV * 16;
+  h4 lo[PF], hi[PF];
+#pragma unroll
+  for (int i = 0; i < PF && i < S; ++i) {
+    lo[i] = lds_read_tr_h4_at(vaddr[i % DT] + buf_off + (i / DT) * kRow16);
+    hi[i] = lds_read_tr_h4_at(vaddr[i % DT] + buf_off + (i / DT) * kRow16 + kRow8);
+  }
+  pack(0);
+  sched_fence();
+#pragma unroll
+  for (int step = 0; step < S; ++step) {
+    const int g = step / DT, dt = step % DT;
+    const h8 vf = cat_h4(lo[step % PF], hi[step % PF]);
+    if (step + PF < S) {
+      const int nx = step + PF;
+      lo[step % PF] = lds_read_tr_h4_at(vaddr[nx % DT] + buf_off + (nx / DT) * kRow16);
+      hi[step % PF] = lds_read_tr_h4_at(vaddr[nx % DT] + buf_off + (nx / DT) * kRow16 + kRow8);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
+    if (dt == 0 && g + 1 < G) pack(g + 1);
+    sched_fence();
+  }
+}
+
 // Epilogue: scale the wave's O^T accumulators per row, round to fp16 (RNE), transpose through a
 // wave-private LDS staging area and store rows with 16-byte coalesced writes.
 // ostage: wave-private LDS, WM rows of O_STRIDE bytes.  og: global pointer to the wave's first output row.
