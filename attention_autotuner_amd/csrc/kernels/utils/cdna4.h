@@ -86,6 +86,7 @@ AAT_DEV void block_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" :::
 template <int NC> AAT_DEV constexpr int swz_rows16(int row, int c) {
   if constexpr (NC % 16 == 0) return c ^ (row & 15);
   else if constexpr (NC == 8) return c ^ ((row >> 1) & 7);
+  else if constexpr (NC == 4) return c ^ ((row >> 2) & 3);
   else return c ^ (row & 7);
 }
 // swz_rows4: for the transposing read ds_read_b64_tr_b16, where one 32-lane phase touches 4
@@ -128,13 +129,17 @@ struct TileDma {
   static constexpr int kDistinct = !kRegular ? kIters : (kDistinctRaw < kIters ? kDistinctRaw : kIters);
   uint32_t loff[kDistinct];                            // per-lane byte offsets inside a tile
 
-  AAT_DEV void init(int tid) {
+  int pitch;                                           // bytes between consecutive tile rows in global memory
+
+  // `row_pitch_bytes`: distance between rows of the source matrix (defaults to a dense tile-wide matrix).
+  AAT_DEV void init(int tid, int row_pitch_bytes = kRowBytes) {
+    pitch = row_pitch_bytes;
 #pragma unroll
     for (int i = 0; i < kDistinct; ++i) {
       const int s = i * NT + tid;
       const int row = s / NC, cs = s % NC;
       const int row0 = kRegular ? tid / NC : row;      // the uniform part carries i * kRowsPerIter rows
-      loff[i] = (uint32_t)(row0 * kRowBytes + swz<NC, MODE>(row, cs) * 16);
+      loff[i] = (uint32_t)(row0 * pitch + swz<NC, MODE>(row, cs) * 16);
     }
   }
   // Issue the copy of one tile.  `g` points at the tile's first row in global memory (wave-uniform),
@@ -147,7 +152,7 @@ struct TileDma {
   AAT_DEV void issue_part(const char* g, char* lds, int wave_base) const {
 #pragma unroll
     for (int i = I0; i < I1; ++i) {
-      uint64_t base = (uint64_t)(uintptr_t)(kRegular ? g + (size_t)i * kRowsPerIter * kRowBytes : g);
+      uint64_t base = (uint64_t)(uintptr_t)(kRegular ? g + (size_t)i * kRowsPerIter * pitch : g);
       asm volatile("" : "+s"(base));                   // keep the uniform part in SGPRs (saddr form)
       const uint32_t lane_off = loff[kRegular ? i % kDistinct : i];
       __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)(base + lane_off),
