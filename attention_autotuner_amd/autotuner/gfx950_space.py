@@ -38,15 +38,23 @@ def dma_divisible(cfg):
 def forward_lds_bytes(cfg):
     main = cfg.num_stages_qk * cfg.Bc * cfg.Kd * 2 + cfg.num_stages_v * cfg.Bc * cfg.D * 2
     if cfg.operation == "ret":
-        main += cfg.num_stages_mask * cfg.Br * cfg.Bc * 2
+        main += max(cfg.num_stages_mask, cfg.num_stages_qk) * cfg.Br * cfg.Bc * 2
     if cfg.fuse_type == "shared":
         main += cfg.Br * (cfg.Bc * 2 + 16)            # P tile, fp16, padded rows
+        main += (cfg.warps_mma1_n * cfg.Br + cfg.Br) * 4 + 64
+        return max(main, cfg.Br * (cfg.D * 2 + 16 * cfg.warps_mma_n))
     epilogue = cfg.Br * (cfg.D * 2 + 16)
     return max(main, epilogue)
 
 
 def forward_reg_estimate(cfg):
     """Per-lane 32-bit registers of the dominant live set."""
+    if cfg.fuse_type == "shared":
+        nw = _waves(cfg)
+        rt1 = cfg.Br // (nw // cfg.warps_mma1_n) // 32
+        nt1 = cfg.Bc // cfg.warps_mma1_n // 32
+        o_regs = cfg.Br * cfg.D // (nw * 64)
+        return rt1 * (cfg.Kd // 16) * 4 + rt1 * nt1 * 16 + o_regs + 48
     rt = rows_per_wave(cfg) // MFMA_M
     q_regs = rt * (cfg.Kd // 16) * 4
     s_regs = rt * (cfg.Bc // 32) * 16
@@ -58,11 +66,27 @@ def forward_reg_estimate(cfg):
         o_regs = (cfg.Br // MFMA_M) * (cfg.D // 32) * 16 // _waves(cfg)
     if getattr(cfg, "sw_pipeline", 0):
         s_regs *= 2                                   # current and next score tile are both live
+    if o_regs > 128 and q_regs + s_regs + o_regs > 320:
+        return 10 ** 6                                # measured: hipcc spills heavily beyond this point
     return q_regs + s_regs + p_regs + o_regs + 32
 
 
+def shared_grid_ok(cfg):
+    """Wave grids of the LDS-fused kernels: W1M x W1N over (rows, kv), W2M x W2N over (rows, d)."""
+    nw, w1n, w2n = _waves(cfg), cfg.warps_mma1_n, cfg.warps_mma_n
+    if not w1n or not w2n or nw % w1n or nw % w2n:
+        return False
+    w1m, w2m = nw // w1n, nw // w2n
+    if cfg.Br % (32 * w1m) or cfg.Bc % (32 * w1n) or cfg.Br % (32 * w2m) or cfg.D % (32 * w2n):
+        return False
+    return True
+
+
 def forward_valid(cfg, arch):
-    if cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * _waves(cfg)):
+    if cfg.fuse_type == "shared":
+        if cfg.Nthreads % WAVE or not shared_grid_ok(cfg):
+            return False
+    elif cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * _waves(cfg)):
         return False
     if cfg.Bc % 32 or cfg.Kd % 64 or cfg.D % 64:
         return False
@@ -88,14 +112,32 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
         for st_qk, st_v in STAGES:
             for wpe in (1, 2, 3):
                 for fuse in fuse_types:
+                    if fuse == "shared":
+                        out.extend(_shared_candidates(op, br, bc, dim_qk, dim_v, st_qk, st_v, nthreads, wpe))
+                        continue
                     if op == "attn":
                         cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, waves_per_eu=wpe)
                     else:
-                        cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, 1, st_v, nthreads, True, waves_per_eu=wpe)
+                        cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_qk, st_v, nthreads, True, waves_per_eu=wpe)
                     out.append(cfg.set_fuse_type(fuse))
                     if op == "attn" and fuse == "register" and (st_qk, st_v) == (2, 2):
                         piped = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 2, 2, nthreads, True, waves_per_eu=wpe, sw_pipeline=1)
                         out.append(piped.set_fuse_type(fuse))
+    return out
+
+
+def _shared_candidates(op, br, bc, dim_qk, dim_v, st_qk, st_v, nthreads, wpe):
+    out = []
+    nw = nthreads // WAVE
+    for w1n in (1, 2):
+        for w2n in sorted({nw, max(1, nw // 2)}):
+            if op == "attn":
+                cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, w1n, w2n, waves_per_eu=wpe)
+            else:
+                cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_qk, st_v, nthreads, True, w1n, w2n, waves_per_eu=wpe)
+            cfg.fuse_type = "shared"
+            if shared_grid_ok(cfg):
+                out.append(cfg)
     return out
 
 
@@ -109,8 +151,19 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
         if op == "attn":
             cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, sq, sv, nt, True, waves_per_eu=wpe)
         else:
-            cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, sq, 1, sv, nt, True, waves_per_eu=wpe)
+            cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, sq, sq, sv, nt, True, waves_per_eu=wpe)
         cfg.set_fuse_type("register")
+        if forward_valid(cfg, arch):
+            return cfg
+    # wide value heads: the LDS-fused kernel keeps the accumulator at Br*D/(64*waves) registers
+    for br, bc, nt, w1n, w2n in ((128, 64, 512, 2, 8), (64, 64, 256, 2, 4)):
+        if (seq_q and seq_q % br) or (seq_k and seq_k % bc):
+            continue
+        if op == "attn":
+            cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 1, 1, nt, True, w1n, w2n, waves_per_eu=1)
+        else:
+            cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 1, 1, 1, nt, True, w1n, w2n, waves_per_eu=1)
+        cfg.fuse_type = "shared"
         if forward_valid(cfg, arch):
             return cfg
     raise ValueError(f"no default {op} configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
