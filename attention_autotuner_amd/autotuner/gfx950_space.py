@@ -160,9 +160,9 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
         if (seq_q and seq_q % br) or (seq_k and seq_k % bc):
             continue
         if op == "attn":
-            cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 1, 1, nt, True, w1n, w2n, waves_per_eu=1)
+            cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 1, 1, nt, True, w1n, w2n, waves_per_eu=nt // 256)
         else:
-            cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 1, 1, 1, nt, True, w1n, w2n, waves_per_eu=1)
+            cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 1, 1, 1, nt, True, w1n, w2n, waves_per_eu=nt // 256)
         cfg.fuse_type = "shared"
         if forward_valid(cfg, arch):
             return cfg

@@ -18,6 +18,8 @@ from .configs import supported_configs
 # (operator, d_qk, d_v) pairs whose default configuration is always built
 DEFAULT_PROBLEMS = [
     ("attn", 64, 64), ("attn", 128, 128), ("attn", 256, 256), ("attn", 192, 192), ("attn", 256, 128), ("attn", 64, 128),
+    ("attn", 256, 512),
+    ("ret", 64, 64), ("ret", 128, 128), ("ret", 256, 256), ("ret", 64, 128), ("ret", 256, 512),
 ]
 
 

@@ -110,7 +110,12 @@ def test_mi355x_space_is_valid_and_nonempty():
         reg = [c for c in cfgs if c.fuse_type == "register"]
         assert reg, (dqk, dv)
         for c in cfgs:
-            assert c.Br % (32 * (c.Nthreads // 64)) == 0
+            if c.fuse_type == "register":
+                assert c.Br % (32 * (c.Nthreads // 64)) == 0      # every wave owns whole 32-row groups
+            else:
+                nw = c.Nthreads // 64
+                assert nw % c.warps_mma1_n == 0 and nw % c.warps_mma_n == 0
+                assert c.Bc % (32 * c.warps_mma1_n) == 0 and dv % (32 * c.warps_mma_n) == 0
             assert c.BlockKSmem == dqk and c.BlockKSmem2 == c.Bc
     with pytest.raises(RuntimeError):
         AttnTunner(A100(), _fake_arrays(64, 64)).tune()
