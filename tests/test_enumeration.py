@@ -108,7 +108,10 @@ def test_mi355x_space_is_valid_and_nonempty():
     for dqk, dv in ((64, 64), (128, 128), (256, 256), (256, 512)):
         cfgs = AttnTunner(arch, _fake_arrays(dqk, dv)).get_tuned_configs()
         reg = [c for c in cfgs if c.fuse_type == "register"]
-        assert reg, (dqk, dv)
+        shared = [c for c in cfgs if c.fuse_type == "shared"]
+        assert shared, (dqk, dv)
+        # d_v = 512 puts 256 accumulator registers on every lane of a register-fused wave: LDS-fused only
+        assert bool(reg) == (dv < 512), (dqk, dv)
         for c in cfgs:
             if c.fuse_type == "register":
                 assert c.Br % (32 * (c.Nthreads // 64)) == 0      # every wave owns whole 32-row groups
