@@ -79,6 +79,8 @@ class BaseTunner:
 
     def _fits_problem(self, config):
         s = self.problem_shape
+        if config.operation == "ret_bwd":             # both lengths are resident in one pass, streamed in another
+            return all(s[n] % config.Br == 0 and s[n] % config.Bc == 0 for n in ("Sq", "Sk"))
         return s["Sq"] % config.Br == 0 and s["Sk"] % config.Bc == 0
 
     def get_tuned_configs(self):

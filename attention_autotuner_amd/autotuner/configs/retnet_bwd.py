@@ -4,8 +4,11 @@ from .base_config import BaseConfig
 class RetBwdConfig(BaseConfig):
     """RetNet parallel backward (reference python/autotuner/configs/retnet_bwd.py:4-26).
 
-    The ``mmawarpsN*`` fields say how the block's waves are split along the N side of each of the
-    contractions (S/dS, dV, dK, dQ)."""
+    On MI355X the gradient is three passes (dV, dK, dQ) of one chained-contraction kernel: ``Br`` is the
+    number of block-resident rows and ``Bc`` the number of streamed rows per step of every pass;
+    ``num_stages_qk`` / ``num_stages_dv`` are the LDS buffer counts of the two streams.  The ``mmawarpsN*``
+    fields (how the reference splits its warps along the N side of each contraction) are carried for
+    file compatibility; every wave here owns whole rows."""
     operation = "ret_bwd"
     kernel_subdir = "retnet/bwd"
     _fields = ("Br", "Bc", "Kd", "D", "mmawarpsN", "mmawarpsN_dv", "mmawarpsN_dk", "mmawarpsN_dq", "Nthreads",

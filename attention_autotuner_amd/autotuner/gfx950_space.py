@@ -167,3 +167,69 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
         if forward_valid(cfg, arch):
             return cfg
     raise ValueError(f"no default {op} configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
+
+
+# ---- backward (RetNet) ---------------------------------------------------------------------------------
+# Three passes of one chained-contraction kernel (dV, dK, dQ).  Br = block-resident rows, Bc = streamed rows
+# per step, for every pass; both sequence lengths must divide by both.
+BWD_BR_LIST = (64, 128)
+BWD_BC_LIST = (32, 64)
+
+
+def backward_lds_bytes(cfg):
+    worst = 0
+    dvb = min(cfg.D, 256)
+    for kx, dzb in ((cfg.Kd, dvb), (cfg.D, cfg.Kd), (cfg.D, cfg.Kd)):
+        main = cfg.num_stages_qk * (cfg.Bc * kx * 2 + cfg.Br * cfg.Bc * 2) + cfg.num_stages_dv * cfg.Bc * dzb * 2
+        worst = max(worst, main, cfg.Br * (dzb * 2 + 16))
+    return worst
+
+
+def backward_reg_estimate(cfg):
+    rt = cfg.Br // _waves(cfg) // MFMA_M
+    worst = 0
+    dvb = min(cfg.D, 256)
+    for kx, dzb in ((cfg.Kd, dvb), (cfg.D, cfg.Kd)):
+        worst = max(worst, rt * (kx // 16) * 4 + rt * (cfg.Bc // 32) * 24 + rt * (dzb // 32) * 16 + 64)
+    return worst
+
+
+def backward_valid(cfg, arch):
+    nw = _waves(cfg)
+    if cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * nw) or cfg.Bc % 32:
+        return False
+    if nw > 4 * cfg.waves_per_eu:
+        return False
+    nt = cfg.Nthreads
+    dvb = min(cfg.D, 256)
+    for cols in (cfg.Kd, cfg.D, dvb, cfg.Br):          # every streamed tile must split evenly over the threads
+        if (cfg.Bc * cols // 8) % nt:
+            return False
+    if (cfg.Br * cfg.Bc // 8) % nt:
+        return False
+    if backward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
+        return False
+    return backward_reg_estimate(cfg) <= arch.register_per_thread // cfg.waves_per_eu
+
+
+def backward_candidates(br, bc, dim_qk, dim_v):
+    out = []
+    for nthreads in (128, 256):
+        for st_y, st_z in ((1, 1), (2, 2), (2, 1)):
+            for wpe in (1, 2):
+                n = nthreads // WAVE
+                out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, BlockKSmem=dim_qk,
+                                        num_stages_qk=st_y, num_stages_mask=st_y, num_stages_dv=st_z, waves_per_eu=wpe))
+    return out
+
+
+def default_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
+    for br, bc, nt, sy, sz, wpe in ((64, 32, 128, 1, 1, 1), (64, 32, 128, 1, 1, 2), (64, 64, 128, 1, 1, 1)):
+        if any(s and (s % br or s % bc) for s in (seq_q, seq_k)):
+            continue
+        n = nt // WAVE
+        cfg = RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nt, True, BlockKSmem=dim_qk, num_stages_qk=sy,
+                           num_stages_mask=sy, num_stages_dv=sz, waves_per_eu=wpe)
+        if backward_valid(cfg, arch):
+            return cfg
+    raise ValueError(f"no default ret_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")

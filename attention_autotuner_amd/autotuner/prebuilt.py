@@ -16,6 +16,9 @@ from .base_tunner import DEFAULT_CACHE_DIR
 from .configs import supported_configs
 
 # (operator, d_qk, d_v) pairs whose default configuration is always built
+# attention smemfuse variants exercised by the parity suite: (Br, Bc, Nthreads, K bufs, V bufs, W1N, W2N, waves/SIMD)
+SHARED_TILES = [(128, 64, 256, 2, 2, 1, 4, 2), (64, 64, 256, 1, 1, 2, 4, 2), (64, 64, 256, 2, 1, 2, 2, 2)]
+
 DEFAULT_PROBLEMS = [
     ("attn", 64, 64), ("attn", 128, 128), ("attn", 256, 256), ("attn", 192, 192), ("attn", 256, 128), ("attn", 64, 128),
     ("attn", 256, 512),
@@ -35,9 +38,18 @@ PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
 
 def extra_configs(arch=None):
     """Additional libraries built ahead of time: the parity matrix."""
-    from .configs import AttnConfig
+    from .configs import AttnConfig, RetConfig
     arch = arch or MI355X()
     out = []
+    # RetNet forward variants at 128/128 (register and both wave grids of the LDS-fused kernel)
+    for fuse, extra in (("register", {}), ("shared", dict(warps_mma1_n=1, warps_mma_n=4)), ("shared", dict(warps_mma1_n=2, warps_mma_n=2))):
+        for st in ((1, 1), (2, 2)):
+            cfg = RetConfig(128 if fuse == "register" else 64, 64, 128, 128, 128, 64, st[0], st[0], st[1], 256, True, waves_per_eu=1, **extra)
+            cfg.fuse_type = fuse
+            if gfx950_space.forward_valid(cfg, arch):
+                out.append(cfg)
+    for dims in ((64, 64), (128, 128), (256, 256), (64, 128), (256, 512)):
+        out.append(gfx950_space.default_backward_config(*dims, arch, 128, 128))
     for dqk, dv in PARITY_DIMS:
         for br, bc, nt, sq, sv, wpe in PARITY_TILES:
             cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
@@ -47,6 +59,12 @@ def extra_configs(arch=None):
                 piped = AttnConfig(br, bc, dqk, dv, dqk, bc, 2, 2, nt, True, waves_per_eu=wpe, sw_pipeline=1).set_fuse_type("register")
                 if gfx950_space.forward_valid(piped, arch):
                     out.append(piped)
+    for dqk, dv in ((64, 64), (128, 128), (256, 512)):
+        for br, bc, nt, sq, sv, w1n, w2n, wpe in SHARED_TILES:
+            cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, w1n, w2n, waves_per_eu=wpe)
+            cfg.fuse_type = "shared"
+            if gfx950_space.forward_valid(cfg, arch):
+                out.append(cfg)
     return out
 
 
@@ -69,6 +87,8 @@ def shipping_set(arch=None):
         if op in ("attn", "ret"):
             for seq in (None, 128, 64):          # defaults differ with what the sequence length divides by
                 cfgs.append(gfx950_space.default_forward_config(op, dqk, dv, arch, seq, seq))
+        if op == "ret":
+            cfgs.append(gfx950_space.default_backward_config(dqk, dv, arch))
     cfgs += extra_configs(arch)
     cfgs += cached_configs()
     seen, unique = set(), []

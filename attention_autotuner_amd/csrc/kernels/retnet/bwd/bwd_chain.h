@@ -1,0 +1,274 @@
+// RetNet parallel retention backward for gfx950 (MI355X).
+//
+// With r held constant (the reference detaches it), P = (Q K^T * M) / r and
+//     dV = P^T dO,      dS = (dO V^T / r) * M,      dK = dS^T Q,      dQ = dS K,
+// P and dS rounded to fp16 before the dependent contraction, fp32 accumulation -- the arithmetic of
+// the reference's column-block kernel (reference: csrc/kernels/retnet/bwd/bwd_colblock.h:445-596, closed
+// forms at :522-576, fp16 rounding at :509 and :551).
+//
+// The reference walks (kv block, q block) pairs once, keeps dK and dV in registers and pushes dQ
+// through fp32 atomics into scratch that a second kernel converts (convert_dq, :742-811).  On MI355X
+// the atomic traffic (S_q*S_kv/Bc*Kd*4 bytes per head) costs more than the arithmetic it saves and
+// dK + dV do not fit one wave's registers at d_qk=256, d_v=512.  Each gradient is instead its own pass
+// of one "chained contraction" kernel, the same shape as the forward kernel:
+//
+//     T^T[y][x] = sum_k Y[y][k] X[x][k]      X: block-resident rows (a lane owns one), Y: streamed tiles
+//     E[y][x]   = half( T * M / r )
+//     Out[x][:] = sum_y E[y][x] Z[y][:]      Z: streamed tiles, read transposed
+//
+//     pass      X    Y    Z    Out   lane owns   r index   mask access
+//     dV  COL   K    Q    dO   dV    kv row      y (q)     transposed (ds_read_b64_tr_b16)
+//     dK  COL   V    dO   Q    dK    kv row      y (q)     transposed
+//     dQ  ROW   dO   V    K    dQ    q row       x (q)     row-major
+//
+// No atomics, no scratch, deterministic; dQ is written directly in fp16, so the reference's second
+// kernel has no counterpart.  Cost: dO V^T is evaluated twice (3*(d_qk+d_v) instead of 3*d_qk+2*d_v
+// multiply-adds per score) and, for an output wider than DZB columns, the first contraction is repeated
+// per column slice (grid.y slices).
+#pragma once
+#include <type_traits>
+
+#include "../../utils/cdna4.h"
+#include "../../utils/retention.h"
+#include "../../utils/tile_ops.h"
+
+#ifndef AAT_PF
+#define AAT_PF 2
+#endif
+
+namespace aat {
+
+enum class BwdPass { Col, Row };
+
+// KX: contraction width of the first product (columns of X and Y); DZ: columns of Z and Out;
+// DZB: output columns handled by one block (DZ / DZB blocks along grid.y);
+// BX: resident rows per block; BY: rows per streamed tile; NSY / NSZ: LDS buffers of the Y(+mask) and Z streams.
+template <int KX, int DZ, int DZB, int BX, int BY, int Nthreads, int NSY, int NSZ, BwdPass PASS>
+struct RetBwdChain {
+  static constexpr int NW = Nthreads / kWave;
+  static constexpr int WM = BX / NW;
+  static constexpr int RT = WM / 32;
+  static constexpr int NT = BY / 32;
+  static constexpr int KS = KX / 16;
+  static constexpr int DT = DZB / 32;
+  static constexpr int NCY = KX / 8, NCZ = DZB / 8;
+  // mask tile: rows = q, columns = kv.  COL: q is the streamed index (BY rows x BX columns); ROW: BX rows x BY columns.
+  static constexpr int kMRows = PASS == BwdPass::Col ? BY : BX;
+  static constexpr int kMCols = PASS == BwdPass::Col ? BX : BY;
+  static constexpr int NCM = kMCols / 8;
+  static_assert(Nthreads % kWave == 0 && BX % NW == 0 && WM % 32 == 0, "each wave owns whole 32-row groups");
+  static_assert(BY % 32 == 0 && KX % 64 == 0 && DZ % DZB == 0 && DZB % 64 == 0, "tile shape");
+  static_assert((NSY == 1 || NSY == 2) && (NSZ == 1 || NSZ == 2), "buffers");
+  using YDma = TileDma<BY, NCY, Nthreads, Swz::Rows16>;
+  using ZDma = TileDma<BY, NCZ, Nthreads, Swz::Rows4>;
+  using MDma = TileDma<kMRows, NCM, Nthreads, PASS == BwdPass::Col ? Swz::Rows4 : Swz::Rows16>;
+  static constexpr int kYBytes = BY * KX * 2, kZBytes = BY * DZB * 2, kMBytes = kMRows * kMCols * 2;
+  static constexpr int kOStride = DZB * 2 + 16;
+  static constexpr int kMainBytes = NSY * (kYBytes + kMBytes) + NSZ * kZBytes;
+  static constexpr int kEpiBytes = BX * kOStride;
+  static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
+};
+
+// x, y, z, out: [B*H, S, width] fp16 with S = seq_x for x/out and seq_y for y/z; mask [H, seq_q, seq_k];
+// r [B*H, seq_q].  For COL passes seq_x = seq_k, seq_y = seq_q; for the ROW pass the other way round.
+// `causal` promises mask == 0 above the diagonal and only shortens the walk over streamed tiles.
+template <int KX, int DZ, int DZB, int BX, int BY, int Nthreads, int NSY, int NSZ, BwdPass PASS, int WPE = 1>
+__global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
+ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const half_t* __restrict__ z,
+              const half_t* __restrict__ mask, const float* __restrict__ r, half_t* __restrict__ out, int H,
+              int seq_k, int seq_q, int causal) {
+  using T = RetBwdChain<KX, DZ, DZB, BX, BY, Nthreads, NSY, NSZ, PASS>;
+  constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCY = T::NCY, NCZ = T::NCZ, NCM = T::NCM, WM = T::WM;
+  constexpr int PF = AAT_PF;
+  constexpr bool COL = PASS == BwdPass::Col;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  char* const ybuf = smem;
+  char* const mbuf = smem + NSY * T::kYBytes;
+  char* const zbuf = mbuf + NSY * T::kMBytes;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int seq_x = COL ? seq_k : seq_q, seq_y = COL ? seq_q : seq_k;
+
+  const int Tx = seq_x / BX;
+  const int tile = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = tile / Tx;
+  const int x0 = (tile % Tx) * BX;
+  const int dz0 = blockIdx.y * DZB;               // first output column of this block
+  const int diag = seq_k - seq_q;                 // mask[q][kv] may be non-zero only for kv <= q + diag
+  int j_begin = 0, j_end = seq_y / BY;
+  if (causal) {
+    if constexpr (COL) {                          // q tiles that reach kv >= x0:  q >= x0 - diag
+      const int first = x0 - diag;
+      j_begin = first <= 0 ? 0 : first / BY;
+    } else {                                      // kv tiles with kv <= x0 + BX - 1 + diag
+      const int last = x0 + BX - 1 + diag;
+      const int lim = last < 0 ? 0 : last / BY + 1;
+      j_end = lim < j_end ? lim : j_end;
+    }
+  }
+
+  const char* yg = reinterpret_cast<const char*>(y + (size_t)bh * seq_y * KX);
+  const char* zg = reinterpret_cast<const char*>(z + ((size_t)bh * seq_y) * DZ + dz0);
+  // mask tile origin: COL -> rows = streamed q, columns = resident kv;  ROW -> rows = resident q, columns = streamed kv
+  const half_t* mhead = mask + (size_t)(bh % H) * seq_q * seq_k;
+  const char* mg = reinterpret_cast<const char*>(COL ? mhead + x0 : mhead + (size_t)x0 * seq_k);
+
+  typename T::YDma ydma;
+  typename T::ZDma zdma;
+  typename T::MDma mdma;
+  ydma.init(tid);
+  zdma.init(tid, DZ * 2);
+  mdma.init(tid, seq_k * 2);
+  const int wave_base = wave * 64;
+
+  h8 xf[RT][KS];
+  load_q_frags<RT, KS, KX>(xf, x + ((size_t)bh * seq_x + x0 + wave * WM + n) * KX + 8 * h);
+  uint32_t yaddr[KS], zaddr[DT], maddr[RT][NT * 4];
+  {
+    int yoff[KS], zoff[DT];
+    k_frag_offsets<KS, NCY>(yoff, n, h);
+    v_frag_offsets<DT, NCZ>(zoff, lane);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) yaddr[ks] = lds_addr(ybuf + yoff[ks]);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) zaddr[dt] = lds_addr(zbuf + zoff[dt]);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < NT * 4; ++i) {
+        if constexpr (COL) {
+          // transposing read: score tile t = i/4, register group g = i%4 -> q rows 32t + 8g + 4h + (lane%16)/4,
+          // kv columns wave*WM + 32rt + 16*((lane/16)%2) + 4*(lane%4) .. +3; this lane receives column n.
+          const int s16 = lane & 15;
+          const int row = 32 * (i >> 2) + 8 * (i & 3) + 4 * h + (s16 >> 2);
+          const int col = wave * WM + rt * 32 + 16 * ((lane >> 4) & 1) + 4 * (s16 & 3);
+          maddr[rt][i] = lds_addr(mbuf + lds_chunk_off<NCM, Swz::Rows4>(row, col >> 3) + (col & 7) * 2);
+        } else {
+          maddr[rt][i] = lds_addr(mbuf + lds_chunk_off<NCM, Swz::Rows16>(wave * WM + rt * 32 + n, i) + 8 * h);
+        }
+      }
+  }
+  float inv_r_row[RT];                            // ROW pass: 1/r of the lane's own query row
+  if constexpr (!COL) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) inv_r_row[rt] = fast_rcp(r[(size_t)bh * seq_q + x0 + wave * WM + rt * 32 + n]);
+  }
+  const float* rg = r + (size_t)bh * seq_q;       // COL pass: r of the streamed query rows
+
+  f16v acc[RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = zero16();
+
+  auto issue_ym = [&](int j, int par) {           // Y tile j and mask tile j travel together
+    ydma.issue(yg + (size_t)j * T::kYBytes, ybuf + (NSY == 2 ? par * T::kYBytes : 0), wave_base);
+    const char* msrc = COL ? mg + (size_t)j * BY * seq_k * 2 : mg + (size_t)j * BY * 2;
+    mdma.issue(msrc, mbuf + (NSY == 2 ? par * T::kMBytes : 0), wave_base);
+  };
+  auto issue_z = [&](int j, int par) {
+    zdma.issue(zg + (size_t)j * BY * DZ * 2, zbuf + (NSZ == 2 ? par * T::kZBytes : 0), wave_base);
+  };
+  if (j_begin < j_end) {
+    issue_ym(j_begin, 0);
+    if constexpr (NSZ == 2) issue_z(j_begin, 0);
+  }
+  auto y_tile = [&](const int j, auto parity_tag) {
+    constexpr int PAR = decltype(parity_tag)::value;
+    const bool more = (j + 1 < j_end);
+    // (A) Y_j, mask_j (and with two Z buffers Z_j) have landed; every wave is past the previous tile.
+    wait_vmcnt<0>();
+    block_sync();
+    if constexpr (NSZ == 1) issue_z(j, 0);
+    if (more) {
+      if constexpr (NSY == 2) issue_ym(j + 1, PAR ^ 1);
+      if constexpr (NSZ == 2) issue_z(j + 1, PAR ^ 1);
+    }
+    f4v rv[COL ? NT * 4 : 1];                     // COL pass: r of this tile's query rows, as this lane sees them
+    if constexpr (COL) {
+#pragma unroll
+      for (int i = 0; i < NT * 4; ++i)
+        rv[i] = *reinterpret_cast<const f4v*>(rg + j * BY + 32 * (i >> 2) + 8 * (i & 3) + 4 * h);
+    }
+
+    f16v tacc[RT][NT];
+    qk_gemm_steps<RT, NT, KS, NCY, PF>(tacc, xf, yaddr, NSY == 2 ? PAR * T::kYBytes : 0, [](int) {});
+    const int moff = NSY == 2 ? PAR * T::kMBytes : 0;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      if constexpr (COL) {
+#pragma unroll
+        for (int i = 0; i < NT * 4; ++i) {
+          const h4 m = lds_read_tr_h4_at(maddr[rt][i] + moff);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            tacc[rt][i >> 2][4 * (i & 3) + e] *= (float)m[e] * fast_rcp(rv[i][e]);
+        }
+      } else {
+        apply_mask<NT>(tacc[rt], maddr[rt], moff);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int vv = 0; vv < 16; ++vv) tacc[rt][t][vv] *= inv_r_row[rt];
+      }
+    }
+
+    // (B) with one buffer: Z_j must have landed / Y and mask buffers must be free before the next fetch.
+    if constexpr (NSZ == 1 || NSY == 1) {
+      if constexpr (NSZ == 1) wait_vmcnt<0>();
+      block_sync();
+      if constexpr (NSY == 1) {
+        if (more) issue_ym(j + 1, 0);
+      }
+    }
+    h8 ef[RT][NT][2];
+    pv_gemm_steps<RT, NT, DT, NCZ, PF>(acc, ef, zaddr, NSZ == 2 ? PAR * T::kZBytes : 0, [&](int g) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) pack_group<NT>(ef[rt], tacc[rt], g);
+    });
+  };
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  for (int j = j_begin; j < j_end; j += 2) {
+    y_tile(j, P0{});
+    if (j + 1 < j_end) y_tile(j + 1, P1{});
+  }
+
+  wait_vmcnt<0>();
+  block_sync();
+  float one[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) one[rt] = 1.f;
+  // the staging rows are DZB wide; the global rows are DZ wide
+  {
+    char* const ostage = smem + wave * WM * T::kOStride;
+    half_t* og = out + ((size_t)bh * seq_x + x0 + wave * WM) * DZ + dz0;
+    constexpr int kChunksPerRow = DZB / 8;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const h2 a = pack_rne(acc[rt][dt][4 * g] * one[rt], acc[rt][dt][4 * g + 1]);
+          const h2 b = pack_rne(acc[rt][dt][4 * g + 2], acc[rt][dt][4 * g + 3]);
+          h4 w;
+          w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
+          *reinterpret_cast<h4*>(ostage + (rt * 32 + n) * T::kOStride + (32 * dt + 8 * g + 4 * h) * 2) = w;
+        }
+    wait_lgkm0();
+    constexpr int kChunks = WM * kChunksPerRow;
+#pragma unroll
+    for (int t = 0; t < kChunks / 64; ++t) {
+      const int idx = t * 64 + lane;
+      const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
+      const u4v val = *reinterpret_cast<const u4v*>(ostage + row * T::kOStride + c * 16);
+      *reinterpret_cast<u4v*>(reinterpret_cast<char*>(og) + (size_t)row * DZ * 2 + c * 16) = val;
+    }
+  }
+}
+
+}  // namespace aat

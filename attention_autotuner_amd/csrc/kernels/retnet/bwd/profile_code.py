@@ -1,0 +1,94 @@
+"""Source text of the per-configuration wrapper for the RetNet backward passes
+(same role as reference csrc/kernels/retnet/bwd/profile_code.py:1-119).
+
+One library launches three passes of the chained-contraction kernel (dV, dK, dQ); ``Br`` is the number
+of block-resident rows and ``Bc`` the number of streamed rows per step of every pass.  ``dqaccum`` is
+accepted for ABI compatibility and never touched: dQ is produced directly, without atomics.
+"""
+
+global_vars = r"""
+#define AAT_OP_RET_BWD 1
+#include "aat_kernel_abi.h"
+#include "kernels/retnet/bwd/bwd_chain.h"
+#include "kernels/utils/host_launch.h"
+
+namespace {{
+constexpr int Br = {Br};                 // block-resident rows of every pass
+constexpr int Bc = {Bc};                 // streamed rows per step of every pass
+constexpr int Kd = {Kd};
+constexpr int D = {D};
+constexpr int Nthreads = {Nthreads};
+constexpr int num_stages_qk = {num_stages_qk};   // LDS buffers of the first-contraction stream (+ mask)
+constexpr int num_stages_dv = {num_stages_dv};   // LDS buffers of the second-contraction stream
+constexpr int waves_per_eu = {waves_per_eu};
+constexpr int DVB = D > 256 ? 256 : D;           // dV columns per block (wider outputs are sliced over grid.y)
+constexpr int DKB = Kd;
+
+using aat::BwdPass;
+using TV = aat::RetBwdChain<Kd, D, DVB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col>;
+using TK = aat::RetBwdChain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col>;
+using TQ = aat::RetBwdChain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row>;
+const auto kernel_dv = &aat::ret_bwd_chain<Kd, D, DVB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu>;
+const auto kernel_dk = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu>;
+const auto kernel_dq = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row, waves_per_eu>;
+
+bool bwd_shape_ok(int B, int H, int Seq_q, int Seq_k) {{
+  // every sequence length plays both roles (resident rows in one pass, streamed rows in another)
+  return aat::shape_ok(B, H, Seq_q, Seq_k, Br, Br) && aat::shape_ok(B, H, Seq_q, Seq_k, Bc, Bc);
+}}
+
+hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
+                  aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k, int causal, hipStream_t stream) {{
+  static const hipError_t ok1 = aat::allow_lds(kernel_dv, TV::kSmemBytes);
+  static const hipError_t ok2 = aat::allow_lds(kernel_dk, TK::kSmemBytes);
+  static const hipError_t ok3 = aat::allow_lds(kernel_dq, TQ::kSmemBytes);
+  if (ok1 != hipSuccess) return ok1;
+  if (ok2 != hipSuccess) return ok2;
+  if (ok3 != hipSuccess) return ok3;
+  using H16 = aat::half_t;
+  const H16 *Q = reinterpret_cast<const H16*>(q), *K = reinterpret_cast<const H16*>(k), *V = reinterpret_cast<const H16*>(v),
+            *M = reinterpret_cast<const H16*>(mask), *G = reinterpret_cast<const H16*>(dO);
+  kernel_dv<<<dim3(B * H * (Seq_k / Br), D / DVB), dim3(Nthreads), TV::kSmemBytes, stream>>>(
+      K, Q, G, M, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, causal);
+  kernel_dk<<<dim3(B * H * (Seq_k / Br), Kd / DKB), dim3(Nthreads), TK::kSmemBytes, stream>>>(
+      V, G, Q, M, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, causal);
+  kernel_dq<<<dim3(B * H * (Seq_q / Br), Kd / DKB), dim3(Nthreads), TQ::kSmemBytes, stream>>>(
+      G, V, K, M, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, causal);
+  return hipGetLastError();
+}}
+}}  // namespace
+
+extern "C" int abi_version(void) {{ return AAT_ABI_VERSION; }}
+extern "C" const char* config_string(void) {{ return "{config_name}"; }}
+extern "C" size_t workspace_size(int, int, int, int) {{ return 0; }}
+"""
+
+profile_func = r"""
+extern "C" float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
+                            aat_half* dk, aat_half* dv, float*, int B, int H, int Seq_q, int Seq_k, int causal, void*,
+                            size_t, void* stream) {{
+  if (!bwd_shape_ok(B, H, Seq_q, Seq_k)) return -1.f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return aat::timed_mean_ms(s, [&] {{ return launch(q, k, v, mask, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, causal, s); }});
+}}
+extern "C" float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
+                         aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q, int Seq_k) {{
+  return profile_ex(q, k, v, mask, dO, r, dq, dk, dv, dqaccum, B, H, Seq_q, Seq_k, 0, nullptr, 0, nullptr);
+}}
+"""
+
+kernel_entry = r"""
+extern "C" int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
+                               aat_half* dq, aat_half* dk, aat_half* dv, float*, int B, int H, int Seq_q, int Seq_k,
+                               int causal, void*, size_t, void* stream) {{
+  if (!bwd_shape_ok(B, H, Seq_q, Seq_k)) return AAT_ERR_SHAPE;
+  return (int)launch(q, k, v, mask, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, causal, static_cast<hipStream_t>(stream));
+}}
+extern "C" int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
+                            aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_k, int Seq_q) {{
+  return kernel_entry_ex(q, k, v, mask, dO, r, dq, dk, dv, dqaccum, B, H, Seq_q, Seq_k, 0, nullptr, 0, nullptr);
+}}
+"""
+
+profile_code = global_vars + profile_func + kernel_entry
+kernel_code = profile_code

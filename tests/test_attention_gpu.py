@@ -110,6 +110,27 @@ def test_every_configuration_agrees_with_the_oracle(dqk, dv):
     assert ran >= 3
 
 
+@pytest.mark.parametrize("dqk,dv", [(64, 64), (128, 128), (256, 512)])
+def test_lds_fused_variants_agree_with_the_oracle(dqk, dv):
+    from attention_autotuner_amd.autotuner.prebuilt import SHARED_TILES
+    q, k, v = _inputs(1, 2, 128, 256, dqk, dv, seed=8)
+    refs = {c: ref_op.attention_ref(q, k, v, None, c) for c in (False, True)}
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    ran = 0
+    for br, bc, nt, sq, sv, w1n, w2n, wpe in SHARED_TILES:
+        cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, w1n, w2n, waves_per_eu=wpe)
+        cfg.fuse_type = "shared"
+        if not gfx950_space.forward_valid(cfg, ARCH):
+            continue
+        assert os.path.exists(codegen.library_path(cfg)), f"library for {cfg} was not built ahead of time"
+        for causal in (False, True):
+            o = torch.zeros(1, 2, 128, dv, dtype=torch.float16, device="cuda")
+            Runtime(ARCH, cfg).apply([qc, kc, vc, o], causal=causal)
+            assert _err(o, refs[causal]) <= TOL, (cfg, causal)
+        ran += 1
+    assert ran >= 1
+
+
 def test_reference_signature_entry_points():
     """profile / kernel_entry keep the reference's argument order (kernel_entry swaps the lengths)
     and its literal behaviour: scale 0.125, non-causal, null stream."""

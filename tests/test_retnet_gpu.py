@@ -1,0 +1,148 @@
+"""GPU parity of the RetNet forward and backward kernels against the CPU oracle, through the C ABI.
+
+Tolerance: |err| <= 2e-3 + 1e-3*|ref| against the fp32 oracle on the same seeded inputs.  The
+relative term matters only where outputs exceed ~4 in magnitude (gradients of rows whose normaliser
+is clamped at 1): there half a unit in the last place of the fp16 output itself is above 2e-3.
+"""
+import ctypes
+import os
+
+import pytest
+import torch
+
+import attention_autotuner_amd as aat
+from attention_autotuner_amd.arch import MI355X
+from attention_autotuner_amd.autotuner import RetBwdConfig, RetConfig, Runtime, codegen, gfx950_space, library
+from oracle import ref_op
+
+pytestmark = pytest.mark.gpu
+ARCH = MI355X()
+ATOL, RTOL = 2e-3, 1e-3
+
+
+def _inputs(b, h, sq, sk, dqk, dv, seed=0, dense_mask=False):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, h, sq, dqk, generator=g).half()
+    k = torch.randn(b, h, sk, dqk, generator=g).half()
+    v = torch.randn(b, h, sk, dv, generator=g).half()
+    do = torch.randn(b, h, sq, dv, generator=g).half()
+    if dense_mask:      # the reference's own runtime test uses a dense N(0,1) mask
+        mask = torch.randn(h, sq, sk, generator=g).half()
+    else:
+        mask = ref_op.retnet_decay_mask(h, sq, sk)
+    return q, k, v, mask, do
+
+
+def _close(got, ref):
+    got, ref = got.detach().float().cpu(), ref.float()
+    excess = ((got - ref).abs() - (ATOL + RTOL * ref.abs())).max().item()
+    return excess <= 0, excess
+
+
+def _run(q, k, v, mask, do, causal=False):
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = aat.RetNetAttnFunc(qc, kc, vc, mask.cuda(), ARCH, causal)
+    o.backward(do.cuda())
+    torch.cuda.synchronize()
+    return o, qc.grad, kc.grad, vc.grad
+
+
+@pytest.mark.parametrize("dqk,dv,dense", [(64, 64, True), (128, 128, False), (256, 256, True), (64, 128, False), (256, 512, False)])
+def test_forward_and_backward_match_the_oracle(dqk, dv, dense):
+    q, k, v, mask, do = _inputs(2, 2, 256, 256, dqk, dv, seed=dqk + dv, dense_mask=dense)
+    o, dq, dk, dv_ = _run(q, k, v, mask, do)
+    o_ref, r_ref = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    ok, ex = _close(o, o_ref)
+    assert ok, ("o", ex)
+    for name, got, want in zip(("dq", "dk", "dv"), (dq, dk, dv_), ref_op.retnet_bwd_ref(q, k, v, mask, do)):
+        ok, ex = _close(got, want)
+        assert ok, (name, ex)
+
+
+def test_config3_forward_b4_h8_s2048_dqk256_dv512_and_r():
+    q, k, v, mask, do = _inputs(4, 8, 2048, 2048, 256, 512, seed=3)
+    arrays = [t.cuda() for t in (q, k, v, mask)]
+    o = torch.empty(4, 8, 2048, 512, dtype=torch.float16, device="cuda")
+    r = torch.empty(4, 8, 2048, dtype=torch.float32, device="cuda")
+    cfg = gfx950_space.default_forward_config("ret", 256, 512, ARCH, 2048, 2048)
+    for causal in (False, True):            # the decay mask is lower-triangular: skipping tiles must not change anything
+        Runtime(ARCH, cfg).apply(arrays + [o, r], causal=causal)
+        for b, h in ((0, 0), (2, 5), (3, 7)):
+            o_ref, r_ref = ref_op.retnet_ref(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mask[h:h + 1], return_r=True)
+            ok, ex = _close(o[b:b + 1, h:h + 1], o_ref)
+            assert ok, (causal, b, h, ex)
+            rel = ((r[b, h].cpu() - r_ref[0, 0]).abs() / r_ref[0, 0]).max().item()
+            assert rel <= 1e-3, (causal, b, h, rel)
+    # size-independent properties on the whole problem
+    assert torch.isfinite(o.float()).all()
+    assert (r >= 1).all()
+
+
+def test_config4_forward_backward_b4_h8_s2048_dqk256_dv512():
+    q, k, v, mask, do = _inputs(4, 8, 2048, 2048, 256, 512, seed=4)
+    o, dq, dk, dv_ = _run(q, k, v, mask, do, causal=True)
+    for b, h in ((0, 0), (3, 7)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        want = ref_op.retnet_bwd_ref(q[sl], k[sl], v[sl], mask[h:h + 1], do[sl])
+        for name, got, w in zip(("dq", "dk", "dv"), (dq, dk, dv_), want):
+            ok, ex = _close(got[sl], w)
+            assert ok, (name, b, h, ex)
+    # linearity in dO on the whole problem: grad(2*dO) == 2*grad(dO) up to fp16 rounding of the outputs
+    o2, dq2, dk2, dv2 = _run(q, k, v, mask, (2 * do.float()).half(), causal=True)
+    for a, b2 in ((dq, dq2), (dk, dk2), (dv_, dv2)):
+        assert torch.equal((2 * a.float()).half(), b2)      # scaling by 2 is exact in fp16 and in every fp32 step
+    # a zero mask gives zero gradients and r == 1
+    zq, zk, zv = (t.cuda().requires_grad_(True) for t in (q[:1, :1], k[:1, :1], v[:1, :1]))
+    oz = aat.RetNetAttnFunc(zq, zk, zv, torch.zeros(1, 2048, 2048, dtype=torch.float16, device="cuda"), ARCH)
+    oz.backward(do[:1, :1].cuda())
+    assert oz.abs().max().item() == 0 and zq.grad.abs().max().item() == 0 and zk.grad.abs().max().item() == 0 and zv.grad.abs().max().item() == 0
+
+
+def test_clamp_active_reduces_to_plain_matmuls():
+    q, k, v, _, do = _inputs(1, 2, 128, 256, 64, 64, seed=5)
+    q = (q.float() * 1e-3).half()
+    mask = torch.ones(2, 128, 256).half()
+    o, dq, dk, dv_ = _run(q, k, v, mask, do)
+    want = (q.float() @ k.float().transpose(-1, -2)) @ v.float()
+    ok, ex = _close(o, want)
+    assert ok, ex
+
+
+def test_non_square_and_every_prebuilt_variant():
+    q, k, v, mask, do = _inputs(1, 2, 128, 384, 128, 128, seed=6, dense_mask=True)
+    o_ref = ref_op.retnet_ref(q, k, v, mask)
+    arrays = [t.cuda() for t in (q, k, v, mask)]
+    ran = 0
+    for fuse, extra in (("register", {}), ("shared", dict(warps_mma1_n=1, warps_mma_n=4)), ("shared", dict(warps_mma1_n=2, warps_mma_n=2))):
+        for st in ((1, 1), (2, 2)):
+            cfg = RetConfig(128 if fuse == "register" else 64, 64, 128, 128, 128, 64, st[0], st[0], st[1], 256, True, waves_per_eu=1, **extra)
+            cfg.fuse_type = fuse
+            if not gfx950_space.forward_valid(cfg, ARCH):
+                continue
+            o = torch.zeros(1, 2, 128, 128, dtype=torch.float16, device="cuda")
+            r = torch.zeros(1, 2, 128, dtype=torch.float32, device="cuda")
+            Runtime(ARCH, cfg).apply(arrays + [o, r])
+            ok, ex = _close(o, o_ref)
+            assert ok, (cfg, ex)
+            ran += 1
+    assert ran >= 4
+
+
+def test_reference_signature_entry_points_bwd():
+    q, k, v, mask, do = _inputs(1, 2, 128, 128, 64, 64, seed=7, dense_mask=True)
+    _, r_ref = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    dev = [t.cuda() for t in (q, k, v, mask, do)]
+    r = r_ref.cuda().contiguous()
+    dq, dk, dv_ = (torch.zeros_like(t) for t in dev[:3])
+    acc = torch.zeros(1, 2, 128, 64, dtype=torch.float32, device="cuda")
+    cfg = gfx950_space.default_backward_config(64, 64, ARCH, 128, 128)
+    lib = library.load(Runtime(ARCH, cfg)._path(), "ret_bwd")
+    ptrs = [ctypes.c_void_p(t.data_ptr()) for t in (*dev, r, dq, dk, dv_, acc)]
+    torch.cuda.synchronize()
+    assert lib.kernel_entry(*ptrs, 1, 2, 128, 128) == 0
+    torch.cuda.synchronize()
+    for got, want in zip((dq, dk, dv_), ref_op.retnet_bwd_ref(q, k, v, mask, do)):
+        ok, ex = _close(got, want)
+        assert ok, ex
+    assert acc.abs().max().item() == 0          # the scratch is never touched
+    assert lib.kernel_entry(*ptrs, 1, 2, 100, 128) == -2
