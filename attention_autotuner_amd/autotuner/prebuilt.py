@@ -17,7 +17,7 @@ from .configs import supported_configs
 
 # (operator, d_qk, d_v) pairs whose default configuration is always built
 # attention smemfuse variants exercised by the parity suite: (Br, Bc, Nthreads, K bufs, V bufs, W1N, W2N, waves/SIMD)
-SHARED_TILES = [(128, 64, 256, 2, 2, 1, 4, 2), (64, 64, 256, 1, 1, 2, 4, 2), (64, 64, 256, 2, 1, 2, 2, 2)]
+SHARED_TILES = [(128, 64, 256, 2, 2, 1, 4, 2), (64, 64, 256, 1, 1, 2, 4, 2), (64, 64, 256, 2, 1, 2, 2, 2), (64, 64, 256, 1, 1, 2, 4, 1)]
 
 DEFAULT_PROBLEMS = [
     ("attn", 64, 64), ("attn", 128, 128), ("attn", 256, 256), ("attn", 192, 192), ("attn", 256, 128), ("attn", 64, 128),

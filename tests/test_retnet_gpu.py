@@ -90,7 +90,8 @@ def test_config4_forward_backward_b4_h8_s2048_dqk256_dv512():
     # linearity in dO on the whole problem: grad(2*dO) == 2*grad(dO) up to fp16 rounding of the outputs
     o2, dq2, dk2, dv2 = _run(q, k, v, mask, (2 * do.float()).half(), causal=True)
     for a, b2 in ((dq, dq2), (dk, dk2), (dv_, dv2)):
-        assert torch.equal((2 * a.float()).half(), b2)      # scaling by 2 is exact in fp16 and in every fp32 step
+        ok, ex = _close(b2, 2 * a.float().cpu())             # exact except where fp16 dS is subnormal
+        assert ok, ex
     # a zero mask gives zero gradients and r == 1
     zq, zk, zv = (t.cuda().requires_grad_(True) for t in (q[:1, :1], k[:1, :1], v[:1, :1]))
     oz = aat.RetNetAttnFunc(zq, zk, zv, torch.zeros(1, 2048, 2048, dtype=torch.float16, device="cuda"), ARCH)
@@ -99,12 +100,16 @@ def test_config4_forward_backward_b4_h8_s2048_dqk256_dv512():
 
 
 def test_clamp_active_reduces_to_plain_matmuls():
-    q, k, v, _, do = _inputs(1, 2, 128, 256, 64, 64, seed=5)
-    q = (q.float() * 1e-3).half()
-    mask = torch.ones(2, 128, 256).half()
+    q, k, v, _, do = _inputs(1, 2, 128, 64, 64, 64, seed=5)
+    q, k = (q.float() * 0.02).half(), (k.float() * 0.02).half()
+    mask = torch.ones(2, 128, 64).half()
+    _, r_ref = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    assert (r_ref == 1).all()                                # every row sum of |S| stays below 1
     o, dq, dk, dv_ = _run(q, k, v, mask, do)
     want = (q.float() @ k.float().transpose(-1, -2)) @ v.float()
     ok, ex = _close(o, want)
+    assert ok, ex
+    ok, ex = _close(dv_, (q.float() @ k.float().transpose(-1, -2)).transpose(-1, -2) @ do.float())
     assert ok, ex
 
 
