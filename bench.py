@@ -91,6 +91,16 @@ def cpu_baseline(heads=8):
             "cpu_model": model, "os_cpu_count": os.cpu_count()}
 
 
+def measured_traffic(cfg):
+    """HBM bytes per launch measured with rocprofv3 (FETCH_SIZE + WRITE_SIZE, each scaled by a plain
+    copy of known size) for this kernel configuration, if a profile of it has been recorded."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f).get(str(cfg), {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,6 +108,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the causal / long-kv / RetNet side measurements")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run plain 256 MiB device copies, so a profiler's HBM byte counters can be scaled by a known transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py measures one GPU: the path has no cross-GPU component (batch x head slices are independent); run with --gpus 1")
@@ -120,6 +132,14 @@ def main():
     q, k, v = mk(B, H, S, D), mk(B, H, S, D), mk(B, H, S, D)
     o = torch.empty(B, H, S, D, dtype=torch.float16, device=dev)
     scale = 1.0 / math.sqrt(D)
+
+    if args.copy_calibration:
+        src = torch.empty(128 * 1024 * 1024, dtype=torch.float16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)                      # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     cfg = resolve_config(aat, arch, [q, k, v, o], False)
     rt = Runtime(arch, cfg)
@@ -145,7 +165,7 @@ def main():
         "config": {"workload": "configs[1]: flash-attention forward q,k,v [4,32,2048,128] fp16 N(0,1), scale 1/sqrt(128), non-causal",
                    "kernel_config": str(cfg), "pct_of_fp16_mfma_peak": round(100 * value / PEAK_TFLOPS, 2)},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": measured_traffic(cfg),
                      "kernel": "flashattn_fwd_" + ("regfuse" if cfg.fuse_type == "register" else "smemfuse"),
                      "launch_ms": round(kern_ms, 5), "algorithmic_flops_per_launch": flops},
         "extras": extras,
