@@ -113,7 +113,8 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
             for wpe in (1, 2, 3):
                 for fuse in fuse_types:
                     if fuse == "shared":
-                        out.extend(_shared_candidates(op, br, bc, dim_qk, dim_v, st_qk, st_v, nthreads, wpe))
+                        if st_qk == st_v and wpe <= 2:   # the LDS-fused kernels gain little from mixed buffering
+                            out.extend(_shared_candidates(op, br, bc, dim_qk, dim_v, st_qk, st_v, nthreads, wpe))
                         continue
                     if op == "attn":
                         cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, waves_per_eu=wpe)

@@ -1,0 +1,94 @@
+"""Tune one problem and record the result (counterpart of the reference's tuner drivers,
+python/tests/attntuner_demo.py:186-192 and python/tests/test_retbwdtunner.py:88-92).
+
+    python -m attention_autotuner_amd.benchmarks.tune attn    B H Sq Sk dqk dv [--causal] [--compile-only]
+    python -m attention_autotuner_amd.benchmarks.tune ret     B H Sq Sk dqk dv [--causal]
+    python -m attention_autotuner_amd.benchmarks.tune ret_bwd B H Sq Sk dqk dv [--causal]
+
+Writes the best configuration into the tuning cache, the per-candidate log next to it, and prints a
+one-line JSON summary.  ``--compile-only`` builds every candidate library (no GPU needed) so that a
+later run on a machine without spare CPU time only has to time them.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+from ..arch import MI355X
+from ..autotuner import AttnTunner, RetBwdTunner, RetTunner, codegen
+from ..ops._resolve import DEFAULT_LOG_DIR
+
+
+def make_tensors(op, b, h, sq, sk, dqk, dv, device, seed=0):
+    g = torch.Generator().manual_seed(seed)
+
+    def mk(*shape):
+        t = torch.randn(*shape, generator=g).half()
+        return t.to(device)
+
+    if device == "meta":
+        def mk(*shape):                                        # noqa: F811 - shapes only
+            return torch.empty(*shape, dtype=torch.float16, device="meta")
+    q, k, v = mk(b, h, sq, dqk), mk(b, h, sk, dqk), mk(b, h, sk, dv)
+    if op == "attn":
+        return [q, k, v, torch.empty(b, h, sq, dv, dtype=torch.float16, device=device)]
+    n = torch.arange(sq, dtype=torch.float64).view(1, sq, 1)
+    m = torch.arange(sk, dtype=torch.float64).view(1, 1, sk)
+    gamma = (1.0 - torch.pow(2.0, -5.0 - torch.arange(h, dtype=torch.float64))).view(h, 1, 1)
+    mask = torch.where(n + (sk - sq) >= m, gamma ** (n + (sk - sq) - m).clamp(min=0), torch.zeros((), dtype=torch.float64))
+    mask = mask.float().half().to(device) if device != "meta" else torch.empty(h, sq, sk, dtype=torch.float16, device="meta")
+    o = torch.empty(b, h, sq, dv, dtype=torch.float16, device=device)
+    r = torch.ones(b, h, sq, dtype=torch.float32, device=device) if device != "meta" else torch.empty(b, h, sq, device="meta")
+    if op == "ret":
+        return [q, k, v, mask, o, r]
+    do = mk(b, h, sq, dv)
+    if device != "meta":
+        r.fill_(50.0)
+    dq, dk, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    acc = torch.zeros(1, dtype=torch.float32, device=device) if device != "meta" else torch.empty(1, device="meta")
+    return [q, k, v, mask, do, r, dq, dk, dv_, acc]
+
+
+def flops(op, b, h, sq, sk, dqk, dv, causal):
+    f = 2.0 * b * h * sq * sk * ((dqk + dv) if op != "ret_bwd" else (3 * dqk + 2 * dv))
+    return f / 2 if (causal and op == "attn") else f
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("op", choices=["attn", "ret", "ret_bwd"])
+    ap.add_argument("dims", type=int, nargs=6, metavar=("B", "H", "Sq", "Sk", "dqk", "dv"))
+    ap.add_argument("--causal", action="store_true")
+    ap.add_argument("--compile-only", action="store_true")
+    ap.add_argument("--log-dir", default=DEFAULT_LOG_DIR)
+    args = ap.parse_args(argv)
+    b, h, sq, sk, dqk, dv = args.dims
+    arch = MI355X()
+    cls = {"attn": AttnTunner, "ret": RetTunner, "ret_bwd": RetBwdTunner}[args.op]
+    device = "meta" if args.compile_only else "cuda"
+    arrays = make_tensors(args.op, b, h, sq, sk, dqk, dv, device)
+    tuner = cls(arch, arrays, causal=args.causal)
+    if args.compile_only:
+        cfgs = [c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)]
+        t0 = time.time()
+        libs = codegen.compile_parallel(cfgs, arch, timeout=300)
+        print(json.dumps({"op": args.op, "candidates": len(cfgs), "built": sum(l is not None for l in libs),
+                          "seconds": round(time.time() - t0, 1)}))
+        return 0
+    log_dir = os.path.join(args.log_dir, f"{args.op}_b{b}h{h}q{sq}k{sk}_c{int(args.causal)}")
+    best = tuner.tune(log_path=log_dir, use_cache=False)
+    ms = tuner.last_timings[best]
+    ok = [t for t in tuner.last_timings.values() if t < 1e7]
+    print(json.dumps({"op": args.op, "problem": args.dims, "causal": args.causal, "best": str(best), "ms": round(ms, 5),
+                      "tflops": round(flops(args.op, b, h, sq, sk, dqk, dv, args.causal) / ms / 1e9, 1),
+                      "candidates": len(tuner.last_timings), "ran": len(ok), "worst_ms": round(max(ok), 4),
+                      "cache": tuner._cache_file(), "log": log_dir}))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
