@@ -79,6 +79,9 @@ class BaseTunner:
 
     def _fits_problem(self, config):
         s = self.problem_shape
+        ns = getattr(config, "kv_splits", 1)
+        if ns > 1 and (s["Sk"] // config.Bc) % ns:
+            return False
         if config.operation == "ret_bwd":             # both lengths are resident in one pass, streamed in another
             return all(s[n] % config.Br == 0 and s[n] % config.Bc == 0 for n in ("Sq", "Sk"))
         return s["Sq"] % config.Br == 0 and s["Sk"] % config.Bc == 0

@@ -106,7 +106,10 @@ def forward_valid(cfg, arch):
     return forward_reg_estimate(cfg) <= arch.register_per_thread // cfg.waves_per_eu
 
 
-def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "shared")):
+KV_SPLITS = (2, 4, 8, 16)
+
+
+def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "shared"), with_splits=False):
     out = []
     for nthreads in THREADS:
         for st_qk, st_v in STAGES:
@@ -124,6 +127,10 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
                     if op == "attn" and fuse == "register" and (st_qk, st_v) == (2, 2):
                         piped = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 2, 2, nthreads, True, waves_per_eu=wpe, sw_pipeline=1)
                         out.append(piped.set_fuse_type(fuse))
+                    if op == "attn" and fuse == "register" and with_splits and st_qk == st_v:
+                        for ns in KV_SPLITS:   # long kv, few query rows: cut the kv range so every CU gets work
+                            sp = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, waves_per_eu=wpe, kv_splits=ns)
+                            out.append(sp.set_fuse_type(fuse))
     return out
 
 

@@ -59,6 +59,8 @@ def extra_configs(arch=None):
                 piped = AttnConfig(br, bc, dqk, dv, dqk, bc, 2, 2, nt, True, waves_per_eu=wpe, sw_pipeline=1).set_fuse_type("register")
                 if gfx950_space.forward_valid(piped, arch):
                     out.append(piped)
+    for dqk, dv, ns in ((128, 128, 4), (128, 128, 8), (64, 64, 2)):     # kv-splitting variants
+        out.append(AttnConfig(128, 64, dqk, dv, dqk, 64, 2, 2, 256, True, waves_per_eu=2, kv_splits=ns).set_fuse_type("register"))
     for dqk, dv in ((64, 64), (128, 128), (256, 512)):
         for br, bc, nt, sq, sv, w1n, w2n, wpe in SHARED_TILES:
             cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, w1n, w2n, waves_per_eu=wpe)
@@ -117,5 +119,20 @@ def build_all(arch=None, force=True, timeout=600, verbose=True):
     return libs
 
 
+def prune_stale(build_dir=None):
+    """Delete libraries (and their sources / logs) built from an older revision of the kernel sources."""
+    root = build_dir or codegen.DEFAULT_BUILD_DIR
+    keep = "-" + codegen.source_digest() + "."
+    removed = 0
+    for dirpath, _, files in os.walk(root):
+        for fn in files:
+            if fn.endswith((".so", ".hip", ".log")) and keep not in fn:
+                os.remove(os.path.join(dirpath, fn))
+                removed += 1
+    return removed
+
+
 if __name__ == "__main__":
+    if "--prune" in sys.argv:
+        print("removed", prune_stale(), "stale files")
     build_all(force="--force" in sys.argv)

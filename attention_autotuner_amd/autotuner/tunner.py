@@ -23,8 +23,15 @@ class _ForwardTunner(BaseTunner):
             self.Bc_list = list(gfx950_space.BC_LIST)
 
     def generate_configs(self, Br, Bc, dim_qk, dim_v):
-        space = gfx950_space if _is_rocm(self.arch) else legacy_space
-        return space.forward_candidates(self.operation, Br, Bc, dim_qk, dim_v)
+        if not _is_rocm(self.arch):
+            return legacy_space.forward_candidates(self.operation, Br, Bc, dim_qk, dim_v)
+        return gfx950_space.forward_candidates(self.operation, Br, Bc, dim_qk, dim_v, with_splits=self._wants_splits(Br))
+
+    def _wants_splits(self, Br):
+        """kv splitting is worth trying when the row blocks alone cannot occupy the chip."""
+        s = self.problem_shape
+        blocks = s["B"] * s["H"] * max(1, s["Sq"] // Br)
+        return self.operation == "attn" and not self.causal and blocks < 2 * self.arch.compute_max_core
 
     def _validate(self, config):
         space = gfx950_space if _is_rocm(self.arch) else legacy_space

@@ -20,6 +20,7 @@ constexpr int Nthreads = {Nthreads};
 constexpr int num_stages_qk = {num_stages_qk};   // LDS buffers for the K tile
 constexpr int num_stages_v = {num_stages_v};     // LDS buffers for the V tile
 constexpr int waves_per_eu = {waves_per_eu};
+constexpr int kv_splits = {kv_splits};           // > 1: the kv range is cut into that many parts (non-causal only)
 constexpr bool sw_pipeline = {sw_pipeline};      // next tile's QK^T MFMAs interleaved with this tile's exponentials
 constexpr float kReferenceScale = 0.125f;        // what the reference kernels hard-code
 
@@ -27,9 +28,30 @@ using Traits = aat::AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_s
 constexpr int shared_mem = Traits::kSmemBytes;
 const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, false>;
 const auto kernel_causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, true>;
+const auto kernel_split = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, false, true>;
+constexpr int shared_mem_split = Traits::kSmemBytesSplit;
+
+size_t split_workspace_bytes(int B, int H, int Seq_q) {{
+  return kv_splits > 1 ? (size_t)kv_splits * B * H * Seq_q * (D + 1) * sizeof(float) : 0;
+}}
+bool split_applies(int Seq_k, int causal) {{ return kv_splits > 1 && !causal && (Seq_k / Bc) % kv_splits == 0; }}
 
 hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k,
-                  float softmax_scale, int causal, hipStream_t stream) {{
+                  float softmax_scale, int causal, void* workspace, hipStream_t stream) {{
+  if (split_applies(Seq_k, causal) && workspace != nullptr) {{
+    static const hipError_t lds_ok_split = aat::allow_lds(kernel_split, shared_mem_split);
+    if (lds_ok_split != hipSuccess) return lds_ok_split;
+    const size_t rows = (size_t)B * H * Seq_q;
+    float* part_o = static_cast<float*>(workspace);
+    float* part_lse = part_o + (size_t)kv_splits * rows * D;
+    kernel_split<<<dim3(B * H * (Seq_q / Br), kv_splits), dim3(Nthreads), shared_mem_split, stream>>>(
+        reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
+        reinterpret_cast<const aat::half_t*>(v), nullptr, nullptr, H, Seq_k, Seq_q, softmax_scale, part_o, part_lse);
+    const size_t threads = rows * (D / 8);
+    aat::attn_split_merge<D><<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream>>>(
+        part_o, part_lse, reinterpret_cast<aat::half_t*>(o), nullptr, (int)rows, kv_splits);
+    return hipGetLastError();
+  }}
   static const hipError_t lds_ok = aat::allow_lds(kernel, shared_mem);
   static const hipError_t lds_ok_causal = aat::allow_lds(kernel_causal, shared_mem);
   if (lds_ok != hipSuccess) return lds_ok;
@@ -37,36 +59,42 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int
   (causal ? kernel_causal : kernel)<<<dim3(B * H * (Seq_q / Br)), dim3(Nthreads), shared_mem, stream>>>(
       reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
       reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<aat::half_t*>(o), nullptr, H, Seq_k, Seq_q,
-      softmax_scale);
+      softmax_scale, nullptr, nullptr);
   return hipGetLastError();
 }}
 }}  // namespace
 
 extern "C" int abi_version(void) {{ return AAT_ABI_VERSION; }}
 extern "C" const char* config_string(void) {{ return "{config_name}"; }}
-extern "C" size_t workspace_size(int, int, int, int) {{ return 0; }}
+extern "C" size_t workspace_size(int B, int H, int Seq_q, int) {{ return split_workspace_bytes(B, H, Seq_q); }}
 """
 
 profile_func = r"""
 extern "C" float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k,
-                            float softmax_scale, int causal, void*, size_t, void* stream) {{
+                            float softmax_scale, int causal, void* workspace, size_t workspace_bytes, void* stream) {{
   if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return -1.f;
+  if (split_applies(Seq_k, causal) && (workspace == nullptr || workspace_bytes < split_workspace_bytes(B, H, Seq_q))) return -1.f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return aat::timed_mean_ms(s, [&] {{ return launch(q, k, v, o, B, H, Seq_q, Seq_k, softmax_scale, causal, s); }});
+  return aat::timed_mean_ms(s, [&] {{ return launch(q, k, v, o, B, H, Seq_q, Seq_k, softmax_scale, causal, workspace, s); }});
 }}
+// The reference signature has no workspace argument: a kv-splitting configuration runs unsplit here.
 extern "C" float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k) {{
-  return profile_ex(q, k, v, o, B, H, Seq_q, Seq_k, kReferenceScale, 0, nullptr, 0, nullptr);
+  if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return -1.f;
+  return aat::timed_mean_ms(nullptr, [&] {{ return launch(q, k, v, o, B, H, Seq_q, Seq_k, kReferenceScale, 0, nullptr, nullptr); }});
 }}
 """
 
 kernel_entry = r"""
 extern "C" int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k,
-                               float softmax_scale, int causal, void*, size_t, void* stream) {{
+                               float softmax_scale, int causal, void* workspace, size_t workspace_bytes, void* stream) {{
   if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return AAT_ERR_SHAPE;
-  return (int)launch(q, k, v, o, B, H, Seq_q, Seq_k, softmax_scale, causal, static_cast<hipStream_t>(stream));
+  if (split_applies(Seq_k, causal) && (workspace == nullptr || workspace_bytes < split_workspace_bytes(B, H, Seq_q)))
+    return AAT_ERR_WORKSPACE;
+  return (int)launch(q, k, v, o, B, H, Seq_q, Seq_k, softmax_scale, causal, workspace, static_cast<hipStream_t>(stream));
 }}
 extern "C" int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_k, int Seq_q) {{
-  return kernel_entry_ex(q, k, v, o, B, H, Seq_q, Seq_k, kReferenceScale, 0, nullptr, 0, nullptr);
+  if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return AAT_ERR_SHAPE;
+  return (int)launch(q, k, v, o, B, H, Seq_q, Seq_k, kReferenceScale, 0, nullptr, nullptr);
 }}
 """
 

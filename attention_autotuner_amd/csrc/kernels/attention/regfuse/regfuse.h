@@ -48,9 +48,12 @@ struct AttnFwdRegfuse {
   static constexpr int kKBytes = Bc * Kd * 2, kVBytes = Bc * D * 2;
   static constexpr int kUnitK = 32 * Kd * 2, kUnitV = 32 * D * 2;   // bytes of one 32-row unit
   static constexpr int kOStride = D * 2 + 16;   // epilogue staging row stride (bytes)
+  static constexpr int kOStride32 = D * 4 + 16; // same, for the fp32 partial outputs of a kv split
   static constexpr int kMainBytes = NSK * kKBytes + NSV * kVBytes;
   static constexpr int kEpiBytes = Br * kOStride;
   static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
+  static constexpr int kEpiBytesSplit = Br * kOStride32;
+  static constexpr int kSmemBytesSplit = kMainBytes > kEpiBytesSplit ? kMainBytes : kEpiBytesSplit;
   // The pipelined schedule copies K in whole 32-row units.
   static constexpr bool kPipeOk = NSK == 2 && NSV == 2 && KDma::kRegular && KDma::kRowsPerIter <= 32 &&
                                   32 % KDma::kRowsPerIter == 0;
@@ -80,16 +83,23 @@ template <bool CAUSAL, class F> AAT_DEV void run_tiles(F& tile, int n_full, int 
 // PIPE selects the software-pipelined schedule (needs two K and two V buffers).  CAUSAL is a
 // compile-time switch so that the non-causal kernel carries no masking code at all; in the causal
 // kernel the tiles the diagonal cannot touch still run the unmasked tile body.
+//
+// SPLIT: the kv range is cut into gridDim.y equal parts (few query rows, long kv: not enough row
+// blocks to fill the chip).  Part s handles kv tiles [s, s+1) * n_tiles / parts and writes its own
+// normalised output (fp32) and log-sum-exp to part_o / part_lse, laid out [part][B*H*S_q][D] and
+// [part][B*H*S_q]; attn_split_merge combines them.  o and lse are not touched.
 template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int WPE = 1, bool PIPE = false,
-          bool CAUSAL = false>
+          bool CAUSAL = false, bool SPLIT = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k,
                       const half_t* __restrict__ v, half_t* __restrict__ o, float* __restrict__ lse,
-                      int H, int seq_k, int seq_q, float softmax_scale) {
+                      int H, int seq_k, int seq_q, float softmax_scale, float* __restrict__ part_o = nullptr,
+                      float* __restrict__ part_lse = nullptr) {
   using T = AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, WM = T::WM;
   constexpr int PF = AAT_PF;                     // operand prefetch distance, in MFMA steps
   static_assert(!PIPE || T::kPipeOk, "the pipelined schedule needs 2+2 buffers and unit-aligned K copies");
+  static_assert(!(SPLIT && CAUSAL), "kv splitting is for non-causal problems");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 #ifdef AAT_CLOCK_PROBE
   const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
@@ -120,8 +130,15 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     n_full &= ~1;                               // keep the masked loop on an even tile: buffer parity 0
   }
 
-  const char* kg = reinterpret_cast<const char*>(k + (size_t)bh * seq_k * Kd);
-  const char* vg = reinterpret_cast<const char*>(v + (size_t)bh * seq_k * D);
+  int tile0 = 0;                                // first kv tile of this block's range
+  if constexpr (SPLIT) {
+    const int per = n_tiles / (int)gridDim.y;   // the launcher guarantees divisibility
+    tile0 = (int)blockIdx.y * per;
+    n_tiles = per;
+    n_full = per;
+  }
+  const char* kg = reinterpret_cast<const char*>(k + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * Kd);
+  const char* vg = reinterpret_cast<const char*>(v + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * D);
 
   typename T::KDma kdma;
   typename T::VDma vdma;
@@ -285,19 +302,69 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   for (int rt = 0; rt < RT; ++rt) {
     const float l_tot = pair_sum(l_run[rt]);
     inv[rt] = l_tot > 0.f ? fast_rcp(l_tot) : 0.f;
-    if (lse != nullptr && h == 0) {
-      const size_t row = (size_t)bh * seq_q + q0 + wave * WM + rt * 32 + n;
-      lse[row] = l_tot > 0.f ? m_run[rt] * softmax_scale + __logf(l_tot) : -INFINITY;
+    const size_t row = (size_t)bh * seq_q + q0 + wave * WM + rt * 32 + n;
+    const float row_lse = l_tot > 0.f ? m_run[rt] * softmax_scale + __logf(l_tot) : -INFINITY;
+    if constexpr (SPLIT) {
+      if (h == 0) part_lse[(size_t)blockIdx.y * gridDim.x * Br + row] = row_lse;   // gridDim.x * Br = B*H*S_q
+    } else {
+      if (lse != nullptr && h == 0) lse[row] = row_lse;
     }
   }
-  store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + wave * WM * T::kOStride,
-                                       o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+  if constexpr (SPLIT) {
+    const size_t rows_total = (size_t)gridDim.x * Br;
+    store_o_tile<RT, DT, D, T::kOStride32, float>(
+        oacc, inv, smem + wave * WM * T::kOStride32,
+        part_o + ((size_t)blockIdx.y * rows_total + (size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+  } else {
+    store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + wave * WM * T::kOStride,
+                                         o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+  }
 #ifdef AAT_CLOCK_PROBE
   if (lse != nullptr && tid == 0 && (blockIdx.x % 64) == 0) {
     lse[2 * (blockIdx.x / 64)] = (float)(clock64() - probe_c0);
     lse[2 * (blockIdx.x / 64) + 1] = (float)(wall_clock64() - probe_w0);
   }
 #endif
+}
+
+// Combine the parts of a kv split: O = sum_s exp(lse_s - lse) O_s with lse = log sum_s exp(lse_s).
+// One thread per (row, 8 output columns); HBM-bound.
+template <int D>
+__global__ void __launch_bounds__(256)
+attn_split_merge(const float* __restrict__ part_o, const float* __restrict__ part_lse, half_t* __restrict__ o,
+                 float* __restrict__ lse, int rows, int parts) {
+  constexpr int kChunks = D / 8;
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)rows * kChunks) return;
+  const size_t row = idx / kChunks;
+  const int c = (int)(idx % kChunks);
+  float m = -INFINITY;
+  for (int s = 0; s < parts; ++s) m = fmaxf(m, part_lse[(size_t)s * rows + row]);
+  const float m_use = (m == -INFINITY) ? 0.f : m;
+  float wsum = 0.f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int s = 0; s < parts; ++s) {
+    const float w = __expf(part_lse[(size_t)s * rows + row] - m_use);
+    wsum += w;
+    const f4v a = *reinterpret_cast<const f4v*>(part_o + ((size_t)s * rows + row) * D + c * 8);
+    const f4v b = *reinterpret_cast<const f4v*>(part_o + ((size_t)s * rows + row) * D + c * 8 + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc[e] += w * a[e];
+      acc[4 + e] += w * b[e];
+    }
+  }
+  const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+  h8 out;
+#pragma unroll
+  for (int e = 0; e < 8; e += 2) {
+    const h2 pr = pack_rne(acc[e] * inv, acc[e + 1] * inv);
+    out[e] = pr[0];
+    out[e + 1] = pr[1];
+  }
+  *reinterpret_cast<h8*>(o + row * D + c * 8) = out;
+  if (lse != nullptr && c == 0) lse[row] = wsum > 0.f ? m_use + __logf(wsum) : -INFINITY;
 }
 
 }  // namespace aat

@@ -167,13 +167,14 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
   }
 }
 
-// Epilogue: scale the wave's O^T accumulators per row, round to fp16 (RNE), transpose through a
-// wave-private LDS staging area and store rows with 16-byte coalesced writes.
+// Epilogue: scale the wave's O^T accumulators per row, convert (fp16 with RNE, or fp32 as is),
+// transpose through a wave-private LDS staging area and store rows with 16-byte coalesced writes.
 // ostage: wave-private LDS, WM rows of O_STRIDE bytes.  og: global pointer to the wave's first output row.
-template <int RT, int DT, int D, int O_STRIDE>
-AAT_DEV void store_o_tile(const f16v (&oacc)[RT][DT], const float (&row_scale)[RT], char* ostage, half_t* og,
+template <int RT, int DT, int D, int O_STRIDE, class OutT = half_t>
+AAT_DEV void store_o_tile(const f16v (&oacc)[RT][DT], const float (&row_scale)[RT], char* ostage, OutT* og,
                           int lane) {
-  constexpr int NCV = D / 8, WM = RT * 32;
+  constexpr int kElem = (int)sizeof(OutT);
+  constexpr int kChunksPerRow = D * kElem / 16, WM = RT * 32;
   const int n = lane & 31, h = lane >> 5;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
@@ -182,23 +183,31 @@ AAT_DEV void store_o_tile(const f16v (&oacc)[RT][DT], const float (&row_scale)[R
     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const h2 a = pack_rne(oacc[rt][dt][4 * g] * sc, oacc[rt][dt][4 * g + 1] * sc);
-        const h2 b = pack_rne(oacc[rt][dt][4 * g + 2] * sc, oacc[rt][dt][4 * g + 3] * sc);
-        h4 w;
-        w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
         const int d0 = 32 * dt + 8 * g + 4 * h;
-        *reinterpret_cast<h4*>(ostage + (rt * 32 + n) * O_STRIDE + d0 * 2) = w;
+        char* dst = ostage + (rt * 32 + n) * O_STRIDE + d0 * kElem;
+        if constexpr (kElem == 2) {
+          const h2 a = pack_rne(oacc[rt][dt][4 * g] * sc, oacc[rt][dt][4 * g + 1] * sc);
+          const h2 b = pack_rne(oacc[rt][dt][4 * g + 2] * sc, oacc[rt][dt][4 * g + 3] * sc);
+          h4 w;
+          w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
+          *reinterpret_cast<h4*>(dst) = w;
+        } else {
+          f4v w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = oacc[rt][dt][4 * g + e] * sc;
+          *reinterpret_cast<f4v*>(dst) = w;
+        }
       }
     }
   }
   wait_lgkm0();                                   // the staging region is private to this wave
-  constexpr int kChunks = WM * NCV;
+  constexpr int kChunks = WM * kChunksPerRow;
 #pragma unroll
   for (int t = 0; t < kChunks / 64; ++t) {
     const int idx = t * 64 + lane;
-    const int row = idx / NCV, c = idx % NCV;
+    const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
     const u4v val = *reinterpret_cast<const u4v*>(ostage + row * O_STRIDE + c * 16);
-    *reinterpret_cast<u4v*>(reinterpret_cast<char*>(og) + ((size_t)row * NCV + c) * 16) = val;
+    *reinterpret_cast<u4v*>(reinterpret_cast<char*>(og) + ((size_t)row * kChunksPerRow + c) * 16) = val;
   }
 }
 

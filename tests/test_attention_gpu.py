@@ -131,6 +131,35 @@ def test_lds_fused_variants_agree_with_the_oracle(dqk, dv):
     assert ran >= 1
 
 
+@pytest.mark.parametrize("dqk,ns,sk", [(128, 4, 1024), (128, 8, 16384), (64, 2, 512)])
+def test_kv_split_matches_the_oracle_and_the_unsplit_kernel(dqk, ns, sk):
+    q, k, v = _inputs(1, 4, 256, sk, dqk, dqk, seed=9)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    cfg = AttnConfig(128, 64, dqk, dqk, dqk, 64, 2, 2, 256, True, waves_per_eu=2, kv_splits=ns).set_fuse_type("register")
+    assert os.path.exists(codegen.library_path(cfg))
+    rt = Runtime(ARCH, cfg)
+    need = rt.workspace_size(1, 4, 256, sk)
+    assert need == ns * 4 * 256 * (dqk + 1) * 4
+    o = torch.zeros(1, 4, 256, dqk, dtype=torch.float16, device="cuda")
+    rt.apply([qc, kc, vc, o])                                   # Runtime allocates the workspace it was asked for
+    assert _err(o, ref_op.attention_ref(q, k, v)) <= TOL
+    unsplit = AttnConfig(128, 64, dqk, dqk, dqk, 64, 2, 2, 256, True, waves_per_eu=2).set_fuse_type("register")
+    o1 = torch.zeros_like(o)
+    Runtime(ARCH, unsplit).apply([qc, kc, vc, o1])
+    assert (o.float() - o1.float()).abs().max().item() <= 1e-3
+    # a causal call on a splitting configuration runs the unsplit causal kernel
+    if sk == 512:
+        q2, k2, v2 = _inputs(1, 4, 512, 512, dqk, dqk, seed=10)
+        o2 = torch.zeros(1, 4, 512, dqk, dtype=torch.float16, device="cuda")
+        rt.apply([q2.cuda(), k2.cuda(), v2.cuda(), o2], causal=True)
+        assert _err(o2, ref_op.attention_ref(q2, k2, v2, None, True)) <= TOL
+    # without a workspace the extended entry point refuses; the reference-signature one runs unsplit
+    lib = library.load(rt._path(), "attn")
+    ptrs = [ctypes.c_void_p(t.data_ptr()) for t in (qc, kc, vc, o)]
+    rc = lib.kernel_entry_ex(*ptrs, 1, 4, 256, sk, ctypes.c_float(0.1), 0, None, 0, None)
+    assert rc == -3
+
+
 def test_reference_signature_entry_points():
     """profile / kernel_entry keep the reference's argument order (kernel_entry swaps the lengths)
     and its literal behaviour: scale 0.125, non-causal, null stream."""
