@@ -1,0 +1,135 @@
+// Stand-alone attention-forward benchmark for MI355X: times hand-picked kernel configurations without
+// Python (counterpart of reference benchmarks/attention.cu:34-308 and benchmarks/configs.h).
+//
+//   hipcc --offload-arch=gfx950 -O3 -fno-math-errno -ffp-contract=fast -fno-honor-nans \
+//         -Xclang -target-feature -Xclang -packed-fp32-ops -I attention_autotuner_amd/csrc \
+//         attention_autotuner_amd/csrc/benchmarks/attention.hip -o attention_bench
+//   ./attention_bench [B H Sq Sk] [--causal] [--no-flush]
+//
+// Inputs are N(0,1) fp16 (Box-Muller on the host from a fixed seed).  Prints mean / median / p20 / p80
+// milliseconds and TFLOP/s (2*B*H*Sq*Sk*(d_qk+d_v), halved when causal) per configuration.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "../kernels/attention/regfuse/regfuse.h"
+#include "../kernels/attention/smemfuse/smemfuse.h"
+#include "do_bench.h"
+
+#define HIP_OK(x)                                                                     \
+  do {                                                                                \
+    hipError_t e_ = (x);                                                              \
+    if (e_ != hipSuccess) {                                                           \
+      std::printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+      std::exit(1);                                                                   \
+    }                                                                                 \
+  } while (0)
+
+struct ProblemShape {
+  int B, H, Sq, Sk;
+  bool causal, flush;
+};
+
+static aat::half_t* device_randn(size_t n, unsigned seed) {
+  std::vector<aat::half_t> h(n);
+  std::mt19937 gen(seed);
+  std::normal_distribution<float> dist(0.f, 1.f);
+  for (auto& x : h) x = (aat::half_t)dist(gen);
+  aat::half_t* d = nullptr;
+  HIP_OK(hipMalloc(&d, n * sizeof(aat::half_t)));
+  HIP_OK(hipMemcpy(d, h.data(), n * sizeof(aat::half_t), hipMemcpyHostToDevice));
+  return d;
+}
+
+struct Buffers {
+  aat::half_t *q, *k, *v, *o;
+};
+
+template <int Kd, int D>
+static Buffers make_buffers(const ProblemShape& ps) {
+  Buffers b;
+  b.q = device_randn((size_t)ps.B * ps.H * ps.Sq * Kd, 1);
+  b.k = device_randn((size_t)ps.B * ps.H * ps.Sk * Kd, 2);
+  b.v = device_randn((size_t)ps.B * ps.H * ps.Sk * D, 3);
+  HIP_OK(hipMalloc(&b.o, (size_t)ps.B * ps.H * ps.Sq * D * sizeof(aat::half_t)));
+  return b;
+}
+
+static void report(const char* what, const ProblemShape& ps, int Kd, int D, const aat_bench::Timing& t) {
+  double fl = 2.0 * ps.B * ps.H * (double)ps.Sq * ps.Sk * (Kd + D) * (ps.causal ? 0.5 : 1.0);
+  std::printf("%-64s mean %.4f ms  median %.4f  p20 %.4f  p80 %.4f  (%d launches)  %.1f TFLOP/s = %.1f%% of 2.5 PFLOP/s\n", what,
+              t.mean_ms, t.median_ms, t.p20_ms, t.p80_ms, t.launches, fl / t.median_ms * 1e-9, fl / t.median_ms * 1e-9 / 25.0);
+}
+
+// Register-fused configuration: <Kd, D, Br, Bc, Nthreads, K buffers, V buffers, waves per SIMD, pipelined>
+template <int Kd, int D, int Br, int Bc, int NT, int NSK, int NSV, int WPE, bool PIPE>
+static void test_regfuse_attention(const ProblemShape& ps, const Buffers& b) {
+  using T = aat::AttnFwdRegfuse<Kd, D, Br, Bc, NT, NSK, NSV>;
+  if (ps.Sq % Br || ps.Sk % Bc) return;
+  auto plain = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, PIPE, false>;
+  auto causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, PIPE, true>;
+  HIP_OK(hipFuncSetAttribute((const void*)plain, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
+  HIP_OK(hipFuncSetAttribute((const void*)causal, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
+  const float scale = 1.f / std::sqrt((float)Kd);
+  auto t = aat_bench::do_bench([&] {
+    (ps.causal ? causal : plain)<<<dim3(ps.B * ps.H * ps.Sq / Br), dim3(NT), T::kSmemBytes, 0>>>(
+        b.q, b.k, b.v, b.o, nullptr, ps.H, ps.Sk, ps.Sq, scale, nullptr, nullptr);
+  }, ps.flush);
+  char name[128];
+  std::snprintf(name, sizeof name, "regfuse  Br=%d Bc=%d thr=%d bufs=%d/%d waves/SIMD=%d%s", Br, Bc, NT, NSK, NSV, WPE, PIPE ? " pipelined" : "");
+  report(name, ps, Kd, D, t);
+}
+
+// LDS-fused configuration: <Kd, D, Br, Bc, Nthreads, K buffers, V buffers, waves along kv, waves along d, waves per SIMD>
+template <int Kd, int D, int Br, int Bc, int NT, int NSK, int NSV, int W1N, int W2N, int WPE>
+static void test_smemfuse_attention(const ProblemShape& ps, const Buffers& b) {
+  using T = aat::AttnFwdSmemfuse<Kd, D, Br, Bc, NT, NSK, NSV, W1N, W2N>;
+  if (ps.Sq % Br || ps.Sk % Bc) return;
+  auto plain = &aat::flashattn_fwd_smemfuse<Kd, D, Br, Bc, NT, NSK, NSV, W1N, W2N, WPE, false>;
+  auto causal = &aat::flashattn_fwd_smemfuse<Kd, D, Br, Bc, NT, NSK, NSV, W1N, W2N, WPE, true>;
+  HIP_OK(hipFuncSetAttribute((const void*)plain, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
+  HIP_OK(hipFuncSetAttribute((const void*)causal, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
+  const float scale = 1.f / std::sqrt((float)Kd);
+  auto t = aat_bench::do_bench([&] {
+    (ps.causal ? causal : plain)<<<dim3(ps.B * ps.H * ps.Sq / Br), dim3(NT), T::kSmemBytes, 0>>>(
+        b.q, b.k, b.v, b.o, nullptr, ps.H, ps.Sk, ps.Sq, scale);
+  }, ps.flush);
+  char name[128];
+  std::snprintf(name, sizeof name, "smemfuse Br=%d Bc=%d thr=%d bufs=%d/%d grid=%dx%d waves/SIMD=%d", Br, Bc, NT, NSK, NSV, W1N, W2N, WPE);
+  report(name, ps, Kd, D, t);
+}
+
+int main(int argc, char** argv) {
+  ProblemShape ps{4, 32, 2048, 2048, false, true};
+  int pos = 0;
+  for (int i = 1; i < argc; ++i) {
+    if (!std::strcmp(argv[i], "--causal")) ps.causal = true;
+    else if (!std::strcmp(argv[i], "--no-flush")) ps.flush = false;
+    else {
+      int v = std::atoi(argv[i]);
+      if (pos == 0) ps.B = v; else if (pos == 1) ps.H = v; else if (pos == 2) ps.Sq = v; else if (pos == 3) ps.Sk = v;
+      ++pos;
+    }
+  }
+  hipDeviceProp_t prop;
+  HIP_OK(hipGetDeviceProperties(&prop, 0));
+  std::printf("%s  %d CUs  LDS/block %zu KB   problem B=%d H=%d Sq=%d Sk=%d d_qk=d_v=128 fp16 %s %s\n", prop.gcnArchName,
+              prop.multiProcessorCount, prop.sharedMemPerBlockOptin / 1024, ps.B, ps.H, ps.Sq, ps.Sk,
+              ps.causal ? "causal" : "non-causal", ps.flush ? "(cache flushed before every launch)" : "(hot cache)");
+  Buffers b = make_buffers<128, 128>(ps);
+  test_regfuse_attention<128, 128, 256, 64, 512, 2, 2, 3, false>(ps, b);
+  test_regfuse_attention<128, 128, 256, 64, 512, 2, 2, 2, false>(ps, b);
+  test_regfuse_attention<128, 128, 128, 64, 256, 2, 2, 3, false>(ps, b);
+  test_regfuse_attention<128, 128, 128, 64, 256, 1, 1, 2, false>(ps, b);
+  test_regfuse_attention<128, 128, 128, 32, 256, 2, 2, 3, false>(ps, b);
+  test_regfuse_attention<128, 128, 128, 32, 256, 2, 2, 2, true>(ps, b);
+  test_smemfuse_attention<128, 128, 128, 64, 256, 2, 2, 1, 4, 2>(ps, b);
+  test_smemfuse_attention<128, 128, 64, 64, 256, 2, 2, 2, 4, 2>(ps, b);
+  HIP_OK(hipFree(b.q)); HIP_OK(hipFree(b.k)); HIP_OK(hipFree(b.v)); HIP_OK(hipFree(b.o));
+  return 0;
+}
