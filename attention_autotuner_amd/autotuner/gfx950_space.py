@@ -184,22 +184,37 @@ BWD_BR_LIST = (64, 128)
 BWD_BC_LIST = (32, 64)
 
 
+def backward_dv_cols(cfg):
+    """dV columns one block produces.  With one wave per SIMD the output accumulators live in the 256
+    accumulation registers, which hold a 32-row group of up to 512 columns; otherwise (or for wider
+    values) the pass is sliced into 256-column blocks over grid.y and repeats its first contraction."""
+    rt = cfg.Br // _waves(cfg) // MFMA_M
+    if cfg.waves_per_eu == 1 and rt * cfg.D <= 512:
+        return cfg.D
+    return min(cfg.D, 256)
+
+
+def _backward_passes(cfg):
+    """(first-contraction width, output columns per block) of the dV, dK and dQ passes."""
+    return ((cfg.Kd, backward_dv_cols(cfg)), (cfg.D, cfg.Kd), (cfg.D, cfg.Kd))
+
+
 def backward_lds_bytes(cfg):
     worst = 0
-    dvb = min(cfg.D, 256)
-    for kx, dzb in ((cfg.Kd, dvb), (cfg.D, cfg.Kd), (cfg.D, cfg.Kd)):
+    for kx, dzb in _backward_passes(cfg):
         main = cfg.num_stages_qk * (cfg.Bc * kx * 2 + cfg.Br * cfg.Bc * 2) + cfg.num_stages_dv * cfg.Bc * dzb * 2
         worst = max(worst, main, cfg.Br * (dzb * 2 + 16))
     return worst
 
 
 def backward_reg_estimate(cfg):
+    """(vector registers, accumulation registers) of the hungriest pass."""
     rt = cfg.Br // _waves(cfg) // MFMA_M
-    worst = 0
-    dvb = min(cfg.D, 256)
-    for kx, dzb in ((cfg.Kd, dvb), (cfg.D, cfg.Kd)):
-        worst = max(worst, rt * (kx // 16) * 4 + rt * (cfg.Bc // 32) * 24 + rt * (dzb // 32) * 16 + 64)
-    return worst
+    vec = acc = 0
+    for kx, dzb in _backward_passes(cfg):
+        vec = max(vec, rt * (kx // 16) * 4 + rt * (cfg.Bc // 32) * 24 + 64)
+        acc = max(acc, rt * (dzb // 32) * 16)
+    return vec, acc
 
 
 def backward_valid(cfg, arch):
@@ -208,22 +223,28 @@ def backward_valid(cfg, arch):
         return False
     if nw > 4 * cfg.waves_per_eu:
         return False
+    if cfg.num_stages_qk not in (1, 2, 3) or cfg.num_stages_dv not in (1, 2):
+        return False
+    if cfg.num_stages_qk == 3 and cfg.num_stages_dv != 2:      # the three-buffer schedule prefetches Z one tile ahead
+        return False
     nt = cfg.Nthreads
-    dvb = min(cfg.D, 256)
-    for cols in (cfg.Kd, cfg.D, dvb, cfg.Br):          # every streamed tile must split evenly over the threads
+    for cols in (cfg.Kd, cfg.D, backward_dv_cols(cfg), cfg.Br):   # every streamed tile must split evenly over the threads
         if (cfg.Bc * cols // 8) % nt:
             return False
     if (cfg.Br * cfg.Bc // 8) % nt:
         return False
     if backward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
         return False
-    return backward_reg_estimate(cfg) <= arch.register_per_thread // cfg.waves_per_eu
+    vec, acc = backward_reg_estimate(cfg)
+    if cfg.waves_per_eu == 1:          # 256 vector + 256 accumulation registers
+        return vec <= 256 and acc <= 256
+    return vec + acc <= arch.register_per_thread // cfg.waves_per_eu
 
 
 def backward_candidates(br, bc, dim_qk, dim_v):
     out = []
     for nthreads in (128, 256):
-        for st_y, st_z in ((1, 1), (2, 2), (2, 1)):
+        for st_y, st_z in ((1, 1), (2, 2), (2, 1), (3, 2)):
             for wpe in (1, 2):
                 n = nthreads // WAVE
                 out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, BlockKSmem=dim_qk,
@@ -232,7 +253,8 @@ def backward_candidates(br, bc, dim_qk, dim_v):
 
 
 def default_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
-    for br, bc, nt, sy, sz, wpe in ((64, 32, 128, 1, 1, 1), (64, 32, 128, 1, 1, 2), (64, 64, 128, 1, 1, 1)):
+    for br, bc, nt, sy, sz, wpe in ((128, 32, 256, 3, 2, 1), (128, 32, 256, 2, 2, 1), (64, 32, 128, 2, 2, 1), (64, 32, 128, 1, 1, 1),
+                                    (64, 32, 128, 1, 1, 2), (64, 64, 128, 1, 1, 1)):
         if any(s and (s % br or s % bc) for s in (seq_q, seq_k)):
             continue
         n = nt // WAVE

@@ -61,7 +61,7 @@ def flops(op, b, h, sq, sk, dqk, dv, causal):
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("op", choices=["attn", "ret", "ret_bwd"])
-    ap.add_argument("dims", type=int, nargs=6, metavar=("B", "H", "Sq", "Sk", "dqk", "dv"))
+    ap.add_argument("dims", type=int, nargs=6, metavar="N", help="B H Sq Sk dqk dv")
     ap.add_argument("--causal", action="store_true")
     ap.add_argument("--compile-only", action="store_true")
     ap.add_argument("--log-dir", default=DEFAULT_LOG_DIR)

@@ -58,7 +58,7 @@ struct RetBwdChain {
   static constexpr int NCM = kMCols / 8;
   static_assert(Nthreads % kWave == 0 && BX % NW == 0 && WM % 32 == 0, "each wave owns whole 32-row groups");
   static_assert(BY % 32 == 0 && KX % 64 == 0 && DZ % DZB == 0 && DZB % 64 == 0, "tile shape");
-  static_assert((NSY == 1 || NSY == 2) && (NSZ == 1 || NSZ == 2), "buffers");
+  static_assert(NSY >= 1 && NSY <= 3 && (NSZ == 1 || NSZ == 2) && (NSY < 3 || NSZ == 2), "buffers");
   using YDma = TileDma<BY, NCY, Nthreads, Swz::Rows16>;
   using ZDma = TileDma<BY, NCZ, Nthreads, Swz::Rows4>;
   using MDma = TileDma<kMRows, NCM, Nthreads, PASS == BwdPass::Col ? Swz::Rows4 : Swz::Rows16>;
@@ -164,39 +164,82 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = zero16();
 
-  auto issue_ym = [&](int j, int par) {           // Y tile j and mask tile j travel together
-    ydma.issue(yg + (size_t)j * T::kYBytes, ybuf + (NSY == 2 ? par * T::kYBytes : 0), wave_base);
+  // Streamed tiles travel through rings of NSY (Y + mask) and NSZ (Z) LDS buffers; `st` is a ring slot.
+  auto issue_ym = [&](int j, int st) {            // Y tile j and mask tile j travel together
+    ydma.issue(yg + (size_t)j * T::kYBytes, ybuf + st * T::kYBytes, wave_base);
     const char* msrc = COL ? mg + (size_t)j * BY * seq_k * 2 : mg + (size_t)j * BY * 2;
-    mdma.issue(msrc, mbuf + (NSY == 2 ? par * T::kMBytes : 0), wave_base);
+    mdma.issue(msrc, mbuf + st * T::kMBytes, wave_base);
   };
-  auto issue_z = [&](int j, int par) {
-    zdma.issue(zg + (size_t)j * BY * DZ * 2, zbuf + (NSZ == 2 ? par * T::kZBytes : 0), wave_base);
+  auto issue_z = [&](int j, int st) {
+    zdma.issue(zg + (size_t)j * BY * DZ * 2, zbuf + st * T::kZBytes, wave_base);
   };
-  if (j_begin < j_end) {
-    issue_ym(j_begin, 0);
-    if constexpr (NSZ == 2) issue_z(j_begin, 0);
-  }
-  auto y_tile = [&](const int j, auto parity_tag) {
-    constexpr int PAR = decltype(parity_tag)::value;
-    const bool more = (j + 1 < j_end);
-    // (A) Y_j, mask_j (and with two Z buffers Z_j) have landed; every wave is past the previous tile.
-    wait_vmcnt<0>();
-    block_sync();
-    if constexpr (NSZ == 1) issue_z(j, 0);
-    if (more) {
-      if constexpr (NSY == 2) issue_ym(j + 1, PAR ^ 1);
-      if constexpr (NSZ == 2) issue_z(j + 1, PAR ^ 1);
-    }
-    f4v rv[COL ? NT * 4 : 1];                     // COL pass: r of this tile's query rows, as this lane sees them
+  auto load_r = [&](f4v (&rv)[COL ? NT * 4 : 1], int j) {   // COL pass: r of tile j's query rows, as this lane sees them
     if constexpr (COL) {
 #pragma unroll
       for (int i = 0; i < NT * 4; ++i)
         rv[i] = *reinterpret_cast<const f4v*>(rg + j * BY + 32 * (i >> 2) + 8 * (i & 3) + 4 * h);
     }
+  };
+  constexpr int kYmInstr = T::YDma::kIters + T::MDma::kIters;   // LDS-DMA instructions per thread for one Y + mask tile
+  constexpr int kRInstr = COL ? NT * 4 : 0;                     // register loads of r per tile
+  // Issue order (three Y/mask buffers):  prologue  YM(j0) Z(j0) YM(j0+1);  tile j  Z(j+1) YM(j+2).
+  // Loads retire in order, so "at most kYmInstr (+ the r loads of the next tile) outstanding" at the top
+  // of tile j means YM(j) and Z(j) have landed while YM(j+1) may still be in flight: a Y/mask tile gets
+  // two tile times to arrive, a Z tile one.  With one or two buffers every wait drains the queue.
+  if (j_begin < j_end) {
+    issue_ym(j_begin, 0);
+    if constexpr (NSZ == 2) issue_z(j_begin, 0);
+    if constexpr (NSY == 3) {
+      if (j_begin + 1 < j_end) issue_ym(j_begin + 1, 1);
+    }
+  }
+  f4v rv[COL ? NT * 4 : 1];
+  if (j_begin < j_end) load_r(rv, j_begin);
+
+  // One tile, with its ring slots as compile-time constants so every LDS offset folds into an immediate;
+  // the walk below repeats with period lcm(NSY, NSZ).
+  auto y_tile = [&](const int j, auto ys_tag, auto zs_tag) {
+    constexpr int ys = decltype(ys_tag)::value, zs = decltype(zs_tag)::value;
+    constexpr int ys1 = (ys + 1) % NSY, ys2 = (ys + 2) % NSY, zs1 = (zs + 1) % NSZ;
+    const bool more = (j + 1 < j_end);
+    if constexpr (WPE == 1) {
+      // Above 256 registers the file is split into 256 vector and 256 accumulation registers.  Pin the
+      // output accumulators to the accumulation half and the resident fragments to the vector half at
+      // every tile boundary; left alone the allocator parks the fragments in accumulation registers and
+      // copies four of them back in front of every MFMA.
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(acc[rt][dt]));
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[rt][ks]));
+      }
+    }
+    f4v rv_next[COL ? NT * 4 : 1];                // r of the next tile's rows: a full tile time to arrive
+    if (more) load_r(rv_next, j + 1);
+    sched_fence();
+    // (A) Y_j and mask_j (and with two Z buffers Z_j) have landed; every wave is past the previous tile.
+    if constexpr (NSY == 3) {
+      if (more) wait_vmcnt<kYmInstr + kRInstr>();
+      else wait_vmcnt<0>();
+    } else {
+      wait_vmcnt<0>();
+    }
+    block_sync();
+    if constexpr (NSZ == 1) issue_z(j, 0);
+    if (more) {
+      if constexpr (NSZ == 2) issue_z(j + 1, zs1);
+      if constexpr (NSY == 2) issue_ym(j + 1, ys1);
+    }
+    if constexpr (NSY == 3) {
+      if (j + 2 < j_end) issue_ym(j + 2, ys2);
+    }
+    constexpr int yoff = ys * T::kYBytes, moff = ys * T::kMBytes, zoff = zs * T::kZBytes;
 
     f16v tacc[RT][NT];
-    qk_gemm_steps<RT, NT, KS, NCY, PF>(tacc, xf, yaddr, NSY == 2 ? PAR * T::kYBytes : 0, [](int) {});
-    const int moff = NSY == 2 ? PAR * T::kMBytes : 0;
+    // the score tile accumulates in vector registers when the outputs fill the accumulation registers
+    constexpr bool kVacc = WPE == 1 && RT * (DT + NT) * 16 > 256;
+    qk_gemm_steps<RT, NT, KS, NCY, PF, kVacc>(tacc, xf, yaddr, yoff, [](int) {});
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       if constexpr (COL) {
@@ -225,16 +268,22 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
       }
     }
     h8 ef[RT][NT][2];
-    pv_gemm_steps<RT, NT, DT, NCZ, PF>(acc, ef, zaddr, NSZ == 2 ? PAR * T::kZBytes : 0, [&](int g) {
+    pv_gemm_steps<RT, NT, DT, NCZ, PF>(acc, ef, zaddr, zoff, [&](int g) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) pack_group<NT>(ef[rt], tacc[rt], g);
     });
+    if constexpr (COL) {
+#pragma unroll
+      for (int i = 0; i < NT * 4; ++i) rv[i] = rv_next[i];
+    }
   };
-  using P0 = std::integral_constant<int, 0>;
-  using P1 = std::integral_constant<int, 1>;
-  for (int j = j_begin; j < j_end; j += 2) {
-    y_tile(j, P0{});
-    if (j + 1 < j_end) y_tile(j + 1, P1{});
+  constexpr int kPeriod = NSY * NSZ / cgcd(NSY, NSZ);
+  for (int j = j_begin; j < j_end; j += kPeriod) {
+    static_for<kPeriod>([&](auto k_tag) {
+      constexpr int k = decltype(k_tag)::value;
+      if (k == 0 || j + k < j_end)
+        y_tile(j + k, std::integral_constant<int, k % NSY>{}, std::integral_constant<int, k % NSZ>{});
+    });
   }
 
   wait_vmcnt<0>();

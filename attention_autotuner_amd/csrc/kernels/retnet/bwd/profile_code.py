@@ -21,7 +21,10 @@ constexpr int Nthreads = {Nthreads};
 constexpr int num_stages_qk = {num_stages_qk};   // LDS buffers of the first-contraction stream (+ mask)
 constexpr int num_stages_dv = {num_stages_dv};   // LDS buffers of the second-contraction stream
 constexpr int waves_per_eu = {waves_per_eu};
-constexpr int DVB = D > 256 ? 256 : D;           // dV columns per block (wider outputs are sliced over grid.y)
+// dV columns per block: the whole row when the accumulators fit the 256 accumulation registers that one
+// wave per SIMD has to itself, else 256-column slices over grid.y (each repeats the first contraction).
+constexpr int RTv = Br / (Nthreads / 64) / 32;
+constexpr int DVB = (waves_per_eu == 1 && RTv * D <= 512) ? D : (D > 256 ? 256 : D);
 constexpr int DKB = Kd;
 
 using aat::BwdPass;

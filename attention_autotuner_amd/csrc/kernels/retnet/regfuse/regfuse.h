@@ -127,6 +127,18 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
     char* const vcur = vbuf + (NSV == 2 ? PAR * T::kVBytes : 0);
     const bool more = (j + 1 < n_tiles);
 
+    if constexpr (WPE == 1) {
+      // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
+      // output accumulators in the accumulation half and the Q fragments in the vector half, or the
+      // allocator parks Q there and copies four registers back in front of every MFMA.
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
+      }
+    }
     // (A) K_j, mask_j (and with two V buffers V_j) have landed; every wave is past iteration j-1.
     wait_vmcnt<0>();
     block_sync();
@@ -137,11 +149,13 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
     }
 
     f16v sacc[RT][NT];
-    qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
+    // the score tile accumulates in vector registers when the outputs fill the accumulation registers
+    constexpr bool kVacc = WPE == 1 && RT * (DT + NT) * 16 > 256;
+    qk_gemm_steps<RT, NT, KS, NCK, PF, kVacc>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       apply_mask<NT>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
-      retention_step<NT, DT>(sacc[rt], row[rt], oacc[rt]);
+      retention_step<NT, DT, WPE == 1>(sacc[rt], row[rt], oacc[rt]);
     }
 
     // (B) with one buffer: V_j must have landed / K and mask buffers must be free before the next fetch.

@@ -15,6 +15,7 @@
 // then a lane owns ONE query row (n) and 16 of every 32 kv positions, row reductions are in-lane plus
 // one exchange with lane^32, and the C registers of S^T are already a valid B operand for O^T = V^T * P^T.
 #pragma once
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
@@ -58,18 +59,8 @@ AAT_DEV constexpr int c_row(int v, int h) { return 8 * (v >> 2) + 4 * h + (v & 3
 // compiler keeps LDS accesses on their side of it; the hardware waits are spelled out by the caller
 // (vmcnt covers global loads AND LDS-DMA writes, lgkmcnt covers ds_read/ds_write).
 template <int N> AAT_DEV void wait_vmcnt() {
-  if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  else if constexpr (N == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-  else if constexpr (N == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-  else if constexpr (N == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-  else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  else if constexpr (N == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-  else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-  else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-  else if constexpr (N == 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-  else if constexpr (N == 32) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // unknown count: be conservative
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 AAT_DEV void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // Workgroup barrier that makes this thread's finished LDS traffic (ds ops and, when the caller has
@@ -109,6 +100,14 @@ template <int NC, Swz MODE> AAT_DEV constexpr int swz(int row, int c) {
 }
 
 constexpr int cgcd(int a, int b) { return b == 0 ? a : cgcd(b, a % b); }
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order.
+template <int N, int I = 0, class F> AAT_DEV void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
 
 // The source address of every copy is split into a wave-uniform part (tile pointer + a compile-time
 // multiple of the row pitch, kept in SGPRs) and one 32-bit per-lane offset, so a tile copy costs one
@@ -151,13 +150,16 @@ struct TileDma {
   template <int I0, int I1>
   AAT_DEV void issue_part(const char* g, char* lds, int wave_base) const {
 #pragma unroll
-    for (int i = I0; i < I1; ++i) {
-      uint64_t base = (uint64_t)(uintptr_t)(kRegular ? g + (size_t)i * kRowsPerIter * pitch : g);
-      asm volatile("" : "+s"(base));                   // keep the uniform part in SGPRs (saddr form)
-      const uint32_t lane_off = loff[kRegular ? i % kDistinct : i];
-      __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)(base + lane_off),
-                                       (AAT_AS3 void*)(lds + (i * NT + wave_base) * 16), 16, 0, 0);
-    }
+    for (int i = I0; i < I1; ++i) issue_one(i, g, lds, wave_base);
+  }
+  // Instruction i alone (i must fold to a constant where this is inlined): lets a caller thread the
+  // copy of a tile between other instructions one LDS-DMA instruction at a time.
+  AAT_DEV void issue_one(int i, const char* g, char* lds, int wave_base) const {
+    uint64_t base = (uint64_t)(uintptr_t)(kRegular ? g + (size_t)i * kRowsPerIter * pitch : g);
+    asm volatile("" : "+s"(base));                     // keep the uniform part in SGPRs (saddr form)
+    const uint32_t lane_off = loff[kRegular ? i % kDistinct : i];
+    __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)(base + lane_off),
+                                     (AAT_AS3 void*)(lds + (i * NT + wave_base) * 16), 16, 0, 0);
   }
 };
 

@@ -37,7 +37,9 @@ AAT_DEV void apply_mask(f16v (&s)[NT], const uint32_t (&maddr)[NT * 4], int buf_
 
 // Fold one masked score tile into the row statistics and turn it into P = S / r_ref (in place).
 // Rescales the O accumulators when the reference scale moves.
-template <int NT, int DT>
+// ACC_PIN: the O accumulators live in accumulation registers (kernels above 256 registers); rescale
+// them one 16-register block at a time so the copies through vector registers stay short-lived.
+template <int NT, int DT, bool ACC_PIN = false>
 AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) {
   float part = 0.f;
 #pragma unroll
@@ -51,9 +53,11 @@ AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) 
     const float alpha = row.r_ref * fast_rcp(r_new);
     row.r_ref = r_new;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+      if constexpr (ACC_PIN) asm volatile("" : "+a"(oacc[dt]));
+    }
   }
   const float inv = fast_rcp(row.r_ref);
 #pragma unroll

@@ -105,32 +105,83 @@ AAT_DEV void sched_fence() {}
 AAT_DEV void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 #endif
 
+// b128 LDS read issued behind the compiler's back, with the wait spelled out by the caller.  While an
+// LDS-DMA copy is in flight the compiler answers every dependency on a tracked LDS load with
+// lgkmcnt(0), which also waits for the prefetches issued after the fragment that is needed; LDS reads
+// retire in order, so "at most N younger reads outstanding" is enough.  `imm` must fold to a constant.
+AAT_DEV h8 lds_read_h8_async(uint32_t base, int imm) {
+  h8 v;
+  const uint32_t hi = (uint32_t)imm & ~0xffffu;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(base + hi), "i"(imm & 0xffff));
+  return v;
+}
+// Wait until at most N LDS operations issued after the one that produced `v` are outstanding.  The
+// operand ties the wait to the value, so no consumer of `v` can be scheduled above it.
+template <int N> AAT_DEV void lds_wait_younger(h8& v) {
+  static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));
+}
+
+// MFMA with its accumulator forced into vector registers.  A kernel that owns more than 256 registers
+// gets every compiler-issued MFMA in the form that accumulates in the 256 accumulation registers; when
+// the output accumulators fill those, the short-lived score tile has to live in vector registers, which
+// only a hand-written instruction can ask for.  The compiler does not see an MFMA here and inserts no
+// wait states after it: mfma_settle() must stand between the last of these and any other reader.
+AAT_DEV void mfma_32x32x16_vacc_first(f16v& c, h8 a, h8 b) {
+  asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+}
+AAT_DEV void mfma_32x32x16_vacc(f16v& c, h8 a, h8 b) {
+  asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+// 24 wait states: more than the 16 passes + 3 the longest matrix instruction needs before another unit
+// may read its result.
+AAT_DEV void mfma_settle(f16v& c) { asm volatile("s_nop 15\n\ts_nop 7" : "+v"(c)); }
+
 // S^T = K Q^T over one kv tile.  kaddr[ks] = LDS address of this lane's chunk for k-step ks in score
 // tile 0 of the K buffer (tile nt adds nt*32 rows).  side(step) runs after the MFMA group of each step.
-template <int RT, int NT, int KS, int NCK, int PF, class Side>
+// VACC: accumulate in vector registers through hand-written MFMAs (see mfma_32x32x16_vacc).
+template <int RT, int NT, int KS, int NCK, int PF, bool VACC = false, class Side>
 AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const uint32_t (&kaddr)[KS],
                            int buf_off, Side&& side) {
   constexpr int S = NT * KS;
   constexpr int kTileStride = 32 * NCK * 16;
+  // With rows of whole 16-chunk groups the swizzle only permutes chunks inside a group, so k-step ks
+  // sits 256 bytes per group behind k-step ks % 8: eight address registers serve any contraction width.
+  constexpr bool kFold = NCK % 16 == 0 && KS > 8;
+  auto read = [&](int i) {
+    const int ks = i % KS;
+    return lds_read_h8_async(kFold ? kaddr[ks % 8] : kaddr[ks],
+                             (kFold ? (ks / 8) * 256 : 0) + buf_off + (i / KS) * kTileStride);
+  };
+  if constexpr (!VACC) {
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) sacc[rt][nt] = zero16();
+      for (int nt = 0; nt < NT; ++nt) sacc[rt][nt] = zero16();
+  }
   h8 ring[PF];
 #pragma unroll
-  for (int i = 0; i < PF && i < S; ++i) ring[i] = lds_read_h8_at(kaddr[i % KS] + buf_off + (i / KS) * kTileStride);
+  for (int i = 0; i < PF && i < S; ++i) ring[i] = read(i);
   sched_fence();
+  static_for<S>([&](auto step_tag) {
+    constexpr int step = decltype(step_tag)::value;
+    h8 cur = ring[step % PF];
+    if constexpr (step + PF < S) ring[step % PF] = read(step + PF);
+    lds_wait_younger<(step + PF < S) ? PF : S - 1 - step>(cur);
 #pragma unroll
-  for (int step = 0; step < S; ++step) {
-    const h8 cur = ring[step % PF];
-    if (step + PF < S) {
-      const int nx = step + PF;
-      ring[step % PF] = lds_read_h8_at(kaddr[nx % KS] + buf_off + (nx / KS) * kTileStride);
+    for (int rt = 0; rt < RT; ++rt) {
+      if constexpr (!VACC) sacc[rt][step / KS] = mfma_32x32x16(cur, qf[rt][step % KS], sacc[rt][step / KS]);
+      else if constexpr (step % KS == 0) mfma_32x32x16_vacc_first(sacc[rt][step / KS], cur, qf[rt][step % KS]);
+      else mfma_32x32x16_vacc(sacc[rt][step / KS], cur, qf[rt][step % KS]);
     }
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) sacc[rt][step / KS] = mfma_32x32x16(cur, qf[rt][step % KS], sacc[rt][step / KS]);
     side(step);
     sched_fence();
+  });
+  if constexpr (VACC) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) mfma_settle(sacc[rt][nt]);
   }
 }
 
