@@ -82,7 +82,7 @@ class BaseTunner:
         ns = getattr(config, "kv_splits", 1)
         if ns > 1 and (s["Sk"] // config.Bc) % ns:
             return False
-        if config.operation == "ret_bwd":             # both lengths are resident in one pass, streamed in another
+        if config.operation in ("ret_bwd", "attn_bwd"):   # both lengths are resident in one pass, streamed in another
             return all(s[n] % config.Br == 0 and s[n] % config.Bc == 0 for n in ("Sq", "Sk"))
         return s["Sq"] % config.Br == 0 and s["Sk"] % config.Bc == 0
 

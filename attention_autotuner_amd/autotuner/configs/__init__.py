@@ -2,12 +2,14 @@ from .base_config import BaseConfig, balanced_wave_split, factor_pairs
 from .attention import AttnConfig
 from .retnet import RetConfig
 from .retnet_bwd import RetBwdConfig
+from .attention_bwd import AttnBwdConfig
 
 supported_configs = {
     "attn": AttnConfig,
     "ret": RetConfig,
     "ret_bwd": RetBwdConfig,
+    "attn_bwd": AttnBwdConfig,
 }
 
-__all__ = ["BaseConfig", "AttnConfig", "RetConfig", "RetBwdConfig", "supported_configs",
+__all__ = ["BaseConfig", "AttnConfig", "RetConfig", "RetBwdConfig", "AttnBwdConfig", "supported_configs",
            "balanced_wave_split", "factor_pairs"]

@@ -6,7 +6,7 @@ whole-tile buffers; and the register file is split between the resident waves of
 occupancy target (``waves_per_eu``) is itself a knob.  Validity is LDS bytes (160 KB per CU, shared by
 all resident blocks) and a per-lane register estimate (512 / waves_per_eu).
 """
-from .configs import AttnConfig, RetConfig, RetBwdConfig
+from .configs import AttnConfig, RetConfig, RetBwdConfig, AttnBwdConfig
 
 WAVE = 64
 MFMA_M = 32
@@ -263,3 +263,61 @@ def default_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
         if backward_valid(cfg, arch):
             return cfg
     raise ValueError(f"no default ret_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
+
+
+# ---- backward (attention) ------------------------------------------------------------------------------
+# A column kernel (dV, dK) and a row kernel (dQ) share Br (resident rows) and Bc (streamed rows per step).
+ATTN_BWD_BR_LIST = (64, 128, 256)
+ATTN_BWD_BC_LIST = (32, 64)
+
+
+def attn_backward_lds_bytes(cfg):
+    stage = cfg.Bc * (cfg.Kd + cfg.D) * 2 + 1024            # streamed tile pair + per-row statistics slot
+    return max(cfg.num_stages_qk * stage, cfg.Br * (max(cfg.Kd, cfg.D) * 2 + 16))
+
+
+def attn_backward_reg_estimate(cfg):
+    """(vector registers, accumulation registers) of the column kernel, the hungrier of the two."""
+    rt = cfg.Br // _waves(cfg) // MFMA_M
+    nt = cfg.Bc // 32
+    vec = rt * ((cfg.Kd + cfg.D) // 16) * 4 + rt * nt * 16 + 72
+    acc = rt * ((cfg.Kd + cfg.D) // 32) * 16 + rt * nt * 32
+    return vec, acc
+
+
+def attn_backward_valid(cfg, arch):
+    nw = _waves(cfg)
+    if cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * nw) or cfg.Bc % 32 or cfg.Bc > 128:
+        return False
+    if nw > 4 * cfg.waves_per_eu or cfg.num_stages_qk not in (2, 3):
+        return False
+    for cols in (cfg.Kd, cfg.D):
+        if cols % 64 or (cols // 8 != 8 and (cols // 8) % 16):     # the dual swizzle covers 64-wide and multiples of 128
+            return False
+        if (cfg.Bc * cols // 8) % cfg.Nthreads:
+            return False
+    if attn_backward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
+        return False
+    vec, acc = attn_backward_reg_estimate(cfg)
+    if cfg.waves_per_eu == 1:
+        return vec <= 256 and acc <= 256
+    return vec + acc <= arch.register_per_thread // cfg.waves_per_eu
+
+
+def attn_backward_candidates(br, bc, dim_qk, dim_v):
+    out = []
+    for nthreads in (128, 256, 512):
+        for stages in (2, 3):
+            for wpe in (1, 2):
+                out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=wpe))
+    return out
+
+
+def default_attn_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
+    for br, bc, nt, st, wpe in ((128, 32, 256, 3, 1), (128, 32, 256, 2, 1), (64, 32, 128, 3, 1), (64, 32, 128, 2, 1), (64, 32, 128, 2, 2)):
+        if any(s and (s % br or s % bc) for s in (seq_q, seq_k)):
+            continue
+        cfg = AttnBwdConfig(br, bc, dim_qk, dim_v, nt, st, waves_per_eu=wpe)
+        if attn_backward_valid(cfg, arch):
+            return cfg
+    raise ValueError(f"no default attn_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")

@@ -5,7 +5,11 @@ import threading
 _VP, _I, _F, _SZ = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
 
 # number of device-pointer arguments per operator
-N_POINTERS = {"attn": 4, "ret": 6, "ret_bwd": 10}
+N_POINTERS = {"attn": 4, "ret": 6, "ret_bwd": 10, "attn_bwd": 9}
+# operators whose extended entry points take a softmax scale in front of the causal flag
+SCALED_OPS = ("attn", "attn_bwd")
+# operators that also export the reference-signature pair profile / kernel_entry
+LEGACY_OPS = ("attn", "ret", "ret_bwd")
 
 _handles = {}
 _lock = threading.Lock()
@@ -24,12 +28,16 @@ def _bind(lib, op):
     lib.config_string.argtypes = []
     lib.workspace_size.restype = _SZ
     lib.workspace_size.argtypes = [_I] * 4
-    lib.profile.restype = _F
-    lib.profile.argtypes = ptrs + [_I] * 4
-    lib.kernel_entry.restype = _I
-    lib.kernel_entry.argtypes = ptrs + [_I] * 4
-    extra = [_F, _I] if op == "attn" else [_I]       # attention: scale + causal; RetNet: causal
+    if op in LEGACY_OPS:
+        lib.profile.restype = _F
+        lib.profile.argtypes = ptrs + [_I] * 4
+        lib.kernel_entry.restype = _I
+        lib.kernel_entry.argtypes = ptrs + [_I] * 4
+    extra = [_F, _I] if op in SCALED_OPS else [_I]   # attention: scale + causal; RetNet: causal
     tail = extra + [_VP, _SZ, _VP]                   # workspace, bytes, stream
+    if op == "attn":
+        lib.kernel_entry_lse.restype = _I
+        lib.kernel_entry_lse.argtypes = [_VP] * 5 + [_I] * 4 + tail
     lib.profile_ex.restype = _F
     lib.profile_ex.argtypes = ptrs + [_I] * 4 + tail
     lib.kernel_entry_ex.restype = _I

@@ -36,6 +36,11 @@ PARITY_TILES = [
 PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
 
 
+ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (256, 128)]
+# (Br, Bc, Nthreads, buffers) variants of the attention backward at 128/128 for the parity suite
+ATTN_BWD_TILES = [(64, 32, 128, 2), (64, 64, 128, 2), (128, 64, 256, 3), (128, 32, 256, 2)]
+
+
 def extra_configs(arch=None):
     """Additional libraries built ahead of time: the parity matrix."""
     from .configs import AttnConfig, RetConfig
@@ -50,6 +55,13 @@ def extra_configs(arch=None):
                 out.append(cfg)
     for dims in ((64, 64), (128, 128), (256, 256), (64, 128), (256, 512)):
         out.append(gfx950_space.default_backward_config(*dims, arch, 128, 128))
+    # attention backward: the defaults per head-size pair and sequence divisibility, plus tile variants
+    from .configs import AttnBwdConfig
+    for dims in ATTN_BWD_DIMS:
+        for seq in (None, 128, 64):
+            out.append(gfx950_space.default_attn_backward_config(*dims, arch, seq, seq))
+    for br, bc, nt, st in ATTN_BWD_TILES:
+        out.append(AttnBwdConfig(br, bc, 128, 128, nt, st))
     for dqk, dv in PARITY_DIMS:
         for br, bc, nt, sq, sv, wpe in PARITY_TILES:
             cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")

@@ -45,7 +45,8 @@ class Runtime:
     def workspace_size(self, B, H, Sq, Sk):
         return int(library.load(self._path(), self.config.operation).workspace_size(B, H, Sq, Sk))
 
-    def apply(self, torch_array, device=None, softmax_scale=None, causal=False, workspace=None):
+    def apply(self, torch_array, device=None, softmax_scale=None, causal=False, workspace=None, lse=None):
+        """``lse`` (attention forward only): fp32 [B,H,S_q] tensor that receives the log-sum-exp of every row."""
         q, k = torch_array[0], torch_array[1]
         if not q.is_cuda:
             raise KernelLaunchError("kernel libraries run on the GPU only; got CPU tensors")
@@ -57,15 +58,20 @@ class Runtime:
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
         ws_ptr = ctypes.c_void_p(workspace.data_ptr() if workspace is not None else 0)
         ws_bytes = ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0)
-        if op == "attn":
+        if op in library.SCALED_OPS:
             scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])
             extra = [ctypes.c_float(scale), ctypes.c_int(int(bool(causal)))]
         else:
             extra = [ctypes.c_int(int(bool(causal)))]
         with torch.cuda.device(q.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            rc = lib.kernel_entry_ex(*[ctypes.c_void_p(t.data_ptr()) for t in torch_array], B, H, Sq, Sk,
-                                     *extra, ws_ptr, ws_bytes, stream)
+            ptrs = [ctypes.c_void_p(t.data_ptr()) for t in torch_array]
+            if lse is not None:
+                if op != "attn":
+                    raise KernelLaunchError("only the attention forward writes a log-sum-exp")
+                rc = lib.kernel_entry_lse(*ptrs, ctypes.c_void_p(lse.data_ptr()), B, H, Sq, Sk, *extra, ws_ptr, ws_bytes, stream)
+            else:
+                rc = lib.kernel_entry_ex(*ptrs, B, H, Sq, Sk, *extra, ws_ptr, ws_bytes, stream)
         if rc != 0:
             raise KernelLaunchError(f"{op}:{self.config} failed with code {rc}: {_ERRORS.get(rc, 'HIP error')}")
         return rc

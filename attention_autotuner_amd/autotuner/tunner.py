@@ -89,3 +89,32 @@ class RetBwdTunner(BaseTunner):
         if not _is_rocm(self.arch):
             raise RuntimeError(f"{self.arch.name} configurations can be enumerated but not built on this platform")
         return super().tune(*a, **kw)
+
+
+class AttnBwdTunner(BaseTunner):
+    """Tuner for the flash-attention backward (no reference counterpart: reference
+    python/ops/attention_interface.py:37-58 leaves the operator empty).  ``torch_array`` is
+    [q, k, v, o, dO, lse, dq, dk, dv]."""
+    operation = "attn_bwd"
+
+    def __init__(self, arch, torch_array, causal=False, softmax_scale=None):
+        super().__init__(arch, torch_array, "attention_bwd", causal=causal, softmax_scale=softmax_scale)
+        self.Br_list = list(gfx950_space.ATTN_BWD_BR_LIST)
+        self.Bc_list = list(gfx950_space.ATTN_BWD_BC_LIST)
+
+    def generate_configs(self, Br, Bc, dim_qk, dim_v):
+        return gfx950_space.attn_backward_candidates(Br, Bc, dim_qk, dim_v)
+
+    def validate_kernel(self, config):
+        return gfx950_space.attn_backward_valid(config, self.arch)
+
+    def _ex_args(self):
+        scale = self.softmax_scale
+        if scale is None:
+            scale = 1.0 / math.sqrt(self.problem_key["dim_qk"])
+        return [ctypes.c_float(scale), ctypes.c_int(int(self.causal))]
+
+    def tune(self, *a, **kw):
+        if not _is_rocm(self.arch):
+            raise RuntimeError(f"{self.arch.name} has no attention-backward kernels")
+        return super().tune(*a, **kw)

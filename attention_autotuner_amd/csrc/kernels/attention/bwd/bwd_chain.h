@@ -1,0 +1,347 @@
+// Flash-attention backward for gfx950 (MI355X).
+//
+// With S = scale * Q K^T, P = exp(S - lse) (lse = the forward's log-sum-exp per query row) and
+// delta = rowsum(dO * O):
+//     dV = P^T dO,      dP = dO V^T,      dS = P * (dP - delta),      dK = scale * dS^T Q,      dQ = scale * dS K.
+// The reference declares this operator and leaves it empty (reference: python/ops/attention_interface.py:37-58,
+// README.md:107); the arithmetic follows its RetNet backward (csrc/kernels/retnet/bwd/bwd_colblock.h:445-596):
+// fp32 accumulation, P and dS rounded to fp16 (RNE) before the dependent contraction.
+//
+// Same construction as the RetNet backward of this library: no atomics, no fp32 dQ scratch.  Two
+// kernels walk the (kv block, q block) pairs, each keeping its resident rows' operands in registers (a
+// lane owns one resident row) and streaming the other side through LDS:
+//
+//     COL  resident kv rows (K, V fragments)  streams Q and dO tiles   ->  dV and dK
+//     ROW  resident q rows (Q, dO fragments)  streams K and V tiles    ->  dQ
+//
+// A streamed tile is read both ways -- row-major b128 fragments for the first contractions
+// (S^T = Q K^T resp. dP^T = dO V^T) and transposing reads for the second ones (dV^T += dO^T P,
+// dK^T += Q^T dS, dQ^T += K^T dS) -- so each tile is fetched once and laid out with the dual swizzle.
+// Cost: S and dP are evaluated by both kernels (7 instead of 5 contractions per score).
+//
+// lse2 = lse * log2(e) and delta come from attn_bwd_prepare (one pass over O and dO); the COL kernel
+// copies the 2 * BY values of a streamed tile into LDS next to the tile.
+#pragma once
+#include <type_traits>
+
+#include "../../utils/cdna4.h"
+#include "../../utils/tile_ops.h"
+
+#ifndef AAT_PF
+#define AAT_PF 2
+#endif
+
+namespace aat {
+
+enum class AttnBwdPass { Col, Row };
+
+// Kd: width of q/k rows; D: width of v/o/dO rows; BX: resident rows per block; BY: rows per streamed
+// tile; NS: LDS buffers of the stream (2 or 3).
+template <int Kd, int D, int BX, int BY, int Nthreads, int NS, AttnBwdPass PASS>
+struct AttnBwdChain {
+  static constexpr bool COL = PASS == AttnBwdPass::Col;
+  static constexpr int NW = Nthreads / kWave;
+  static constexpr int WM = BX / NW;
+  static constexpr int RT = WM / 32;
+  static constexpr int NT = BY / 32;
+  static constexpr int KS = Kd / 16, DS = D / 16;       // k-steps of the two first contractions
+  static constexpr int KT = Kd / 32, DT = D / 32;       // output tiles of the second contractions
+  static constexpr int NCK = Kd / 8, NCD = D / 8;
+  static_assert(Nthreads % kWave == 0 && BX % NW == 0 && WM % 32 == 0, "each wave owns whole 32-row groups");
+  static_assert(BY % 32 == 0 && Kd % 64 == 0 && D % 64 == 0, "tile shape");
+  static_assert(NS == 2 || NS == 3, "buffers");
+  using Y1Dma = TileDma<BY, NCK, Nthreads, Swz::Both>;  // Q (COL) or K (ROW) tile
+  using Y2Dma = TileDma<BY, NCD, Nthreads, Swz::Both>;  // dO (COL) or V (ROW) tile
+  static constexpr int kY1Bytes = BY * Kd * 2, kY2Bytes = BY * D * 2;
+  static constexpr int kStatBytes = COL ? 1024 : 0;     // lse2 and delta of the streamed rows (2 * BY floats)
+  static_assert(2 * BY * 4 <= 1024, "statistics slot");
+  static constexpr int kStatInstr = COL ? (2 * BY + 63) / 64 : 0;
+  static constexpr int kStageBytes = kY1Bytes + kY2Bytes + kStatBytes;
+  static constexpr int kTileInstr = Y1Dma::kIters + Y2Dma::kIters + kStatInstr;   // LDS-DMA instructions per thread per tile
+  static constexpr int kOCols = COL ? (D > Kd ? D : Kd) : Kd;
+  static constexpr int kOStride = kOCols * 2 + 16;
+  static constexpr int kMainBytes = NS * kStageBytes;
+  static constexpr int kEpiBytes = BX * kOStride;
+  static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
+};
+
+// delta[row] = sum_d dO[row][d] * O[row][d], lse2[row] = lse[row] * log2(e); one wave per 64/(D/8) rows.
+template <int D>
+__global__ void __launch_bounds__(256) attn_bwd_prepare(const half_t* __restrict__ o, const half_t* __restrict__ dO,
+                                                        const float* __restrict__ lse, float* __restrict__ lse2,
+                                                        float* __restrict__ delta, int rows) {
+  constexpr int kLanesPerRow = D / 8;                   // 16-byte chunks per row: 8, 16, 32 or 64
+  static_assert(64 % kLanesPerRow == 0, "row width");
+  constexpr int kRowsPerWave = 64 / kLanesPerRow;
+  const int lane = threadIdx.x & 63;
+  const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6;
+  const int row = wave * kRowsPerWave + lane / kLanesPerRow;
+  float s = 0.f;
+  if (row < rows) {
+    const size_t off = (size_t)row * D + (lane % kLanesPerRow) * 8;
+    const h8 a = *reinterpret_cast<const h8*>(o + off);
+    const h8 b = *reinterpret_cast<const h8*>(dO + off);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += (float)a[i] * (float)b[i];
+  }
+#pragma unroll
+  for (int m = 1; m < kLanesPerRow; m <<= 1) s += __shfl_xor(s, m, 64);
+  if (row < rows && lane % kLanesPerRow == 0) {
+    delta[row] = s;
+    lse2[row] = lse[row] * 1.4426950408889634f;
+  }
+}
+
+// x1, x2: resident-side matrices (COL: k, v; ROW: q, dO); y1, y2: streamed-side matrices (COL: q, dO;
+// ROW: k, v); all [B*H, S, width] fp16.  lse2, delta: [B*H, seq_q] fp32.  COL writes out1 = dV and
+// out2 = dK; ROW writes out2 = dQ.  c2 = softmax_scale * log2(e); out_scale = softmax_scale.
+template <int Kd, int D, int BX, int BY, int Nthreads, int NS, AttnBwdPass PASS, int WPE = 1>
+__global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
+attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, const half_t* __restrict__ y1,
+               const half_t* __restrict__ y2, const float* __restrict__ lse2, const float* __restrict__ delta,
+               half_t* __restrict__ out1, half_t* __restrict__ out2, int H, int seq_k, int seq_q, float c2,
+               float out_scale, int causal) {
+  using T = AttnBwdChain<Kd, D, BX, BY, Nthreads, NS, PASS>;
+  constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DS = T::DS, KT = T::KT, DT = T::DT, NCK = T::NCK, NCD = T::NCD,
+                WM = T::WM;
+  constexpr int PF = AAT_PF;
+  constexpr bool COL = T::COL;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, h = lane >> 5;
+  const int seq_x = COL ? seq_k : seq_q, seq_y = COL ? seq_q : seq_k;
+
+  const int Tx = seq_x / BX;
+  const int tile = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = tile / Tx;
+  const int x0 = (tile % Tx) * BX;
+  const int diag = seq_k - seq_q;                 // causal: score (q, kv) is kept when kv <= q + diag
+  int j_begin = 0, j_end = seq_y / BY;
+  if (causal) {
+    if constexpr (COL) {                          // q tiles that reach kv >= x0:  q >= x0 - diag
+      const int first = x0 - diag;
+      j_begin = first <= 0 ? 0 : first / BY;
+    } else {                                      // kv tiles with kv <= x0 + BX - 1 + diag
+      const int last = x0 + BX - 1 + diag;
+      const int lim = last < 0 ? 0 : last / BY + 1;
+      j_end = lim < j_end ? lim : j_end;
+    }
+  }
+
+  const char* y1g = reinterpret_cast<const char*>(y1 + (size_t)bh * seq_y * Kd);
+  const char* y2g = reinterpret_cast<const char*>(y2 + (size_t)bh * seq_y * D);
+  const float* lse_g = lse2 + (size_t)bh * seq_q;
+  const float* delta_g = delta + (size_t)bh * seq_q;
+
+  typename T::Y1Dma y1dma;
+  typename T::Y2Dma y2dma;
+  y1dma.init(tid);
+  y2dma.init(tid);
+  const int wave_base = wave * 64;
+
+  // resident operands: this lane's row of X1 (width Kd) and of X2 (width D) as MFMA B fragments
+  h8 x1f[RT][KS], x2f[RT][DS];
+  load_q_frags<RT, KS, Kd>(x1f, x1 + ((size_t)bh * seq_x + x0 + wave * WM + n) * Kd + 8 * h);
+  load_q_frags<RT, DS, D>(x2f, x2 + ((size_t)bh * seq_x + x0 + wave * WM + n) * D + 8 * h);
+
+  // LDS addresses inside stage 0: first-contraction fragments (rows n, chunk 2ks+h) and transposing reads
+  uint32_t y1addr[KS], y2addr[DS], z1lo[KT], z1hi[KT], z2lo[DT], z2hi[DT];
+  {
+    int o1[KS], o2[DS];
+    k_frag_offsets<KS, NCK, Swz::Both>(o1, n, h);
+    k_frag_offsets<DS, NCD, Swz::Both>(o2, n, h);
+#pragma unroll
+    for (int i = 0; i < KS; ++i) y1addr[i] = lds_addr(smem + o1[i]);
+#pragma unroll
+    for (int i = 0; i < DS; ++i) y2addr[i] = lds_addr(smem + T::kY1Bytes + o2[i]);
+    // transposing reads: rows 4h + (lane%16)/4 (+8 for the second half; the dual swizzle sees row bit 3,
+    // so the second half has its own address), columns 32*tile + 16*((lane/16)%2) + 4*(lane%4) .. +3
+    const int s16 = lane & 15;
+    const int row = 4 * h + (s16 >> 2);
+    const int col = 16 * ((lane >> 4) & 1) + 4 * (s16 & 3);
+#pragma unroll
+    for (int i = 0; i < KT; ++i) {
+      z1lo[i] = lds_addr(smem + lds_chunk_off<NCK, Swz::Both>(row, 4 * i + (col >> 3)) + (col & 7) * 2);
+      z1hi[i] = lds_addr(smem + lds_chunk_off<NCK, Swz::Both>(row + 8, 4 * i + (col >> 3)) + (col & 7) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < DT; ++i) {
+      z2lo[i] = lds_addr(smem + T::kY1Bytes + lds_chunk_off<NCD, Swz::Both>(row, 4 * i + (col >> 3)) + (col & 7) * 2);
+      z2hi[i] = lds_addr(smem + T::kY1Bytes + lds_chunk_off<NCD, Swz::Both>(row + 8, 4 * i + (col >> 3)) + (col & 7) * 2);
+    }
+  }
+  const uint32_t stat_addr = lds_addr(smem + T::kY1Bytes + T::kY2Bytes + 16 * h);   // + 32 B per register group
+
+  // ROW: the lane's own query row statistics
+  float lse_row[RT], delta_row[RT];
+  if constexpr (!COL) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      lse_row[rt] = lse_g[x0 + wave * WM + rt * 32 + n];
+      delta_row[rt] = delta_g[x0 + wave * WM + rt * 32 + n];
+    }
+  }
+
+  // accumulators: acc1 = dV^T (COL only, D wide), acc2 = dK^T (COL) or dQ^T (ROW), Kd wide
+  f16v acc1[RT][COL ? DT : 1], acc2[RT][KT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+    for (int i = 0; i < (COL ? DT : 1); ++i) acc1[rt][i] = zero16();
+#pragma unroll
+    for (int i = 0; i < KT; ++i) acc2[rt][i] = zero16();
+  }
+
+  auto issue = [&](int j, int st) {
+    char* base = smem + st * T::kStageBytes;
+    y1dma.issue(y1g + (size_t)j * T::kY1Bytes, base, wave_base);
+    y2dma.issue(y2g + (size_t)j * T::kY2Bytes, base + T::kY1Bytes, wave_base);
+    if constexpr (COL) {
+      // every wave copies the tile's 2*BY statistics (same bytes, same place): uniform instruction counts
+#pragma unroll
+      for (int i = 0; i < T::kStatInstr; ++i) {
+        const int idx = i * 64 + lane;              // [0, BY): lse2, [BY, 2BY): delta
+        const int c = idx < 2 * BY ? idx : 2 * BY - 1;
+        const float* src = c < BY ? lse_g + j * BY + c : delta_g + j * BY + (c - BY);
+        __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)src,
+                                         (AAT_AS3 void*)(base + T::kY1Bytes + T::kY2Bytes + i * 256), 4, 0, 0);
+      }
+    }
+  };
+  if (j_begin < j_end) {
+    issue(j_begin, 0);
+    if constexpr (NS == 3) {
+      if (j_begin + 1 < j_end) issue(j_begin + 1, 1);
+    }
+  }
+
+  auto y_tile = [&](const int j, auto st_tag) {
+    constexpr int st = decltype(st_tag)::value;
+    constexpr int off = st * T::kStageBytes;
+    const bool more = (j + 1 < j_end);
+    if constexpr (WPE == 1) {
+      // one wave per SIMD: outputs in the accumulation registers, resident fragments in vector registers
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if constexpr (COL) {
+#pragma unroll
+          for (int i = 0; i < DT; ++i) asm volatile("" : "+a"(acc1[rt][i]));
+        }
+#pragma unroll
+        for (int i = 0; i < KT; ++i) asm volatile("" : "+a"(acc2[rt][i]));
+#pragma unroll
+        for (int i = 0; i < KS; ++i) asm volatile("" : "+v"(x1f[rt][i]));
+#pragma unroll
+        for (int i = 0; i < DS; ++i) asm volatile("" : "+v"(x2f[rt][i]));
+      }
+    }
+    // tile j has landed (with three buffers tile j+1 may still be in flight); every wave is past tile j-1
+    if constexpr (NS == 3) {
+      if (more) wait_vmcnt<T::kTileInstr>();
+      else wait_vmcnt<0>();
+    } else {
+      wait_vmcnt<0>();
+    }
+    block_sync();
+    if constexpr (NS == 3) {
+      if (j + 2 < j_end) issue(j + 2, (st + 2) % 3);
+    } else {
+      if (more) issue(j + 1, st ^ 1);
+    }
+
+    // first contractions: s = Y1 X1^T (scores), p = Y2 X2^T (dP), both transposed (lane owns resident row)
+    f16v s[RT][NT], dp[RT][NT];
+    qk_gemm_steps<RT, NT, KS, NCK, PF>(s, x1f, y1addr, off, [](int) {});
+    qk_gemm_steps<RT, NT, DS, NCD, PF>(dp, x2f, y2addr, off, [](int) {});
+
+    // P = exp2(s*c2 - lse2[q]),  dS = P * (dP - delta[q]);  register v of tile t is streamed row 32t + 8(v/4) + 4h + v%4
+    const bool diag_tile = causal && (COL ? (x0 + BX - 1 > j * BY + diag) : ((j + 1) * BY - 1 > x0 + diag));
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int xrow = x0 + wave * WM + rt * 32 + n;             // resident row of this lane
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f4v l2, dl;
+          if constexpr (COL) {
+            l2 = *reinterpret_cast<AAT_AS3 const f4v*>((uintptr_t)(stat_addr + off + (32 * t + 8 * g) * 4));
+            dl = *reinterpret_cast<AAT_AS3 const f4v*>((uintptr_t)(stat_addr + off + (BY + 32 * t + 8 * g) * 4));
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int v = 4 * g + e;
+            const float lrow = COL ? l2[e] : lse_row[rt];
+            const float drow = COL ? dl[e] : delta_row[rt];
+            float p = fast_exp2(s[rt][t][v] * c2 - lrow);
+            if (diag_tile) {
+              const int yrow = j * BY + 32 * t + 8 * g + 4 * h + e;   // streamed row
+              const int qi = COL ? yrow : xrow, ki = COL ? xrow : yrow;
+              if (ki > qi + diag) p = 0.f;
+            }
+            s[rt][t][v] = p;
+            dp[rt][t][v] = p * (dp[rt][t][v] - drow);
+          }
+        }
+      }
+    }
+
+    // second contractions: COL  dV^T += dO^T P  and  dK^T += Q^T dS;   ROW  dQ^T += K^T dS
+    h8 ef[RT][NT][2];
+    if constexpr (COL) {
+      pv_gemm_steps_hl<RT, NT, DT, NCD, PF>(acc1, ef, z2lo, z2hi, off, [&](int g) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) ef[rt][g >> 1][g & 1] = pack8_rne(s[rt][g >> 1], 8 * (g & 1));
+      });
+    }
+    pv_gemm_steps_hl<RT, NT, KT, NCK, PF>(acc2, ef, z1lo, z1hi, off, [&](int g) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) ef[rt][g >> 1][g & 1] = pack8_rne(dp[rt][g >> 1], 8 * (g & 1));
+    });
+  };
+  for (int j = j_begin; j < j_end; j += NS) {
+    static_for<NS>([&](auto k_tag) {
+      constexpr int k = decltype(k_tag)::value;
+      if (k == 0 || j + k < j_end) y_tile(j + k, std::integral_constant<int, k>{});
+    });
+  }
+
+  // ---- epilogue: scale, round, transpose through wave-private LDS, 16-byte stores ---------------------
+  wait_vmcnt<0>();
+  block_sync();
+  char* const ostage = smem + wave * WM * T::kOStride;
+  auto store = [&](auto& acc, auto cols_tag, half_t* out, float sc) {
+    constexpr int W = decltype(cols_tag)::value;           // output row width
+    constexpr int NTILE = W / 32, kChunksPerRow = W / 8;
+    half_t* og = out + ((size_t)bh * seq_x + x0 + wave * WM) * W;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int dt = 0; dt < NTILE; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const h2 a = pack_rne(acc[rt][dt][4 * g] * sc, acc[rt][dt][4 * g + 1] * sc);
+          const h2 b = pack_rne(acc[rt][dt][4 * g + 2] * sc, acc[rt][dt][4 * g + 3] * sc);
+          h4 w;
+          w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
+          *reinterpret_cast<h4*>(ostage + (rt * 32 + n) * T::kOStride + (32 * dt + 8 * g + 4 * h) * 2) = w;
+        }
+    wait_lgkm0();
+    constexpr int kChunks = WM * kChunksPerRow;
+#pragma unroll
+    for (int t = 0; t < kChunks / 64; ++t) {
+      const int idx = t * 64 + lane;
+      const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
+      const u4v val = *reinterpret_cast<const u4v*>(ostage + row * T::kOStride + c * 16);
+      *reinterpret_cast<u4v*>(reinterpret_cast<char*>(og) + (size_t)row * W * 2 + c * 16) = val;
+    }
+    wait_lgkm0();                                           // the staging rows are reused by the next output
+  };
+  if constexpr (COL) store(acc1, std::integral_constant<int, D>{}, out1, 1.0f);
+  store(acc2, std::integral_constant<int, Kd>{}, out2, out_scale);
+}
+
+}  // namespace aat

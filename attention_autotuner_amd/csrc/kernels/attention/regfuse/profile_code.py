@@ -37,7 +37,7 @@ size_t split_workspace_bytes(int B, int H, int Seq_q) {{
 bool split_applies(int Seq_k, int causal) {{ return kv_splits > 1 && !causal && (Seq_k / Bc) % kv_splits == 0; }}
 
 hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k,
-                  float softmax_scale, int causal, void* workspace, hipStream_t stream) {{
+                  float softmax_scale, int causal, void* workspace, hipStream_t stream, float* lse = nullptr) {{
   if (split_applies(Seq_k, causal) && workspace != nullptr) {{
     static const hipError_t lds_ok_split = aat::allow_lds(kernel_split, shared_mem_split);
     if (lds_ok_split != hipSuccess) return lds_ok_split;
@@ -49,7 +49,7 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int
         reinterpret_cast<const aat::half_t*>(v), nullptr, nullptr, H, Seq_k, Seq_q, softmax_scale, part_o, part_lse);
     const size_t threads = rows * (D / 8);
     aat::attn_split_merge<D><<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream>>>(
-        part_o, part_lse, reinterpret_cast<aat::half_t*>(o), nullptr, (int)rows, kv_splits);
+        part_o, part_lse, reinterpret_cast<aat::half_t*>(o), lse, (int)rows, kv_splits);
     return hipGetLastError();
   }}
   static const hipError_t lds_ok = aat::allow_lds(kernel, shared_mem);
@@ -58,7 +58,7 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int
   if (lds_ok_causal != hipSuccess) return lds_ok_causal;
   (causal ? kernel_causal : kernel)<<<dim3(B * H * (Seq_q / Br)), dim3(Nthreads), shared_mem, stream>>>(
       reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
-      reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<aat::half_t*>(o), nullptr, H, Seq_k, Seq_q,
+      reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<aat::half_t*>(o), lse, H, Seq_k, Seq_q,
       softmax_scale, nullptr, nullptr);
   return hipGetLastError();
 }}
@@ -95,6 +95,14 @@ extern "C" int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* 
 extern "C" int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_k, int Seq_q) {{
   if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return AAT_ERR_SHAPE;
   return (int)launch(q, k, v, o, B, H, Seq_q, Seq_k, kReferenceScale, 0, nullptr, nullptr);
+}}
+extern "C" int kernel_entry_lse(aat_half* q, aat_half* k, aat_half* v, aat_half* o, float* lse, int B, int H, int Seq_q,
+                                int Seq_k, float softmax_scale, int causal, void* workspace, size_t workspace_bytes,
+                                void* stream) {{
+  if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return AAT_ERR_SHAPE;
+  if (split_applies(Seq_k, causal) && (workspace == nullptr || workspace_bytes < split_workspace_bytes(B, H, Seq_q)))
+    return AAT_ERR_WORKSPACE;
+  return (int)launch(q, k, v, o, B, H, Seq_q, Seq_k, softmax_scale, causal, workspace, static_cast<hipStream_t>(stream), lse);
 }}
 """
 

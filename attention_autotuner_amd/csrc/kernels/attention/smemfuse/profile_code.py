@@ -30,14 +30,14 @@ const auto kernel = &aat::flashattn_fwd_smemfuse<Kd, D, Br, Bc, Nthreads, num_st
 const auto kernel_causal = &aat::flashattn_fwd_smemfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, warps_mma1_N, warps_mma_N, waves_per_eu, true>;
 
 hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q, int Seq_k,
-                  float softmax_scale, int causal, hipStream_t stream) {{
+                  float softmax_scale, int causal, hipStream_t stream, float* lse = nullptr) {{
   static const hipError_t lds_ok = aat::allow_lds(kernel, shared_mem);
   static const hipError_t lds_ok_causal = aat::allow_lds(kernel_causal, shared_mem);
   if (lds_ok != hipSuccess) return lds_ok;
   if (lds_ok_causal != hipSuccess) return lds_ok_causal;
   (causal ? kernel_causal : kernel)<<<dim3(B * H * (Seq_q / Br)), dim3(Nthreads), shared_mem, stream>>>(
       reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
-      reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<aat::half_t*>(o), nullptr, H, Seq_k, Seq_q,
+      reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<aat::half_t*>(o), lse, H, Seq_k, Seq_q,
       softmax_scale);
   return hipGetLastError();
 }}
@@ -68,6 +68,11 @@ extern "C" int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* 
 }}
 extern "C" int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_k, int Seq_q) {{
   return kernel_entry_ex(q, k, v, o, B, H, Seq_q, Seq_k, kReferenceScale, 0, nullptr, 0, nullptr);
+}}
+extern "C" int kernel_entry_lse(aat_half* q, aat_half* k, aat_half* v, aat_half* o, float* lse, int B, int H, int Seq_q,
+                                int Seq_k, float softmax_scale, int causal, void*, size_t, void* stream) {{
+  if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return AAT_ERR_SHAPE;
+  return (int)launch(q, k, v, o, B, H, Seq_q, Seq_k, softmax_scale, causal, static_cast<hipStream_t>(stream), lse);
 }}
 """
 

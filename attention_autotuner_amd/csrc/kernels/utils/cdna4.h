@@ -92,11 +92,26 @@ template <int NC> AAT_DEV constexpr int swz_rows4(int row, int c) {
 // writes lane i's data at  lds_base + 16*i  with lds_base wave-uniform.  No VGPR staging; completion is
 // tracked by vmcnt.  A tile of ROWS x (NC*8) halfs is ROWS*NC chunks; thread t of NT copies chunks
 // t, t+NT, ...  Chunk slot s sits at LDS byte 16*s and holds global chunk (row = s/NC, c = SWZ(row, s%NC)).
-enum class Swz { Rows16, Rows4 };
+enum class Swz { Rows16, Rows4, Both };
+
+// swz_both: one tile read BOTH ways (b128 operand reads of 16 consecutive rows and transposing reads of
+// 4 consecutive rows x 4 chunks).  The XOR term must be a bijection of the row bits that a b128 phase
+// walks (so 16 rows of one chunk hit 16 different slots) whose chunk-group bits also change with the two
+// low row bits (so the 4 rows of a transposing phase hit 4 different 64-byte groups).
+template <int NC> AAT_DEV constexpr int swz_both(int row, int c) {
+  if constexpr (NC % 16 == 0) {
+    return c ^ ((row & 15) ^ ((row & 3) << 2));                      // (b3^b1, b2^b0, b1, b0)
+  } else {
+    static_assert(NC == 8, "tiles read both ways are 64 or a multiple of 128 halfs wide");
+    const int b1 = (row >> 1) & 1, b2 = (row >> 2) & 1, b3 = (row >> 3) & 1;
+    return c ^ (((b3 ^ b1) << 2) | (b2 << 1) | b1);                  // two rows share a 256-byte line
+  }
+}
 
 template <int NC, Swz MODE> AAT_DEV constexpr int swz(int row, int c) {
   if constexpr (MODE == Swz::Rows16) return swz_rows16<NC>(row, c);
-  else return swz_rows4<NC>(row, c);
+  else if constexpr (MODE == Swz::Rows4) return swz_rows4<NC>(row, c);
+  else return swz_both<NC>(row, c);
 }
 
 constexpr int cgcd(int a, int b) { return b == 0 ? a : cgcd(b, a % b); }
@@ -123,7 +138,7 @@ struct TileDma {
   static constexpr int kRowBytes = NC * 16;
   static constexpr bool kRegular = (NT % NC == 0);
   static constexpr int kRowsPerIter = kRegular ? NT / NC : 1;
-  static constexpr int kPeriod = (MODE == Swz::Rows16) ? 16 : 4;   // rows after which the swizzle repeats
+  static constexpr int kPeriod = (MODE == Swz::Rows4) ? 4 : 16;    // rows after which the swizzle repeats
   static constexpr int kDistinctRaw = kPeriod / cgcd(kRowsPerIter, kPeriod);
   static constexpr int kDistinct = !kRegular ? kIters : (kDistinctRaw < kIters ? kDistinctRaw : kIters);
   uint32_t loff[kDistinct];                            // per-lane byte offsets inside a tile

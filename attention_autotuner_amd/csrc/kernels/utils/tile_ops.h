@@ -19,22 +19,22 @@ AAT_DEV void load_q_frags(h8 (&qf)[RT][KS], const half_t* qrow) {
 }
 
 // Byte offsets, inside a Rows16-swizzled [rows][Kd] tile, of this lane's A-operand chunks for tile row n.
-template <int KS, int NCK>
+template <int KS, int NCK, Swz MODE = Swz::Rows16>
 AAT_DEV void k_frag_offsets(int (&koff)[KS], int n, int h) {
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) koff[ks] = lds_chunk_off<NCK, Swz::Rows16>(n, 2 * ks + h);
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = lds_chunk_off<NCK, MODE>(n, 2 * ks + h);
 }
 
 // Byte offsets, inside a Rows4-swizzled [rows][D] tile, of the address this lane presents to the
 // transposing read for d-tile dt (kv rows 4h .. 4h+3 of a 16-row step; add 8 rows for the second half).
-template <int DT, int NCV>
+template <int DT, int NCV, Swz MODE = Swz::Rows4>
 AAT_DEV void v_frag_offsets(int (&voff)[DT], int lane) {
   const int h = lane >> 5, s16 = lane & 15;
   const int row = 4 * h + (s16 >> 2);
   const int vcol = 16 * ((lane >> 4) & 1) + 4 * (s16 & 3);
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
-    voff[dt] = lds_chunk_off<NCV, Swz::Rows4>(row, 4 * dt + (vcol >> 3)) + (vcol & 7) * 2;
+    voff[dt] = lds_chunk_off<NCV, MODE>(row, 4 * dt + (vcol >> 3)) + (vcol & 7) * 2;
 }
 
 // One MFMA step of S^T = K Q^T: score tile nt, k-step ks.
@@ -182,6 +182,40 @@ AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const u
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) mfma_settle(sacc[rt][nt]);
+  }
+}
+
+// O^T += V^T P^T over one kv tile.  vlo[dt] / vhi[dt] = LDS addresses this lane presents to the two
+// transposing reads of d-tile dt (kv rows 4h..4h+3 and 8+4h..8+4h+3 of the first 16-row step; later steps
+// add 16 rows, which no swizzle here sees).  pack(g) must fill pf[*][g/2][g%2] (the P operand of kv rows
+// 16g .. 16g+15); it is called one group ahead of use, between MFMAs.
+template <int RT, int NT, int DT, int NCV, int PF, class Pack>
+AAT_DEV void pv_gemm_steps_hl(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint32_t (&vlo)[DT],
+                              const uint32_t (&vhi)[DT], int buf_off, Pack&& pack) {
+  constexpr int G = NT * 2;              // groups of 16 kv rows
+  constexpr int S = G * DT;
+  constexpr int kRow16 = 16 * NCV * 16;
+  h4 lo[PF], hi[PF];
+#pragma unroll
+  for (int i = 0; i < PF && i < S; ++i) {
+    lo[i] = lds_read_tr_h4_at(vlo[i % DT] + buf_off + (i / DT) * kRow16);
+    hi[i] = lds_read_tr_h4_at(vhi[i % DT] + buf_off + (i / DT) * kRow16);
+  }
+  pack(0);
+  sched_fence();
+#pragma unroll
+  for (int step = 0; step < S; ++step) {
+    const int g = step / DT, dt = step % DT;
+    const h8 vf = cat_h4(lo[step % PF], hi[step % PF]);
+    if (step + PF < S) {
+      const int nx = step + PF;
+      lo[step % PF] = lds_read_tr_h4_at(vlo[nx % DT] + buf_off + (nx / DT) * kRow16);
+      hi[step % PF] = lds_read_tr_h4_at(vhi[nx % DT] + buf_off + (nx / DT) * kRow16);
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
+    if (dt == 0 && g + 1 < G) pack(g + 1);
+    sched_fence();
   }
 }
 

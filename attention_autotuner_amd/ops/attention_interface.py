@@ -2,8 +2,11 @@
 
 Drop-in for reference python/ops/attention_interface.py:8-60: same tensor layout ([B, H, S, D] fp16 on
 the GPU), same positional arguments, same asserts on the head sizes, same tune-then-launch flow.
-Additions: ``causal`` is honoured (the reference accepts and ignores it) and ``softmax_scale``
-defaults to 1/sqrt(d_qk) (the reference hard-codes 0.125, available as REFERENCE_SOFTMAX_SCALE).
+Additions: ``causal`` is honoured (the reference accepts and ignores it), ``softmax_scale``
+defaults to 1/sqrt(d_qk) (the reference hard-codes 0.125, available as REFERENCE_SOFTMAX_SCALE), and
+``backward`` is implemented (the reference's is an empty stub, python/ops/attention_interface.py:37-58):
+when any input requires a gradient the forward also stores the log-sum-exp of every row, and the
+backward launches the attention-backward library (dq, dk, dv in fp16, no atomics).
 """
 import math
 
@@ -12,7 +15,7 @@ import torch
 from ..arch import Arch
 from ..autotuner import gfx950_space
 from ..autotuner.runtime import Runtime
-from ..autotuner.tunner import AttnTunner
+from ..autotuner.tunner import AttnBwdTunner, AttnTunner
 from ._resolve import resolve
 
 REFERENCE_SOFTMAX_SCALE = 0.125
@@ -40,14 +43,33 @@ class MultiHeadAttnFunc(torch.autograd.Function):
         o = torch.empty(batch_size, nheads, seqlen_q, head_dim, device=q.device, dtype=q.dtype)
         tuner = AttnTunner(arch=device_type, torch_array=[q, k, v, o], causal=causal, softmax_scale=softmax_scale)
         cc = resolve(tuner, lambda: gfx950_space.default_forward_config("attn", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        Runtime(device_type, cc).apply([q, k, v, o], softmax_scale=softmax_scale, causal=causal)
-        ctx.save_for_backward(q, k, v)
+        needs_grad = any(ctx.needs_input_grad[:3])
+        lse = torch.empty(batch_size, nheads, seqlen_q, device=q.device, dtype=torch.float32) if needs_grad else None
+        Runtime(device_type, cc).apply([q, k, v, o], softmax_scale=softmax_scale, causal=causal, lse=lse)
+        if needs_grad:
+            ctx.save_for_backward(q, k, v, o, lse)
         ctx.device_type = device_type
+        ctx.causal = bool(causal)
+        ctx.softmax_scale = float(softmax_scale)
         return o
 
     @staticmethod
     def backward(ctx, do):
-        raise NotImplementedError("attention backward is not part of this operator (the reference leaves it empty as well)")
+        q, k, v, o, lse = ctx.saved_tensors
+        device_type = ctx.device_type
+        key_dim, head_dim = q.shape[-1], v.shape[-1]
+        seqlen_q, seqlen_k = q.shape[2], k.shape[2]
+        do = do.contiguous()
+        assert do.dtype == torch.float16 and do.shape == o.shape
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        arrays = [q, k, v, o, do, lse, dq, dk, dv]
+        tuner = AttnBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal, softmax_scale=ctx.softmax_scale)
+        try:
+            cc = resolve(tuner, lambda: gfx950_space.default_attn_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+        except (ValueError, RuntimeError) as e:
+            raise NotImplementedError(f"attention backward: {e}") from e
+        Runtime(device_type, cc).apply(arrays, softmax_scale=ctx.softmax_scale, causal=ctx.causal)
+        return dq, dk, dv, None, None, None
 
 
 flash_attn_func = MultiHeadAttnFunc.apply

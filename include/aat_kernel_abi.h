@@ -3,7 +3,7 @@
  * The autotuner turns every candidate configuration (tile sizes, wave count, LDS buffering, fuse
  * type) into its own shared object, exactly as the reference does, and binds it with ctypes.  Each
  * such library exports the symbols declared below for ONE operator; which operator is selected at
- * compile time by defining AAT_OP_ATTN, AAT_OP_RET or AAT_OP_RET_BWD before including this header
+ * compile time by defining AAT_OP_ATTN, AAT_OP_RET, AAT_OP_RET_BWD or AAT_OP_ATTN_BWD before including this header
  * (the generated wrapper does that, so the compiler checks the definitions against this file).
  *
  * Conventions (same as the reference unless stated):
@@ -32,7 +32,7 @@
 
 #include <stddef.h>
 
-#define AAT_ABI_VERSION 1
+#define AAT_ABI_VERSION 2
 #define AAT_ERR_SHAPE (-2)      /* Seq_q / Seq_k not divisible by the tile, or a non-positive size */
 #define AAT_ERR_WORKSPACE (-3)  /* workspace missing or smaller than workspace_size() */
 
@@ -59,6 +59,14 @@ float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int 
 int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int H, int Seq_q,
                     int Seq_k, float softmax_scale, int causal, void* workspace,
                     size_t workspace_bytes, void* stream);
+/* kernel_entry_ex that also writes lse [B,H,Seq_q] fp32, the natural log-sum-exp of the scaled scores of
+ * every query row (-inf for a row with no visible key), which the backward needs.  The reference computes
+ * this value (csrc/kernels/attention/regfuse/regfuse.h:411) but never stores it and declares no such
+ * entry point; its operator's commented-out `ctx.save_for_backward(q, k, v) # , lse)`
+ * (python/ops/attention_interface.py:33) is the call site this serves. */
+int kernel_entry_lse(aat_half* q, aat_half* k, aat_half* v, aat_half* o, float* lse, int B, int H,
+                     int Seq_q, int Seq_k, float softmax_scale, int causal, void* workspace,
+                     size_t workspace_bytes, void* stream);
 
 #elif defined(AAT_OP_RET)
 /* RetNet parallel forward.  Replaces: reference csrc/kernels/retnet/regfuse/profile_code.py:34 and :72
@@ -90,6 +98,20 @@ float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half
 int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
                     aat_half* dq, aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q,
                     int Seq_k, int causal, void* workspace, size_t workspace_bytes, void* stream);
+
+#elif defined(AAT_OP_ATTN_BWD)
+/* Flash-attention backward: dq, dk, dv from q, k, v, o, dO and the forward's lse (see kernel_entry_lse).
+ * No counterpart in the reference, whose MultiHeadAttnFunc.backward is an empty stub
+ * (python/ops/attention_interface.py:37-58, README.md:107); this is the entry point that stub would bind.
+ * Seq_q and Seq_k must both be multiples of the library's Br and Bc.  workspace_size() bytes of
+ * workspace are required (two fp32 values per query row); dq, dk, dv are fully overwritten. */
+float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, aat_half* dO, float* lse,
+                 aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k,
+                 float softmax_scale, int causal, void* workspace, size_t workspace_bytes, void* stream);
+int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, aat_half* dO, float* lse,
+                    aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k,
+                    float softmax_scale, int causal, void* workspace, size_t workspace_bytes,
+                    void* stream);
 #endif
 
 #ifdef __cplusplus

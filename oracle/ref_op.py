@@ -8,6 +8,10 @@ reference uses as its own correctness check:
 * ``attention_ref``   follows reference python/utils/ref_op.py:2-6  (``softmax(q k^T * scale) v``); the
   reference hard-codes scale = 0.125, here it is an argument (``None`` -> 1/sqrt(d_qk)) and a causal
   lower-triangular mask (aligned to the bottom-right corner when S_q != S_kv) can be applied.
+* ``attention_bwd_ref`` is the closed form of the attention gradients (the reference declares the
+  operator, python/ops/attention_interface.py:37-58, and leaves it empty): with ``P = softmax(S)``,
+  ``delta = rowsum(dO * O)``: ``dV = P^T dO``, ``dS = P * (dO V^T - delta)``, ``dK = scale dS^T Q``,
+  ``dQ = scale dS K``; pinned by autograd through ``attention_ref`` and fp64 gradcheck.
 * ``retnet_ref``      follows reference python/utils/ref_op.py:8-13 (``S = q k^T * mask``,
   ``r = clamp(sum|S|, min=1)`` detached, ``o = (S / r) v``) and also returns ``r``.
 * ``retnet_bwd_ref``  is the closed form the backward kernel evaluates, reference
@@ -53,6 +57,26 @@ def attention_ref(q, k, v, softmax_scale=None, causal=False, return_lse=False):
     p = torch.nan_to_num(p, nan=0.0)  # rows with no visible kv produce 0, not NaN
     o = p @ v
     return (o, lse) if return_lse else o
+
+
+def attention_bwd_ref(q, k, v, do, softmax_scale=None, causal=False, o=None, lse=None):
+    """Gradients of ``attention_ref`` w.r.t. q, k, v.  ``o`` / ``lse`` (as a forward kernel stored them) are
+    used for delta and P when given, otherwise recomputed."""
+    q, k, v, do = _f32(q), _f32(k), _f32(v), _f32(do)
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(q.shape[-1])
+    s = (q @ k.transpose(-1, -2)) * softmax_scale
+    if causal:
+        s = s.masked_fill(~causal_allowed(q.shape[-2], k.shape[-2]), float("-inf"))
+    lse = torch.logsumexp(s, dim=-1) if lse is None else _f32(lse)
+    p = torch.nan_to_num(torch.exp(s - lse.unsqueeze(-1)), nan=0.0, posinf=0.0)
+    o = p @ v if o is None else _f32(o)
+    delta = (do * o).sum(dim=-1, keepdim=True)
+    dv = p.transpose(-1, -2) @ do
+    ds = p * (do @ v.transpose(-1, -2) - delta)
+    dk = (ds.transpose(-1, -2) @ q) * softmax_scale
+    dq = (ds @ k) * softmax_scale
+    return dq, dk, dv
 
 
 def retnet_ref(q, k, v, mask, return_r=False):

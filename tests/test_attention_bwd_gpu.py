@@ -1,0 +1,132 @@
+"""GPU parity of the attention backward (dq, dk, dv) against the CPU oracle, through the operator and
+through the C ABI.
+
+Tolerance: |err| <= 2e-3 + 1e-3 * |ref| on fp16 gradients versus the fp32 oracle on the same seeded
+inputs (a gradient entry above 4 in magnitude has half an fp16 ulp of 2e-3 already); the forward's
+log-sum-exp is compared at 1e-3 absolute.
+"""
+import ctypes
+import math
+
+import pytest
+import torch
+
+import attention_autotuner_amd as aat
+from attention_autotuner_amd.arch import MI355X
+from attention_autotuner_amd.autotuner import Runtime, codegen, gfx950_space, library, prebuilt
+from attention_autotuner_amd.autotuner.configs import AttnBwdConfig
+from oracle import ref_op
+
+pytestmark = pytest.mark.gpu
+ARCH = MI355X()
+
+
+def _inputs(b, h, sq, sk, dqk, dv, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(b, h, sq, dqk, generator=g).half()
+    k = torch.randn(b, h, sk, dqk, generator=g).half()
+    v = torch.randn(b, h, sk, dv, generator=g).half()
+    do = torch.randn(b, h, sq, dv, generator=g).half()
+    return q, k, v, do
+
+
+def _close(got, ref):
+    err = (got.float().cpu() - ref).abs()
+    return bool((err <= 2e-3 + 1e-3 * ref.abs()).all()), err.max().item()
+
+
+def _op_grads(q, k, v, do, causal, scale=None):
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = aat.flash_attn_func(qc, kc, vc, ARCH, causal, scale)
+    o.backward(do.cuda())
+    return o, qc.grad, kc.grad, vc.grad
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dqk,dv", prebuilt.ATTN_BWD_DIMS)
+@pytest.mark.parametrize("sq,sk", [(256, 256), (128, 384), (384, 128)])
+def test_operator_backward_matches_oracle(dqk, dv, sq, sk, causal):
+    q, k, v, do = _inputs(2, 3, sq, sk, dqk, dv, seed=sq + dqk)
+    o, dq, dk, dv_ = _op_grads(q, k, v, do, causal)
+    ref = ref_op.attention_bwd_ref(q, k, v, do, None, causal)
+    for name, g, r in zip(("dq", "dk", "dv"), (dq, dk, dv_), ref):
+        ok, worst = _close(g, r)
+        assert ok, (name, worst)
+
+
+def test_forward_lse_entry_matches_oracle():
+    q, k, v, _ = _inputs(1, 4, 256, 512, 128, 128, seed=3)
+    for causal in (False, True):
+        cfg = gfx950_space.default_forward_config("attn", 128, 128, ARCH, 256, 512)
+        o = torch.empty(1, 4, 256, 128, dtype=torch.float16, device="cuda")
+        lse = torch.empty(1, 4, 256, dtype=torch.float32, device="cuda")
+        Runtime(ARCH, cfg).apply([q.cuda(), k.cuda(), v.cuda(), o], causal=causal, lse=lse)
+        ref_o, ref_lse = ref_op.attention_ref(q, k, v, None, causal, return_lse=True)
+        assert (lse.cpu() - ref_lse).abs().max().item() <= 1e-3
+        assert (o.float().cpu() - ref_o).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_config2_backward_b4_h32_s2048_d128(causal):
+    q, k, v, do = _inputs(4, 32, 2048, 2048, 128, 128, seed=1)
+    o, dq, dk, dv_ = _op_grads(q, k, v, do, causal)
+    for b, h in ((0, 0), (2, 17), (3, 31)):          # (batch, head) slices are independent
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = ref_op.attention_bwd_ref(q[sl], k[sl], v[sl], do[sl], None, causal)
+        for name, g, r in zip(("dq", "dk", "dv"), (dq[sl], dk[sl], dv_[sl]), ref):
+            ok, worst = _close(g, r)
+            assert ok, (name, b, h, worst)
+    # size-independent properties on the whole problem: rows of dS sum to zero, so with K := 1 dQ vanishes;
+    # and the gradients are linear in dO
+    ones = torch.ones_like(k)
+    _, dq1, _, _ = _op_grads(q, ones, v, do, causal)
+    assert dq1.float().abs().max().item() <= 2e-3
+    _, dq2, dk2, dv2 = _op_grads(q, k, v, (2 * do.float()).half(), causal)
+    for g1, g2 in ((dq, dq2), (dk, dk2), (dv_, dv2)):
+        assert (2 * g1.float() - g2.float()).abs().max().item() <= 4e-3 + 2e-3 * g2.float().abs().max().item()
+
+
+@pytest.mark.parametrize("br,bc,nt,st", prebuilt.ATTN_BWD_TILES)
+def test_tile_variants_agree(br, bc, nt, st):
+    q, k, v, do = _inputs(1, 2, 256, 256, 128, 128, seed=5)
+    o_ref, lse_ref = ref_op.attention_ref(q, k, v, 0.11, True, return_lse=True)
+    cfg = AttnBwdConfig(br, bc, 128, 128, nt, st)
+    assert gfx950_space.attn_backward_valid(cfg, ARCH)
+    arrays = [t.cuda() for t in (q, k, v, o_ref.half(), do, lse_ref)]
+    grads = [torch.empty_like(arrays[0]), torch.empty_like(arrays[1]), torch.empty_like(arrays[2])]
+    Runtime(ARCH, cfg).apply(arrays + grads, softmax_scale=0.11, causal=True)
+    ref = ref_op.attention_bwd_ref(q, k, v, do, 0.11, True)
+    for name, g, r in zip(("dq", "dk", "dv"), grads, ref):
+        ok, worst = _close(g, r)
+        assert ok, (cfg, name, worst)
+
+
+def test_abi_error_paths_and_stream():
+    cfg = gfx950_space.default_attn_backward_config(128, 128, ARCH, 128, 128)
+    lib = library.load(codegen.compile_config(cfg, ARCH), "attn_bwd")
+    q, k, v, do = (t.cuda() for t in _inputs(1, 1, 256, 256, 128, 128, seed=7))
+    o = torch.zeros_like(do)
+    lse = torch.zeros(1, 1, 256, device="cuda")
+    dq, dk, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    ptrs = [ctypes.c_void_p(t.data_ptr()) for t in (q, k, v, o, do, lse, dq, dk, dv_)]
+    null = ctypes.c_void_p(0)
+    # no workspace -> AAT_ERR_WORKSPACE; indivisible length -> AAT_ERR_SHAPE; nothing is launched in either case
+    assert lib.kernel_entry_ex(*ptrs, 1, 1, 256, 256, ctypes.c_float(0.1), 0, null, ctypes.c_size_t(0), null) == -3
+    ws = torch.empty(lib.workspace_size(1, 1, 256, 256), dtype=torch.uint8, device="cuda")
+    wsp, wsn = ctypes.c_void_p(ws.data_ptr()), ctypes.c_size_t(ws.numel())
+    assert lib.kernel_entry_ex(*ptrs, 1, 1, 200, 256, ctypes.c_float(0.1), 0, wsp, wsn, null) == -2
+    assert lib.profile_ex(*ptrs, 1, 1, 256, 256, ctypes.c_float(0.1), 0, null, ctypes.c_size_t(0), null) == -1.0
+    # launches on the stream it is given
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        rc = lib.kernel_entry_ex(*ptrs, 1, 1, 256, 256, ctypes.c_float(0.1), 0, wsp, wsn, ctypes.c_void_p(side.cuda_stream))
+    side.synchronize()
+    assert rc == 0 and torch.isfinite(dq.float()).all()
+
+
+def test_unsupported_head_sizes_say_so():
+    q, k, v, do = _inputs(1, 1, 128, 128, 256, 256, seed=9)
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = aat.flash_attn_func(qc, kc, vc, ARCH)
+    with pytest.raises(NotImplementedError):
+        o.backward(do.cuda())

@@ -28,9 +28,12 @@ def _declared_symbols(op_macro):
 
 
 def test_header_declares_the_reference_pair_for_every_operator():
-    for macro in ("AAT_OP_ATTN", "AAT_OP_RET", "AAT_OP_RET_BWD"):
-        names = _declared_symbols(macro)
-        assert names == ["abi_version", "config_string", "kernel_entry", "kernel_entry_ex", "profile", "profile_ex", "workspace_size"]
+    pair = ["abi_version", "config_string", "kernel_entry", "kernel_entry_ex", "profile", "profile_ex", "workspace_size"]
+    assert _declared_symbols("AAT_OP_ATTN") == sorted(pair + ["kernel_entry_lse"])
+    for macro in ("AAT_OP_RET", "AAT_OP_RET_BWD"):
+        assert _declared_symbols(macro) == pair
+    # the attention backward has no reference signature to keep: only the extended entry points
+    assert _declared_symbols("AAT_OP_ATTN_BWD") == ["abi_version", "config_string", "kernel_entry_ex", "profile_ex", "workspace_size"]
 
 
 def test_wrapper_text_carries_the_configuration():
@@ -48,7 +51,8 @@ def test_wrapper_text_carries_the_configuration():
 def test_shipping_set_is_built_and_exports_the_abi():
     cfgs = prebuilt.shipping_set(ARCH)
     assert cfgs
-    macro = {"attn": "AAT_OP_ATTN", "ret": "AAT_OP_RET", "ret_bwd": "AAT_OP_RET_BWD"}
+    macro = {"attn": "AAT_OP_ATTN", "ret": "AAT_OP_RET", "ret_bwd": "AAT_OP_RET_BWD", "attn_bwd": "AAT_OP_ATTN_BWD"}
+    assert {c.operation for c in cfgs} == set(macro)
     for cfg in cfgs:
         path = codegen.compile_config(cfg, ARCH, timeout=600)          # already built by build(); builds if not
         assert path and os.path.exists(path), cfg
@@ -56,9 +60,11 @@ def test_shipping_set_is_built_and_exports_the_abi():
         for name in _declared_symbols(macro[cfg.operation]):
             assert hasattr(raw, name), (cfg, name)
         lib = library.load(path, cfg.operation)
-        assert lib.abi_version() == 1
+        assert lib.abi_version() == 2
         assert lib.config_string().decode() == f"{cfg.operation}:{cfg}"
-        if getattr(cfg, "kv_splits", 1) == 1:
+        if cfg.operation == "attn_bwd":
+            assert lib.workspace_size(2, 3, 256, 512) == 2 * 2 * 3 * 256 * 4      # lse2 + delta, fp32 per query row
+        elif getattr(cfg, "kv_splits", 1) == 1:
             assert lib.workspace_size(1, 1, 256, 256) == 0
 
 

@@ -190,3 +190,61 @@ def test_retnet_bwd_linearity_and_zero_mask():
         torch.testing.assert_close(2 * a - 3 * b, c, rtol=1e-4, atol=1e-4)
     for g in ref_op.retnet_bwd_ref(q, k, v, torch.zeros_like(mask), d1):
         assert g.abs().max() == 0
+
+
+# ---------------------------------------------------------------------------------- attention backward
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("sq,sk", [(8, 8), (6, 10)])
+def test_attention_bwd_matches_autograd_through_sdpa(causal, sq, sk):
+    """Independent route: autograd through torch's own scaled_dot_product_attention in fp64."""
+    q, k, v = _rand(2, 2, sq, 64, seed=51), _rand(2, 2, sk, 64, seed=52), _rand(2, 2, sk, 128, seed=53)
+    do = _rand(2, 2, sq, 128, seed=54)
+    scale = 0.2
+    qq, kk, vv = (t.double().clone().requires_grad_(True) for t in (q, k, v))
+    allowed = ref_op.causal_allowed(sq, sk) if causal else None
+    out = F.scaled_dot_product_attention(qq, kk, vv, attn_mask=allowed, scale=scale)
+    out.backward(do.double())
+    got = ref_op.attention_bwd_ref(q, k, v, do, scale, causal)
+    for g, w in zip(got, (qq.grad, kk.grad, vv.grad)):
+        torch.testing.assert_close(g, w.float(), rtol=1e-4, atol=1e-4)
+
+
+def test_attention_bwd_gradcheck_fp64_and_stored_forward():
+    g = torch.Generator().manual_seed(55)
+    q, k, v = (torch.randn(1, 1, 4, 6, generator=g, dtype=torch.float64) for _ in range(3))
+    do = torch.randn(1, 1, 4, 6, generator=g, dtype=torch.float64)
+
+    def f(qq, kk, vv):
+        return torch.softmax((qq @ kk.transpose(-1, -2)) * 0.3, dim=-1) @ vv
+
+    assert torch.autograd.gradcheck(f, tuple(t.clone().requires_grad_(True) for t in (q, k, v)), eps=1e-6, atol=1e-6)
+    want = torch.autograd.grad(f(*(t.requires_grad_(True) for t in (q, k, v))), (q, k, v), do)
+    got = ref_op.attention_bwd_ref(q, k, v, do, 0.3)
+    for a, b in zip(got, want):
+        torch.testing.assert_close(a, b.float(), rtol=1e-4, atol=1e-4)
+    # the o / lse a forward kernel stored reproduce the same gradients as the recomputed ones
+    o, lse = ref_op.attention_ref(q, k, v, 0.3, return_lse=True)
+    again = ref_op.attention_bwd_ref(q, k, v, do, 0.3, o=o, lse=lse)
+    for a, b in zip(got, again):
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-5)
+
+
+def test_attention_bwd_closed_forms():
+    q, k, v = _rand(1, 2, 8, 64, seed=56), _rand(1, 2, 8, 64, seed=57), _rand(1, 2, 8, 64, seed=58)
+    d1, d2 = _rand(1, 2, 8, 64, seed=59), _rand(1, 2, 8, 64, seed=60)
+    # linear in dO
+    g1, g2 = ref_op.attention_bwd_ref(q, k, v, d1.float()), ref_op.attention_bwd_ref(q, k, v, d2.float())
+    g12 = ref_op.attention_bwd_ref(q, k, v, 2 * d1.float() - 3 * d2.float())
+    for a, b, c in zip(g1, g2, g12):
+        torch.testing.assert_close(2 * a - 3 * b, c, rtol=1e-4, atol=1e-4)
+    # scale 0: P is uniform, so dQ = dK = 0 and every dV row is the mean of dO
+    dq, dk, dv = ref_op.attention_bwd_ref(q, k, v, d1, 0.0)
+    assert dq.abs().max() == 0 and dk.abs().max() == 0
+    torch.testing.assert_close(dv, d1.float().mean(dim=-2, keepdim=True).expand_as(dv), rtol=1e-5, atol=1e-5)
+    # softmax rows sum to one, so dS rows sum to zero: a shift of every key by one vector leaves dQ's
+    # projection on that vector unchanged -> sum over kv of dS is 0  <=>  dQ computed with K := 1 vanishes
+    dq1, _, _ = ref_op.attention_bwd_ref(q, torch.ones_like(k), v, d1)
+    assert dq1.abs().max() < 1e-5
+    # causal, first query row sees one key: P = 1 there, so dS = P (dP - delta) = 0 and dQ[0] = 0
+    dqc, _, dvc = ref_op.attention_bwd_ref(q, k, v, d1, None, True)
+    assert dqc[..., 0, :].abs().max() < 1e-6
