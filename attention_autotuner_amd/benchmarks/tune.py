@@ -4,6 +4,7 @@ python/tests/attntuner_demo.py:186-192 and python/tests/test_retbwdtunner.py:88-
     python -m attention_autotuner_amd.benchmarks.tune attn    B H Sq Sk dqk dv [--causal] [--compile-only]
     python -m attention_autotuner_amd.benchmarks.tune ret     B H Sq Sk dqk dv [--causal]
     python -m attention_autotuner_amd.benchmarks.tune ret_bwd B H Sq Sk dqk dv [--causal]
+    python -m attention_autotuner_amd.benchmarks.tune attn_bwd B H Sq Sk dqk dv [--causal]
 
 Writes the best configuration into the tuning cache, the per-candidate log next to it, and prints a
 one-line JSON summary.  ``--compile-only`` builds every candidate library (no GPU needed) so that a
@@ -20,6 +21,7 @@ import torch
 
 from ..arch import MI355X
 from ..autotuner import AttnTunner, RetBwdTunner, RetTunner, codegen
+from ..autotuner.tunner import AttnBwdTunner
 from ..ops._resolve import DEFAULT_LOG_DIR
 
 
@@ -36,6 +38,13 @@ def make_tensors(op, b, h, sq, sk, dqk, dv, device, seed=0):
     q, k, v = mk(b, h, sq, dqk), mk(b, h, sk, dqk), mk(b, h, sk, dv)
     if op == "attn":
         return [q, k, v, torch.empty(b, h, sq, dv, dtype=torch.float16, device=device)]
+    if op == "attn_bwd":
+        # timing only: any finite o and a log-sum-exp of the right magnitude (log S_kv) will do
+        o, do = mk(b, h, sq, dv), mk(b, h, sq, dv)
+        lse = torch.empty(b, h, sq, dtype=torch.float32, device=device)
+        if device != "meta":
+            lse.fill_(math.log(sk))
+        return [q, k, v, o, do, lse, torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)]
     n = torch.arange(sq, dtype=torch.float64).view(1, sq, 1)
     m = torch.arange(sk, dtype=torch.float64).view(1, 1, sk)
     gamma = (1.0 - torch.pow(2.0, -5.0 - torch.arange(h, dtype=torch.float64))).view(h, 1, 1)
@@ -54,13 +63,13 @@ def make_tensors(op, b, h, sq, sk, dqk, dv, device, seed=0):
 
 
 def flops(op, b, h, sq, sk, dqk, dv, causal):
-    f = 2.0 * b * h * sq * sk * ((dqk + dv) if op != "ret_bwd" else (3 * dqk + 2 * dv))
-    return f / 2 if (causal and op == "attn") else f
+    f = 2.0 * b * h * sq * sk * ((dqk + dv) if op in ("attn", "ret") else (3 * dqk + 2 * dv))
+    return f / 2 if (causal and op in ("attn", "attn_bwd")) else f
 
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("op", choices=["attn", "ret", "ret_bwd"])
+    ap.add_argument("op", choices=["attn", "ret", "ret_bwd", "attn_bwd"])
     ap.add_argument("dims", type=int, nargs=6, metavar="N", help="B H Sq Sk dqk dv")
     ap.add_argument("--causal", action="store_true")
     ap.add_argument("--compile-only", action="store_true")
@@ -68,7 +77,7 @@ def main(argv=None):
     args = ap.parse_args(argv)
     b, h, sq, sk, dqk, dv = args.dims
     arch = MI355X()
-    cls = {"attn": AttnTunner, "ret": RetTunner, "ret_bwd": RetBwdTunner}[args.op]
+    cls = {"attn": AttnTunner, "ret": RetTunner, "ret_bwd": RetBwdTunner, "attn_bwd": AttnBwdTunner}[args.op]
     device = "meta" if args.compile_only else "cuda"
     arrays = make_tensors(args.op, b, h, sq, sk, dqk, dv, device)
     tuner = cls(arch, arrays, causal=args.causal)

@@ -197,8 +197,24 @@ def side_measurements(aat, arch, Runtime, mk, steps, warmup):
     res["attn_longkv_b1h32q256k16384d128"] = {"ms": round(ms, 5), "tflops": round(attn_flops(1, 32, 256, 16384, D, D) / ms / 1e9, 1),
                                               "gbps": round(bytes5 / ms / 1e6, 1), "config": str(cfg5)}
     log(f"attention fwd long-kv: {ms:.4f} ms -> {res['attn_longkv_b1h32q256k16384d128']}")
+    res.update(attention_backward_measurement(aat, arch, mk, steps, warmup))
     res.update(retnet_measurements(aat, arch, mk, steps, warmup))
     return res
+
+
+def attention_backward_measurement(aat, arch, mk, steps, warmup):
+    """Forward + backward of the headline problem through the operator (autograd), non-causal."""
+    q, k, v, do = (mk(B, H, S, D) for _ in range(4))
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    fwd, bwd = attn_flops(B, H, S, S, D, D), 2.0 * B * H * S * S * (3 * D + 2 * D)
+
+    def fb():
+        q.grad = k.grad = v.grad = None
+        aat.flash_attn_func(q, k, v, arch).backward(do)
+
+    _, ms = time_launches(fb, steps, warmup)
+    log(f"attention fwd+bwd: {ms:.4f} ms -> {(fwd + bwd) / ms / 1e9:.1f} TFLOP/s")
+    return {"attn_fwd_bwd_b4h32s2048d128": {"ms": round(ms, 5), "tflops": round((fwd + bwd) / ms / 1e9, 1)}}
 
 
 def retnet_measurements(aat, arch, mk, steps, warmup):
