@@ -281,8 +281,11 @@ def attn_backward_reg_estimate(cfg):
     rt = cfg.Br // _waves(cfg) // MFMA_M
     nt = cfg.Bc // 32
     vec = rt * ((cfg.Kd + cfg.D) // 16) * 4 + rt * nt * 16 + 72
-    acc = rt * ((cfg.Kd + cfg.D) // 32) * 16 + rt * nt * 32
-    return vec, acc
+    acc = rt * ((cfg.Kd + cfg.D) // 32) * 16                # dV + dK accumulators
+    scores = rt * nt * 32                                    # S and dP tiles
+    if cfg.waves_per_eu == 1 and acc + scores > 256:        # the kernel then keeps the score tiles in vector registers
+        return vec + scores - rt * nt * 16, acc
+    return vec, acc + scores
 
 
 def attn_backward_valid(cfg, arch):

@@ -36,7 +36,7 @@ PARITY_TILES = [
 PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
 
 
-ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (256, 128)]
+ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (256, 128), (256, 256)]
 # (Br, Bc, Nthreads, buffers) variants of the attention backward at 128/128 for the parity suite
 ATTN_BWD_TILES = [(64, 32, 128, 2), (64, 64, 128, 2), (128, 64, 256, 3), (128, 32, 256, 2)]
 

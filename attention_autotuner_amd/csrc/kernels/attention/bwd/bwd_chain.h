@@ -253,9 +253,11 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
     }
 
     // first contractions: s = Y1 X1^T (scores), p = Y2 X2^T (dP), both transposed (lane owns resident row)
+    // the score tiles accumulate in vector registers when the outputs alone fill the accumulation registers
+    constexpr bool kVacc = WPE == 1 && RT * ((COL ? DT : 0) + KT + 2 * NT) * 16 > 256;
     f16v s[RT][NT], dp[RT][NT];
-    qk_gemm_steps<RT, NT, KS, NCK, PF>(s, x1f, y1addr, off, [](int) {});
-    qk_gemm_steps<RT, NT, DS, NCD, PF>(dp, x2f, y2addr, off, [](int) {});
+    qk_gemm_steps<RT, NT, KS, NCK, PF, kVacc>(s, x1f, y1addr, off, [](int) {});
+    qk_gemm_steps<RT, NT, DS, NCD, PF, kVacc>(dp, x2f, y2addr, off, [](int) {});
 
     // P = exp2(s*c2 - lse2[q]),  dS = P * (dP - delta[q]);  register v of tile t is streamed row 32t + 8(v/4) + 4h + v%4
     const bool diag_tile = causal && (COL ? (x0 + BX - 1 > j * BY + diag) : ((j + 1) * BY - 1 > x0 + diag));

@@ -114,6 +114,46 @@ template <int NC, Swz MODE> AAT_DEV constexpr int swz(int row, int c) {
   else return swz_both<NC>(row, c);
 }
 
+// Compile-time proof that the swizzles do what they are for.  LDS serves 256 bytes per cycle: the 16
+// lanes of a b128 phase (16 consecutive rows, one logical chunk) and the 32 lanes of a transposing b64
+// phase (4 consecutive rows x 4 consecutive chunks) must each touch 16 different 16-byte slots mod 256.
+template <int NC, Swz MODE> constexpr bool b128_phase_conflict_free() {
+  for (int r0 = 0; r0 < 32; r0 += 16)
+    for (int c = 0; c < NC; ++c) {
+      unsigned seen = 0;
+      for (int i = 0; i < 16; ++i) {
+        const unsigned slot = ((r0 + i) * NC + swz<NC, MODE>(r0 + i, c)) % 16;
+        if (seen >> slot & 1u) return false;
+        seen |= 1u << slot;
+      }
+    }
+  return true;
+}
+template <int NC, Swz MODE> constexpr bool transposing_phase_conflict_free() {
+  for (int r0 = 0; r0 < 32; r0 += 4)
+    for (int g = 0; g < NC / 4; ++g) {
+      unsigned seen = 0;
+      for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j) {
+          const unsigned slot = ((r0 + i) * NC + swz<NC, MODE>(r0 + i, 4 * g + j)) % 16;
+          if (seen >> slot & 1u) return false;
+          seen |= 1u << slot;
+        }
+    }
+  return true;
+}
+static_assert(b128_phase_conflict_free<8, Swz::Rows16>() && b128_phase_conflict_free<16, Swz::Rows16>() &&
+              b128_phase_conflict_free<32, Swz::Rows16>() && b128_phase_conflict_free<64, Swz::Rows16>(),
+              "operand reads of 64/128/256/512-wide tiles are conflict-free");
+static_assert(transposing_phase_conflict_free<8, Swz::Rows4>() && transposing_phase_conflict_free<16, Swz::Rows4>() &&
+              transposing_phase_conflict_free<24, Swz::Rows4>() && transposing_phase_conflict_free<32, Swz::Rows4>() &&
+              transposing_phase_conflict_free<64, Swz::Rows4>(),
+              "transposing reads of 64..512-wide tiles are conflict-free");
+static_assert(b128_phase_conflict_free<8, Swz::Both>() && transposing_phase_conflict_free<8, Swz::Both>() &&
+              b128_phase_conflict_free<16, Swz::Both>() && transposing_phase_conflict_free<16, Swz::Both>() &&
+              b128_phase_conflict_free<32, Swz::Both>() && transposing_phase_conflict_free<32, Swz::Both>(),
+              "tiles read both ways (64/128/256 wide) are conflict-free for both access patterns");
+
 constexpr int cgcd(int a, int b) { return b == 0 ? a : cgcd(b, a % b); }
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order.

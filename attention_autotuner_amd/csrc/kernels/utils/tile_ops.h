@@ -37,49 +37,8 @@ AAT_DEV void v_frag_offsets(int (&voff)[DT], int lane) {
     voff[dt] = lds_chunk_off<NCV, MODE>(row, 4 * dt + (vcol >> 3)) + (vcol & 7) * 2;
 }
 
-// One MFMA step of S^T = K Q^T: score tile nt, k-step ks.
-template <int RT, int NT, int KS, int NCK>
-AAT_DEV void qk_step(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const char* ktile, const int (&koff)[KS],
-                     int nt, int ks) {
-  const h8 kf = lds_read_h8(ktile + nt * 32 * NCK * 16 + koff[ks]);
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) sacc[rt][nt] = mfma_32x32x16(kf, qf[rt][ks], sacc[rt][nt]);
-}
-
-template <int RT, int NT, int KS, int NCK>
-AAT_DEV void qk_gemm(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const char* ktile, const int (&koff)[KS]) {
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) sacc[rt][nt] = zero16();
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qk_step<RT, NT, KS, NCK>(sacc, qf, ktile, koff, nt, ks);
-}
-
-// O^T += V^T P^T over one kv tile.  pf[rt][nt][s] is the fp16 P operand for kv rows 32*nt + 16*s ..+15.
-template <int RT, int NT, int DT, int NCV>
-AAT_DEV void pv_gemm(f16v (&oacc)[RT][DT], const h8 (&pf)[RT][NT][2], const char* vtile, const int (&voff)[DT]) {
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const char* vrow = vtile + (32 * nt + 16 * s) * NCV * 16;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const h4 lo = lds_read_tr_h4(vrow + voff[dt]);
-        const h4 hi = lds_read_tr_h4(vrow + 8 * NCV * 16 + voff[dt]);
-        const h8 vf = cat_h4(lo, hi);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][nt][s], oacc[rt][dt]);
-      }
-    }
-  }
-}
-
 // ---------------------------------------------------------------------------------------------------
-// Explicitly scheduled variants.  The compiler's own ordering of ds_read / MFMA / VALU leaves the
+// Explicitly scheduled contractions.  The compiler's own ordering of ds_read / MFMA / VALU leaves the
 // first MFMA chain waiting on every LDS read and clusters vector work away from the matrix work, so
 // the two contractions below are written as a sequence of steps -- prefetch the operand PF steps
 // ahead, one MFMA group, a slice of caller-supplied vector work -- with a scheduling barrier after

@@ -125,7 +125,7 @@ def test_abi_error_paths_and_stream():
 
 
 def test_unsupported_head_sizes_say_so():
-    q, k, v, do = _inputs(1, 1, 128, 128, 256, 256, seed=9)
+    q, k, v, do = _inputs(1, 1, 128, 128, 256, 512, seed=9)
     qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
     o = aat.flash_attn_func(qc, kc, vc, ARCH)
     with pytest.raises(NotImplementedError):
