@@ -117,7 +117,9 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
   const int Tx = seq_x / BX;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = tile / Tx;
-  const int x0 = (tile % Tx) * BX;
+  int xb = tile % Tx;
+  if (causal && !COL) xb = Tx - 1 - xb;           // query blocks near the end walk the most kv tiles: start them first
+  const int x0 = xb * BX;
   const int diag = seq_k - seq_q;                 // causal: score (q, kv) is kept when kv <= q + diag
   int j_begin = 0, j_end = seq_y / BY;
   if (causal) {

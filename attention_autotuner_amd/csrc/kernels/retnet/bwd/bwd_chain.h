@@ -95,7 +95,9 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   const int Tx = seq_x / BX;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = tile / Tx;
-  const int x0 = (tile % Tx) * BX;
+  int xb = tile % Tx;
+  if (causal && !COL) xb = Tx - 1 - xb;           // query blocks near the end walk the most kv tiles: start them first
+  const int x0 = xb * BX;
   const int dz0 = blockIdx.y * DZB;               // first output column of this block
   const int diag = seq_k - seq_q;                 // mask[q][kv] may be non-zero only for kv <= q + diag
   int j_begin = 0, j_end = seq_y / BY;
