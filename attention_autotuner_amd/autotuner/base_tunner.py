@@ -9,7 +9,9 @@ an on-disk cache first -- with these deliberate changes:
   the reference's ``best_config_{op}_{dqk}_{dv}.json`` name is still read as a fallback;
 * a configuration whose compile fails or times out is skipped (the reference dereferences None);
 * timing calls ``profile_ex`` on the caller's stream with the caller's softmax scale / causal flag;
-* compiled libraries are kept (content-addressed), so a later ``Runtime`` reuses the tuned binary.
+* compiled libraries are kept (content-addressed), so a later ``Runtime`` reuses the tuned binary;
+* the winner is run once and compared with plain torch math on the GPU before it is cached; a library
+  that is fast but wrong is discarded and the next fastest is tried (``AAT_TUNE_VERIFY=0`` skips this).
 """
 import ctypes
 import json
@@ -19,7 +21,7 @@ import time
 
 import torch
 
-from . import codegen, library
+from . import codegen, library, verify
 from .configs import supported_configs
 
 _PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
@@ -118,6 +120,23 @@ class BaseTunner:
                             ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
         return FAILED if ms < 0 else float(ms)
 
+    def verify(self, libname):
+        """Run ``libname`` once on this tuner's tensors and compare its outputs with torch math."""
+        if not hasattr(self, "_reference"):
+            scale = None if len(self._ex_args()) == 1 else self._ex_args()[0].value
+            self._reference = verify.reference_outputs(self.operation, self.torch_array, scale, self.causal)
+        lib = library.load(libname, self.operation)
+        s = self.problem_shape
+        need = lib.workspace_size(s["B"], s["H"], s["Sq"], s["Sk"])
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=self.torch_array[0].device) if need else None
+        for idx in self._reference:
+            self.torch_array[idx].zero_()
+        ptrs = [ctypes.c_void_p(t.data_ptr()) for t in self.torch_array]
+        rc = lib.kernel_entry_ex(*ptrs, s["B"], s["H"], s["Sq"], s["Sk"], *self._ex_args(),
+                                 ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
+        torch.cuda.synchronize()
+        return rc == 0 and verify.outputs_match(self.torch_array, self._reference)
+
     # ---- cache -----------------------------------------------------------------------------------------
     def _cache_file(self):
         k, s = self.problem_key, self.problem_shape
@@ -179,8 +198,18 @@ class BaseTunner:
             timings[res.config] = ms
             if ms < best_ms:
                 best, best_ms = res.config, ms
+        if best is not None and os.environ.get("AAT_TUNE_VERIFY", "1") != "0":
+            libs = {res.config: res.lib_name for res in results}
+            best = None
+            for cfg in sorted((c for c, ms in timings.items() if ms < FAILED), key=timings.get):
+                if self.verify(libs[cfg]):
+                    best, best_ms = cfg, timings[cfg]
+                    break
+                timings[cfg] = FAILED                     # fast but wrong: never cache it
+                if self.verbose:
+                    print("output mismatch, discarded:", cfg)
         if best is None:
-            raise RuntimeError(f"every {self.op_name} candidate failed to compile or run")
+            raise RuntimeError(f"every {self.op_name} candidate failed to compile, run or verify")
         elapsed = time.time() - started
         if self.verbose:
             print("#" * 58)

@@ -1,0 +1,80 @@
+"""The tuning loop on the GPU: times prebuilt candidates, checks the winner against torch math before
+caching it, and discards a candidate whose output is wrong (nothing is compiled inside these tests:
+the candidate lists are restricted to libraries of the shipping set)."""
+import json
+import os
+
+import pytest
+import torch
+
+from attention_autotuner_amd.arch import MI355X
+from attention_autotuner_amd.autotuner import AttnConfig, AttnTunner, RetBwdTunner, codegen, gfx950_space, prebuilt, verify
+from attention_autotuner_amd.autotuner.tunner import AttnBwdTunner
+from attention_autotuner_amd.benchmarks.tune import make_tensors
+
+pytestmark = pytest.mark.gpu
+ARCH = MI355X()
+
+
+def _prebuilt_attention_candidates(dqk, dv):
+    out = []
+    for br, bc, nt, sq, sv, wpe in prebuilt.PARITY_TILES[:4]:
+        cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+        if gfx950_space.forward_valid(cfg, ARCH) and os.path.exists(codegen.library_path(cfg)):
+            out.append(cfg)
+    return out
+
+
+def test_tune_times_verifies_and_caches(tmp_path, monkeypatch):
+    arrays = make_tensors("attn", 1, 4, 512, 512, 128, 128, "cuda")
+    tuner = AttnTunner(ARCH, arrays, causal=True)
+    tuner.cache_path = str(tmp_path / "cache")
+    cands = _prebuilt_attention_candidates(128, 128)
+    assert len(cands) >= 2
+    monkeypatch.setattr(tuner, "get_tuned_configs", lambda: cands)
+    best = tuner.tune(log_path=str(tmp_path / "logs"), use_cache=False)
+    assert best in cands and tuner.last_timings[best] == min(tuner.last_timings.values())
+    with open(tuner._cache_file()) as f:
+        assert json.load(f)["Br"] == best.Br
+    log = (tmp_path / "logs" / "profile_result_attn_128_128.txt").read_text()
+    assert "best config:" in log and log.count("Config(") == len(cands) + 1
+    # a second tuner for the same problem finds the cached entry without timing anything
+    again = AttnTunner(ARCH, arrays, causal=True)
+    again.cache_path = tuner.cache_path
+    assert again.check_cache() == best
+
+
+def test_a_fast_but_wrong_candidate_is_discarded(tmp_path, monkeypatch):
+    arrays = make_tensors("attn", 1, 4, 512, 512, 128, 128, "cuda")
+    tuner = AttnTunner(ARCH, arrays)
+    tuner.cache_path = str(tmp_path / "cache")
+    cands = _prebuilt_attention_candidates(128, 128)
+    monkeypatch.setattr(tuner, "get_tuned_configs", lambda: cands)
+    fastest = {}
+    real = verify.outputs_match
+
+    def first_call_fails(arrs, ref):
+        if not fastest:
+            fastest["seen"] = True
+            return False
+        return real(arrs, ref)
+
+    monkeypatch.setattr(verify, "outputs_match", first_call_fails)
+    best = tuner.tune(log_path=None, use_cache=False)
+    ranked = sorted((c for c in tuner.last_timings), key=lambda c: tuner.last_timings[c])
+    assert tuner.last_timings[ranked[-1]] == 1e8           # the discarded winner is recorded as failed
+    assert best == ranked[0] and best != ranked[-1]
+
+
+@pytest.mark.parametrize("op,cls,dims", [("ret_bwd", RetBwdTunner, (1, 2, 256, 256, 64, 64)),
+                                         ("attn_bwd", AttnBwdTunner, (1, 2, 256, 256, 128, 128))])
+def test_backward_libraries_pass_the_guard(op, cls, dims):
+    arrays = make_tensors(op, *dims, "cuda")
+    tuner = cls(ARCH, arrays, causal=False)
+    cfg = (gfx950_space.default_backward_config(dims[4], dims[5], ARCH, 128, 128) if op == "ret_bwd"
+           else gfx950_space.default_attn_backward_config(dims[4], dims[5], ARCH, 128, 128))
+    assert tuner.verify(codegen.compile_config(cfg, ARCH))
+    # and the guard does notice a wrong output
+    idx = next(iter(tuner._reference))
+    tuner._reference[idx] = tuner._reference[idx] + 1.0
+    assert not tuner.verify(codegen.compile_config(cfg, ARCH))
