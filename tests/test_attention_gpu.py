@@ -192,3 +192,49 @@ def test_runs_on_the_current_stream():
         o = aat.flash_attn_func(q.cuda(), k.cuda(), v.cuda(), ARCH)
     s.synchronize()
     assert _err(o, ref_op.attention_ref(q, k, v)) <= TOL
+
+
+def test_offsets_beyond_int32_elements():
+    """k and v hold 2^31 elements each: the last (batch, head) slice sits past every 32-bit element offset.
+    The kernel must give that slice exactly what it gives the same data placed at offset zero."""
+    b, h, sq, sk, d = 16, 32, 256, 32768, 128
+    g = torch.Generator(device="cuda").manual_seed(11)
+    k = torch.empty(b, h, sk, d, dtype=torch.float16, device="cuda")
+    v = torch.empty(b, h, sk, d, dtype=torch.float16, device="cuda")
+    assert k.numel() == 2 ** 31
+    k[-1, -1].normal_(generator=g)
+    v[-1, -1].normal_(generator=g)
+    k[0, 0].normal_(generator=g)
+    v[0, 0].normal_(generator=g)
+    q = torch.randn(b, h, sq, d, generator=g, dtype=torch.float16, device="cuda")
+    o = aat.flash_attn_func(q, k, v, ARCH)
+    for bi, hi in ((b - 1, h - 1), (0, 0)):
+        small = aat.flash_attn_func(q[bi:bi + 1, hi:hi + 1].contiguous(), k[bi:bi + 1, hi:hi + 1].contiguous(),
+                                    v[bi:bi + 1, hi:hi + 1].contiguous(), ARCH)
+        ref = ref_op.attention_ref(q[bi:bi + 1, hi:hi + 1].cpu(), k[bi:bi + 1, hi:hi + 1].cpu(), v[bi:bi + 1, hi:hi + 1].cpu())
+        assert _err(o[bi:bi + 1, hi:hi + 1], ref) <= TOL
+        assert _err(small, ref) <= TOL
+
+
+def test_forward_replays_from_a_captured_graph():
+    """A launch through the C ABI can be captured (it allocates nothing and uses the stream it is given);
+    replays with new inputs match eager launches."""
+    q, k, v = (t.cuda() for t in _inputs(2, 4, 512, 512, 128, 128, seed=21))
+    cfg = gfx950_space.default_forward_config("attn", 128, 128, ARCH, 512, 512)
+    rt = Runtime(ARCH, cfg)
+    o = torch.empty_like(q)
+    rt.apply([q, k, v, o], causal=True)                  # first call outside capture: one-time LDS opt-in
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rt.apply([q, k, v, o], causal=True)
+    for seed in (22, 23, 24):
+        q2, k2, v2 = (t.cuda() for t in _inputs(2, 4, 512, 512, 128, 128, seed=seed))
+        q.copy_(q2), k.copy_(k2), v.copy_(v2)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(o)
+        rt.apply([q, k, v, eager], causal=True)
+        torch.cuda.synchronize()
+        assert torch.equal(o, eager)
+        assert _err(o, ref_op.attention_ref(q2, k2, v2, None, True)) <= TOL
