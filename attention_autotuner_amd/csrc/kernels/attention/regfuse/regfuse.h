@@ -184,6 +184,18 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
       constexpr bool MASKED = decltype(masked_tag)::value;   // the causal diagonal may cross this tile
       char* const vcur = vbuf + (NSV == 2 ? PAR * T::kVBytes : 0);
       const bool more = (j + 1 < n_tiles);
+      if constexpr (WPE == 1) {
+        // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
+        // output accumulators in the accumulation half and the Q fragments in the vector half, or the
+        // allocator parks Q there and copies four registers back in front of every MFMA.
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
+        }
+      }
 
       // (A) K_j (and with two V buffers V_j) has landed; every wave is past iteration j-1.
       wait_vmcnt<0>();
@@ -250,6 +262,18 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
       constexpr int PAR = decltype(parity_tag)::value;
       constexpr bool MASKED = decltype(masked_tag)::value;
       const bool last_tile = (j + 1 >= n_tiles);
+      if constexpr (WPE == 1) {
+        // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
+        // output accumulators in the accumulation half and the Q fragments in the vector half, or the
+        // allocator parks Q there and copies four registers back in front of every MFMA.
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
+        }
+      }
       // K copy j and V_j have landed; every wave finished iteration j-1 (frees the other buffers).
       wait_vmcnt<0>();
       block_sync();
