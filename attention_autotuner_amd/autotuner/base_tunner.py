@@ -44,8 +44,9 @@ def _stream_ptr():
 class BaseTunner:
     operation = None                  # config operation name ("attn", ...)
 
-    def __init__(self, arch, torch_array, op_name, causal=False, softmax_scale=None):
+    def __init__(self, arch, torch_array, op_name, causal=False, softmax_scale=None, decay=False):
         self.arch = arch
+        self.decay = bool(decay)                  # RetNet only: torch_array[3] is log2(gamma) [H], not a mask
         self.torch_array = torch_array
         self.op_name = op_name
         self.causal = bool(causal)
@@ -116,15 +117,16 @@ class BaseTunner:
         need = lib.workspace_size(s["B"], s["H"], s["Sq"], s["Sk"])
         ws = torch.empty(max(need, 1), dtype=torch.uint8, device=self.torch_array[0].device) if need else None
         ptrs = [ctypes.c_void_p(t.data_ptr()) for t in self.torch_array]
-        ms = lib.profile_ex(*ptrs, s["B"], s["H"], s["Sq"], s["Sk"], *self._ex_args(),
-                            ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
+        entry = lib.profile_decay if self.decay else lib.profile_ex
+        ms = entry(*ptrs, s["B"], s["H"], s["Sq"], s["Sk"], *([] if self.decay else self._ex_args()),
+                   ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
         return FAILED if ms < 0 else float(ms)
 
     def verify(self, libname):
         """Run ``libname`` once on this tuner's tensors and compare its outputs with torch math."""
         if not hasattr(self, "_reference"):
             scale = None if len(self._ex_args()) == 1 else self._ex_args()[0].value
-            self._reference = verify.reference_outputs(self.operation, self.torch_array, scale, self.causal)
+            self._reference = verify.reference_outputs(self.operation, self.torch_array, scale, self.causal, self.decay)
         lib = library.load(libname, self.operation)
         s = self.problem_shape
         need = lib.workspace_size(s["B"], s["H"], s["Sq"], s["Sk"])
@@ -132,8 +134,9 @@ class BaseTunner:
         for idx in self._reference:
             self.torch_array[idx].zero_()
         ptrs = [ctypes.c_void_p(t.data_ptr()) for t in self.torch_array]
-        rc = lib.kernel_entry_ex(*ptrs, s["B"], s["H"], s["Sq"], s["Sk"], *self._ex_args(),
-                                 ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
+        entry = lib.kernel_entry_decay if self.decay else lib.kernel_entry_ex
+        rc = entry(*ptrs, s["B"], s["H"], s["Sq"], s["Sk"], *([] if self.decay else self._ex_args()),
+                   ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
         torch.cuda.synchronize()
         return rc == 0 and verify.outputs_match(self.torch_array, self._reference)
 
@@ -141,7 +144,7 @@ class BaseTunner:
     def _cache_file(self):
         k, s = self.problem_key, self.problem_shape
         return os.path.join(self.cache_path, "best_config_{}_{}_{}_{}_b{}h{}q{}k{}_c{}.json".format(
-            self.op_name, self.arch.name, k["dim_qk"], k["dim_v"], s["B"], s["H"], s["Sq"], s["Sk"], int(self.causal)))
+            self.op_name + ("_decay" if self.decay else ""), self.arch.name, k["dim_qk"], k["dim_v"], s["B"], s["H"], s["Sq"], s["Sk"], int(self.causal)))
 
     def _legacy_cache_file(self):
         k = self.problem_key

@@ -10,6 +10,8 @@ N_POINTERS = {"attn": 4, "ret": 6, "ret_bwd": 10, "attn_bwd": 9}
 SCALED_OPS = ("attn", "attn_bwd")
 # operators that also export the reference-signature pair profile / kernel_entry
 LEGACY_OPS = ("attn", "ret", "ret_bwd")
+# operators with a decay-mask variant (profile_decay / kernel_entry_decay)
+DECAY_OPS = ("ret", "ret_bwd")
 
 _handles = {}
 _lock = threading.Lock()
@@ -38,6 +40,12 @@ def _bind(lib, op):
     if op == "attn":
         lib.kernel_entry_lse.restype = _I
         lib.kernel_entry_lse.argtypes = [_VP] * 5 + [_I] * 4 + tail
+    if op in DECAY_OPS:                               # mask slot carries log2(gamma) [H]; dqaccum and causal are gone
+        nd = n - 1 if op == "ret_bwd" else n
+        lib.profile_decay.restype = _F
+        lib.profile_decay.argtypes = [_VP] * nd + [_I] * 4 + [_VP, _SZ, _VP]
+        lib.kernel_entry_decay.restype = _I
+        lib.kernel_entry_decay.argtypes = [_VP] * nd + [_I] * 4 + [_VP, _SZ, _VP]
     lib.profile_ex.restype = _F
     lib.profile_ex.argtypes = ptrs + [_I] * 4 + tail
     lib.kernel_entry_ex.restype = _I

@@ -45,8 +45,10 @@ class Runtime:
     def workspace_size(self, B, H, Sq, Sk):
         return int(library.load(self._path(), self.config.operation).workspace_size(B, H, Sq, Sk))
 
-    def apply(self, torch_array, device=None, softmax_scale=None, causal=False, workspace=None, lse=None):
-        """``lse`` (attention forward only): fp32 [B,H,S_q] tensor that receives the log-sum-exp of every row."""
+    def apply(self, torch_array, device=None, softmax_scale=None, causal=False, workspace=None, lse=None, decay=False):
+        """``lse`` (attention forward only): fp32 [B,H,S_q] tensor that receives the log-sum-exp of every row.
+        ``decay`` (RetNet only): the mask slot of ``torch_array`` holds log2(gamma) [H] fp32 and the decay
+        mask is built in registers; the backward's array then has no dqaccum entry."""
         q, k = torch_array[0], torch_array[1]
         if not q.is_cuda:
             raise KernelLaunchError("kernel libraries run on the GPU only; got CPU tensors")
@@ -66,7 +68,11 @@ class Runtime:
         with torch.cuda.device(q.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             ptrs = [ctypes.c_void_p(t.data_ptr()) for t in torch_array]
-            if lse is not None:
+            if decay:
+                if op not in library.DECAY_OPS:
+                    raise KernelLaunchError("only the RetNet operators have a decay-mask variant")
+                rc = lib.kernel_entry_decay(*ptrs, B, H, Sq, Sk, ws_ptr, ws_bytes, stream)
+            elif lse is not None:
                 if op != "attn":
                     raise KernelLaunchError("only the attention forward writes a log-sum-exp")
                 rc = lib.kernel_entry_lse(*ptrs, ctypes.c_void_p(lse.data_ptr()), B, H, Sq, Sk, *extra, ws_ptr, ws_bytes, stream)

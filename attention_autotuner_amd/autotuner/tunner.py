@@ -62,15 +62,15 @@ class AttnTunner(_ForwardTunner):
 class RetTunner(_ForwardTunner):
     operation = "ret"
 
-    def __init__(self, arch, torch_array, causal=False):
-        super().__init__(arch, torch_array, "retnet", causal=causal)
+    def __init__(self, arch, torch_array, causal=False, decay=False):
+        super().__init__(arch, torch_array, "retnet", causal=causal or decay, decay=decay)
 
 
 class RetBwdTunner(BaseTunner):
     operation = "ret_bwd"
 
-    def __init__(self, arch, torch_array, causal=False):
-        super().__init__(arch, torch_array, "retnet_bwd", causal=causal)
+    def __init__(self, arch, torch_array, causal=False, decay=False):
+        super().__init__(arch, torch_array, "retnet_bwd", causal=causal or decay, decay=decay)
         if _is_rocm(arch):
             self.Br_list = list(getattr(gfx950_space, "BWD_BR_LIST", (64, 128)))
             self.Bc_list = list(getattr(gfx950_space, "BWD_BC_LIST", (32, 64, 128)))

@@ -91,8 +91,19 @@ def retnet_backward(q, k, v, mask, do, r):
     return {6: dq, 7: dk, 8: dv}
 
 
-def reference_outputs(op, arrays, scale=None, causal=False):
+def decay_mask(lg2gamma, sq, sk):
+    """[H, sq, sk] fp32: gamma_h^(i + sk - sq - j) on and below that diagonal, zero above it."""
+    e = (torch.arange(sq, device=lg2gamma.device).view(1, sq, 1) + (sk - sq)
+         - torch.arange(sk, device=lg2gamma.device).view(1, 1, sk)).float()
+    d = torch.exp2(lg2gamma.float().view(-1, 1, 1) * e.clamp(min=0))
+    return torch.where(e >= 0, d, torch.zeros((), device=d.device))
+
+
+def reference_outputs(op, arrays, scale=None, causal=False, decay=False):
     """{index into ``arrays``: fp32 reference tensor} for the output tensors of operator ``op``."""
+    if decay:                     # arrays[3] is log2(gamma); the backward's list has no dqaccum at the end
+        arrays = list(arrays)
+        arrays[3] = decay_mask(arrays[3], arrays[0].shape[2], arrays[1].shape[2])
     if op == "attn":
         q, k, v = arrays[:3]
         return attention_forward(q, k, v, scale if scale is not None else 1.0 / math.sqrt(q.shape[-1]), causal)

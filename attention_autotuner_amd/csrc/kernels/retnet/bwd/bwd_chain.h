@@ -72,11 +72,15 @@ struct RetBwdChain {
 // x, y, z, out: [B*H, S, width] fp16 with S = seq_x for x/out and seq_y for y/z; mask [H, seq_q, seq_k];
 // r [B*H, seq_q].  For COL passes seq_x = seq_k, seq_y = seq_q; for the ROW pass the other way round.
 // `causal` promises mask == 0 above the diagonal and only shortens the walk over streamed tiles.
-template <int KX, int DZ, int DZB, int BX, int BY, int Nthreads, int NSY, int NSZ, BwdPass PASS, int WPE = 1>
+// DECAY: the mask is gamma_h^(q + diag - kv) below the diagonal and zero above it, built in registers
+// from lg2gamma[h] = log2(gamma_h); `mask` is not read and tiles above the diagonal are skipped.
+template <int KX, int DZ, int DZB, int BX, int BY, int Nthreads, int NSY, int NSZ, BwdPass PASS, int WPE = 1,
+          bool DECAY = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const half_t* __restrict__ z,
               const half_t* __restrict__ mask, const float* __restrict__ r, half_t* __restrict__ out, int H,
-              int seq_k, int seq_q, int causal) {
+              int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr) {
+  if constexpr (DECAY) causal = 1;
   using T = RetBwdChain<KX, DZ, DZB, BX, BY, Nthreads, NSY, NSZ, PASS>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCY = T::NCY, NCZ = T::NCZ, NCM = T::NCM, WM = T::WM;
   constexpr int PF = AAT_PF;
@@ -115,8 +119,10 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   const char* yg = reinterpret_cast<const char*>(y + (size_t)bh * seq_y * KX);
   const char* zg = reinterpret_cast<const char*>(z + ((size_t)bh * seq_y) * DZ + dz0);
   // mask tile origin: COL -> rows = streamed q, columns = resident kv;  ROW -> rows = resident q, columns = streamed kv
-  const half_t* mhead = mask + (size_t)(bh % H) * seq_q * seq_k;
-  const char* mg = reinterpret_cast<const char*>(COL ? mhead + x0 : mhead + (size_t)x0 * seq_k);
+  const half_t* mhead = DECAY ? nullptr : mask + (size_t)(bh % H) * seq_q * seq_k;
+  const char* mg = DECAY ? nullptr : reinterpret_cast<const char*>(COL ? mhead + x0 : mhead + (size_t)x0 * seq_k);
+  DecayMask<NT, !COL> decay;
+  if constexpr (DECAY) decay.init(lg2gamma[bh % H], h);
 
   typename T::YDma ydma;
   typename T::ZDma zdma;
@@ -169,8 +175,10 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   // Streamed tiles travel through rings of NSY (Y + mask) and NSZ (Z) LDS buffers; `st` is a ring slot.
   auto issue_ym = [&](int j, int st) {            // Y tile j and mask tile j travel together
     ydma.issue(yg + (size_t)j * T::kYBytes, ybuf + st * T::kYBytes, wave_base);
-    const char* msrc = COL ? mg + (size_t)j * BY * seq_k * 2 : mg + (size_t)j * BY * 2;
-    mdma.issue(msrc, mbuf + st * T::kMBytes, wave_base);
+    if constexpr (!DECAY) {
+      const char* msrc = COL ? mg + (size_t)j * BY * seq_k * 2 : mg + (size_t)j * BY * 2;
+      mdma.issue(msrc, mbuf + st * T::kMBytes, wave_base);
+    }
   };
   auto issue_z = [&](int j, int st) {
     zdma.issue(zg + (size_t)j * BY * DZ * 2, zbuf + st * T::kZBytes, wave_base);
@@ -182,7 +190,7 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
         rv[i] = *reinterpret_cast<const f4v*>(rg + j * BY + 32 * (i >> 2) + 8 * (i & 3) + 4 * h);
     }
   };
-  constexpr int kYmInstr = T::YDma::kIters + T::MDma::kIters;   // LDS-DMA instructions per thread for one Y + mask tile
+  constexpr int kYmInstr = T::YDma::kIters + (DECAY ? 0 : T::MDma::kIters);   // LDS-DMA instructions per thread for one Y (+ mask) tile
   constexpr int kRInstr = COL ? NT * 4 : 0;                     // register loads of r per tile
   // Issue order (three Y/mask buffers):  prologue  YM(j0) Z(j0) YM(j0+1);  tile j  Z(j+1) YM(j+2).
   // Loads retire in order, so "at most kYmInstr (+ the r loads of the next tile) outstanding" at the top
@@ -244,7 +252,22 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
     qk_gemm_steps<RT, NT, KS, NCY, PF, kVacc>(tacc, xf, yaddr, yoff, [](int) {});
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      if constexpr (COL) {
+      if constexpr (DECAY) {
+        // this lane's resident index, shifted so that the exponent is (streamed origin) -/+ own
+        const int xrow0 = x0 + wave * WM + rt * 32;
+        if constexpr (COL) {                       // lane owns kv = xrow0 + n; registers run over q rows j*BY + off
+          const int base = j * BY - (xrow0 + n - diag);
+          const auto inv_r = [&](int t, int v) { return fast_rcp(rv[4 * t + (v >> 2)][v & 3]); };
+          if (j * BY < xrow0 + 31 - diag) decay.template apply<true>(tacc[rt], base, inv_r);
+          else decay.template apply<false>(tacc[rt], base, inv_r);
+        } else {                                   // lane owns q = xrow0 + n; registers run over kv columns j*BY + off
+          const int base = xrow0 + n + diag - j * BY;
+          const float ir = inv_r_row[rt];
+          const auto inv_r = [&](int, int) { return ir; };
+          if ((j + 1) * BY - 1 > xrow0 + diag) decay.template apply<true>(tacc[rt], base, inv_r);
+          else decay.template apply<false>(tacc[rt], base, inv_r);
+        }
+      } else if constexpr (COL) {
 #pragma unroll
         for (int i = 0; i < NT * 4; ++i) {
           const h4 m = lds_read_tr_h4_at(maddr[rt][i] + moff);

@@ -34,6 +34,9 @@ using TQ = aat::RetBwdChain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_sta
 const auto kernel_dv = &aat::ret_bwd_chain<Kd, D, DVB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu>;
 const auto kernel_dk = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu>;
 const auto kernel_dq = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row, waves_per_eu>;
+const auto decay_dv = &aat::ret_bwd_chain<Kd, D, DVB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu, true>;
+const auto decay_dk = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu, true>;
+const auto decay_dq = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row, waves_per_eu, true>;
 
 bool bwd_shape_ok(int B, int H, int Seq_q, int Seq_k) {{
   // every sequence length plays both roles (resident rows in one pass, streamed rows in another)
@@ -52,11 +55,31 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_hal
   const H16 *Q = reinterpret_cast<const H16*>(q), *K = reinterpret_cast<const H16*>(k), *V = reinterpret_cast<const H16*>(v),
             *M = reinterpret_cast<const H16*>(mask), *G = reinterpret_cast<const H16*>(dO);
   kernel_dv<<<dim3(B * H * (Seq_k / Br), D / DVB), dim3(Nthreads), TV::kSmemBytes, stream>>>(
-      K, Q, G, M, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, causal);
+      K, Q, G, M, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, causal, nullptr);
   kernel_dk<<<dim3(B * H * (Seq_k / Br), Kd / DKB), dim3(Nthreads), TK::kSmemBytes, stream>>>(
-      V, G, Q, M, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, causal);
+      V, G, Q, M, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, causal, nullptr);
   kernel_dq<<<dim3(B * H * (Seq_q / Br), Kd / DKB), dim3(Nthreads), TQ::kSmemBytes, stream>>>(
-      G, V, K, M, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, causal);
+      G, V, K, M, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, causal, nullptr);
+  return hipGetLastError();
+}}
+// Decay-mask variant: the mask is gamma_h^(q + Seq_k - Seq_q - kv) below the diagonal, zero above it.
+hipError_t launch_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* dO, float* r,
+                        aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k, hipStream_t stream) {{
+  static const hipError_t ok1 = aat::allow_lds(decay_dv, TV::kSmemBytes);
+  static const hipError_t ok2 = aat::allow_lds(decay_dk, TK::kSmemBytes);
+  static const hipError_t ok3 = aat::allow_lds(decay_dq, TQ::kSmemBytes);
+  if (ok1 != hipSuccess) return ok1;
+  if (ok2 != hipSuccess) return ok2;
+  if (ok3 != hipSuccess) return ok3;
+  using H16 = aat::half_t;
+  const H16 *Q = reinterpret_cast<const H16*>(q), *K = reinterpret_cast<const H16*>(k), *V = reinterpret_cast<const H16*>(v),
+            *G = reinterpret_cast<const H16*>(dO);
+  decay_dv<<<dim3(B * H * (Seq_k / Br), D / DVB), dim3(Nthreads), TV::kSmemBytes, stream>>>(
+      K, Q, G, nullptr, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, 1, log2_gamma);
+  decay_dk<<<dim3(B * H * (Seq_k / Br), Kd / DKB), dim3(Nthreads), TK::kSmemBytes, stream>>>(
+      V, G, Q, nullptr, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, 1, log2_gamma);
+  decay_dq<<<dim3(B * H * (Seq_q / Br), Kd / DKB), dim3(Nthreads), TQ::kSmemBytes, stream>>>(
+      G, V, K, nullptr, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, 1, log2_gamma);
   return hipGetLastError();
 }}
 }}  // namespace
@@ -93,5 +116,21 @@ extern "C" int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* mas
 }}
 """
 
-profile_code = global_vars + profile_func + kernel_entry
+decay_entry = r"""
+extern "C" float profile_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* dO, float* r,
+                               aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k, void*, size_t,
+                               void* stream) {{
+  if (!bwd_shape_ok(B, H, Seq_q, Seq_k)) return -1.f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return aat::timed_mean_ms(s, [&] {{ return launch_decay(q, k, v, log2_gamma, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, s); }});
+}}
+extern "C" int kernel_entry_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* dO, float* r,
+                                  aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k, void*,
+                                  size_t, void* stream) {{
+  if (!bwd_shape_ok(B, H, Seq_q, Seq_k)) return AAT_ERR_SHAPE;
+  return (int)launch_decay(q, k, v, log2_gamma, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, static_cast<hipStream_t>(stream));
+}}
+"""
+
+profile_code = global_vars + profile_func + kernel_entry + decay_entry
 kernel_code = profile_code

@@ -22,6 +22,7 @@ constexpr int stages_mask = num_stages_mask < num_stages_qk ? num_stages_qk : nu
 using Traits = aat::RetFwdRegfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, stages_mask>;
 constexpr int shared_mem = Traits::kSmemBytes;
 const auto kernel = &aat::ret_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, stages_mask, waves_per_eu>;
+const auto kernel_decay = &aat::ret_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, stages_mask, waves_per_eu, true>;
 
 hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* o, float* r, int B, int H,
                   int Seq_q, int Seq_k, int causal, hipStream_t stream) {{
@@ -30,7 +31,18 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_hal
   kernel<<<dim3(B * H * (Seq_q / Br)), dim3(Nthreads), shared_mem, stream>>>(
       reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
       reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<const aat::half_t*>(mask),
-      reinterpret_cast<aat::half_t*>(o), r, H, Seq_k, Seq_q, causal);
+      reinterpret_cast<aat::half_t*>(o), r, H, Seq_k, Seq_q, causal, nullptr);
+  return hipGetLastError();
+}}
+// Decay-mask variant: the mask is gamma_h^(q + Seq_k - Seq_q - kv) below the diagonal, zero above it.
+hipError_t launch_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* o, float* r, int B,
+                        int H, int Seq_q, int Seq_k, hipStream_t stream) {{
+  static const hipError_t lds_ok = aat::allow_lds(kernel_decay, shared_mem);
+  if (lds_ok != hipSuccess) return lds_ok;
+  kernel_decay<<<dim3(B * H * (Seq_q / Br)), dim3(Nthreads), shared_mem, stream>>>(
+      reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
+      reinterpret_cast<const aat::half_t*>(v), nullptr, reinterpret_cast<aat::half_t*>(o), r, H, Seq_k, Seq_q, 1,
+      log2_gamma);
   return hipGetLastError();
 }}
 }}  // namespace
@@ -65,5 +77,19 @@ extern "C" int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* mas
 }}
 """
 
-profile_code = global_vars + profile_func + kernel_entry
+decay_entry = r"""
+extern "C" float profile_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* o, float* r,
+                               int B, int H, int Seq_q, int Seq_k, void*, size_t, void* stream) {{
+  if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return -1.f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return aat::timed_mean_ms(s, [&] {{ return launch_decay(q, k, v, log2_gamma, o, r, B, H, Seq_q, Seq_k, s); }});
+}}
+extern "C" int kernel_entry_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* o, float* r,
+                                  int B, int H, int Seq_q, int Seq_k, void*, size_t, void* stream) {{
+  if (!aat::shape_ok(B, H, Seq_q, Seq_k, Br, Bc)) return AAT_ERR_SHAPE;
+  return (int)launch_decay(q, k, v, log2_gamma, o, r, B, H, Seq_q, Seq_k, static_cast<hipStream_t>(stream));
+}}
+"""
+
+profile_code = global_vars + profile_func + kernel_entry + decay_entry
 kernel_code = profile_code

@@ -43,11 +43,14 @@ struct RetFwdRegfuse {
   static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
 };
 
-template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int NSM, int WPE = 1>
+// DECAY: the mask is gamma_h^(q + diag - kv) below the diagonal and zero above it, built in registers
+// from lg2gamma[h] = log2(gamma_h); `mask` is not read and tiles above the diagonal are skipped.
+template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int NSM, int WPE = 1, bool DECAY = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
                 const half_t* __restrict__ mask, half_t* __restrict__ o, float* __restrict__ r, int H,
-                int seq_k, int seq_q, int causal) {
+                int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr) {
+  if constexpr (DECAY) causal = 1;
   using T = RetFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV, NSM>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, NCM = T::NCM, WM = T::WM;
   constexpr int PF = AAT_PF;
@@ -76,7 +79,10 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
 
   const char* kg = reinterpret_cast<const char*>(k + (size_t)bh * seq_k * Kd);
   const char* vg = reinterpret_cast<const char*>(v + (size_t)bh * seq_k * D);
-  const char* mg = reinterpret_cast<const char*>(mask + ((size_t)(bh % H) * seq_q + q0) * seq_k);
+  const char* mg = DECAY ? nullptr : reinterpret_cast<const char*>(mask + ((size_t)(bh % H) * seq_q + q0) * seq_k);
+  const int diag = seq_k - seq_q;
+  DecayMask<NT, true> decay;
+  if constexpr (DECAY) decay.init(lg2gamma[bh % H], h);
 
   typename T::KDma kdma;
   typename T::VDma vdma;
@@ -116,7 +122,7 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
 
   auto issue_km = [&](int j, int par) {          // K tile j and mask tile j travel together
     kdma.issue(kg + (size_t)j * T::kKBytes, kbuf + (NSK == 2 ? par * T::kKBytes : 0), wave_base);
-    mdma.issue(mg + (size_t)j * Bc * 2, mbuf + (NSM == 2 ? par * T::kMBytes : 0), wave_base);
+    if constexpr (!DECAY) mdma.issue(mg + (size_t)j * Bc * 2, mbuf + (NSM == 2 ? par * T::kMBytes : 0), wave_base);
   };
   if (n_tiles > 0) {
     issue_km(0, 0);
@@ -154,7 +160,14 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
     qk_gemm_steps<RT, NT, KS, NCK, PF, kVacc>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      apply_mask<NT>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
+      if constexpr (DECAY) {
+        const int own0 = q0 + wave * WM + rt * 32 + diag;              // q + diag of the group's first row
+        const auto one = [](int, int) { return 1.0f; };
+        if ((j + 1) * Bc - 1 > own0) decay.template apply<true>(sacc[rt], own0 + n - j * Bc, one);
+        else decay.template apply<false>(sacc[rt], own0 + n - j * Bc, one);
+      } else {
+        apply_mask<NT>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
+      }
       retention_step<NT, DT, WPE == 1>(sacc[rt], row[rt], oacc[rt]);
     }
 

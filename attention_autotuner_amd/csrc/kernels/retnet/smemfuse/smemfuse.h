@@ -39,11 +39,15 @@ struct RetFwdSmemfuse {
   static constexpr int kSmemBytes = kMainBytes > G::kEpiBytes ? kMainBytes : G::kEpiBytes;
 };
 
-template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int NSM, int W1N, int W2N, int WPE = 1>
+// DECAY: the mask is gamma_h^(q + diag - kv) below the diagonal and zero above it, built in registers
+// from lg2gamma[h] = log2(gamma_h); `mask` is not read and tiles above the diagonal are skipped.
+template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int NSM, int W1N, int W2N, int WPE = 1,
+          bool DECAY = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 ret_fwd_smemfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
                  const half_t* __restrict__ mask, half_t* __restrict__ o, float* __restrict__ r, int H,
-                 int seq_k, int seq_q, int causal) {
+                 int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr) {
+  if constexpr (DECAY) causal = 1;
   using T = RetFwdSmemfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV, NSM, W1N, W2N>;
   using G = typename T::G;
   constexpr int RT1 = G::RT1, NT1 = G::NT1, RT2 = G::RT2, DT2 = G::DT2, KS = T::KS, NCK = T::NCK, NCV = T::NCV, NCM = T::NCM;
@@ -79,7 +83,10 @@ ret_fwd_smemfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, con
 
   const char* kg = reinterpret_cast<const char*>(k + (size_t)bh * seq_k * Kd);
   const char* vg = reinterpret_cast<const char*>(v + (size_t)bh * seq_k * D);
-  const char* mg = reinterpret_cast<const char*>(mask + ((size_t)(bh % H) * seq_q + q0) * seq_k);
+  const char* mg = DECAY ? nullptr : reinterpret_cast<const char*>(mask + ((size_t)(bh % H) * seq_q + q0) * seq_k);
+  const int diag = seq_k - seq_q;
+  DecayMask<NT1, true> decay;
+  if constexpr (DECAY) decay.init(lg2gamma[bh % H], h);
   typename T::KDma kdma;
   typename T::VDma vdma;
   typename T::MDma mdma;
@@ -124,7 +131,7 @@ ret_fwd_smemfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, con
 
   auto issue_km = [&](int j, int par) {
     kdma.issue(kg + (size_t)j * T::kKBytes, kbuf + (NSK == 2 ? par * T::kKBytes : 0), wave_base);
-    mdma.issue(mg + (size_t)j * Bc * 2, mbuf + (NSM == 2 ? par * T::kMBytes : 0), wave_base);
+    if constexpr (!DECAY) mdma.issue(mg + (size_t)j * Bc * 2, mbuf + (NSM == 2 ? par * T::kMBytes : 0), wave_base);
   };
   if (n_tiles > 0) {
     issue_km(0, 0);
@@ -146,7 +153,15 @@ ret_fwd_smemfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, con
     float tile_abs[RT1];
 #pragma unroll
     for (int rt = 0; rt < RT1; ++rt) {
-      apply_mask<NT1>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
+      if constexpr (DECAY) {
+        const int own0 = q0 + row1 + rt * 32 + diag;                   // q + diag of the group's first row
+        const int kv_org = j * Bc + w1n * G::CN1;                       // first kv column of this wave's score tiles
+        const auto one = [](int, int) { return 1.0f; };
+        if (kv_org + G::CN1 - 1 > own0) decay.template apply<true>(sacc[rt], own0 + n - kv_org, one);
+        else decay.template apply<false>(sacc[rt], own0 + n - kv_org, one);
+      } else {
+        apply_mask<NT1>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
+      }
       float a = 0.f;
 #pragma unroll
       for (int nt = 0; nt < NT1; ++nt)

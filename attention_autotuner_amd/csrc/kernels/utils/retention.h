@@ -35,6 +35,54 @@ AAT_DEV void apply_mask(f16v (&s)[NT], const uint32_t (&maddr)[NT * 4], int buf_
   }
 }
 
+// Decay mask evaluated in registers instead of read from a [H, S_q, S_kv] tensor.  The reference always
+// streams the tensor (reference: python/ops/retnet_interface.py:26-31) and lists "causal config" and the
+// mask stream's cost ("retnet performance issue ... mask stage 2?") as open items (README.md:102-114):
+//     D[q][kv] = gamma^(q + diag - kv)  for kv <= q + diag,   0 above the diagonal,   diag = S_kv - S_q.
+// In the transposed score layout a lane owns one index and its 16*NT registers run over the other one
+// at fixed offsets off(t, v) = 32t + 8(v/4) + 4h + v%4 from the tile origin, so with lg = log2(gamma)
+//     D = exp2(lg * base) * fac[t][v]
+// is one per-lane scalar per tile times 16*NT per-lane constants:
+//     OWN_Q  (lane owns q, registers run over kv):  base = (q + diag) - kv_origin,  fac = exp2(-lg * off)
+//     !OWN_Q (lane owns kv, registers run over q):  base = q_origin - (kv - diag),  fac = exp2(+lg * off)
+// Off the diagonal |lg| * tile_rows bounds the exponents, so nothing overflows for gamma >= 0.5 and
+// tiles of up to 128 rows; far below the diagonal the scalar underflows to zero, as the fp16 tensor does.
+template <int NT, bool OWN_Q>
+struct DecayMask {
+  float fac[NT][16];
+  float lg;
+  int h4;
+
+  AAT_DEV void init(float lg2gamma, int h) {
+    lg = lg2gamma;
+    h4 = 4 * h;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float off = (float)(32 * t + 8 * (v >> 2) + h4 + (v & 3));
+        fac[t][v] = fast_exp2((OWN_Q ? -lg : lg) * off);
+      }
+  }
+  // s <- s * D * extra for the tile whose origin makes `base` (see above).  DIAG: the diagonal may cross
+  // this tile, entries above it are zeroed.
+  template <bool DIAG, class Extra>
+  AAT_DEV void apply(f16v (&s)[NT], int base, Extra&& extra) const {
+    const float tf = fast_exp2(lg * (float)base);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float m = tf * fac[t][v] * extra(t, v);
+        if constexpr (DIAG) {
+          const int off = 32 * t + 8 * (v >> 2) + h4 + (v & 3);
+          if ((OWN_Q ? base - off : base + off) < 0) m = 0.f;
+        }
+        s[t][v] *= m;
+      }
+  }
+};
+
 // Fold one masked score tile into the row statistics and turn it into P = S / r_ref (in place).
 // Rescales the O accumulators when the reference scale moves.
 // ACC_PIN: the O accumulators live in accumulation registers (kernels above 256 registers); rescale

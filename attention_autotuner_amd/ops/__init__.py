@@ -1,4 +1,4 @@
 from .attention_interface import flash_attn_func, MultiHeadAttnFunc, REFERENCE_SOFTMAX_SCALE
-from .retnet_interface import RetNetAttnFunc, RetNetAttn
+from .retnet_interface import RetNetAttnFunc, RetNetAttn, RetNetDecayAttnFunc, RetNetDecayAttn
 
-__all__ = ["flash_attn_func", "MultiHeadAttnFunc", "RetNetAttnFunc", "RetNetAttn", "REFERENCE_SOFTMAX_SCALE"]
+__all__ = ["flash_attn_func", "MultiHeadAttnFunc", "RetNetAttnFunc", "RetNetAttn", "RetNetDecayAttnFunc", "RetNetDecayAttn", "REFERENCE_SOFTMAX_SCALE"]

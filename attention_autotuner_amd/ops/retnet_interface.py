@@ -5,6 +5,12 @@ Drop-in for reference python/ops/retnet_interface.py:8-57:
 ``o = (S / r) v``.  mask is [H, S_q, S_kv] fp16.  ``causal=True`` promises the mask is zero above the
 diagonal, which lets the kernels skip those tiles (the reference accepts and ignores the flag).
 backward returns one gradient per forward input (the reference returns one too few).
+
+``RetNetDecayAttnFunc(q, k, v, gamma, device_type)`` is the same operator for RetNet's own mask,
+``mask[h, i, j] = gamma_h^(i + S_kv - S_q - j)`` on and below that diagonal and 0 above it: the mask is
+built in registers from ``gamma`` ([H], 0.5 <= gamma_h <= 1) instead of being streamed from a
+[H, S_q, S_kv] tensor, and tiles above the diagonal are skipped.  The reference has no such entry (it
+always streams the tensor, python/ops/retnet_interface.py:26-31).
 """
 import torch
 
@@ -53,15 +59,57 @@ class RetNetAttn(torch.autograd.Function):
         dq = torch.empty_like(q)
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)
-        dq_accum = torch.zeros([batch_size, nheads, seqlen_q, key_dim], device=q.device, dtype=torch.float32)
+        # The reference's kernel accumulates dQ into this fp32 scratch with atomics; the kernels here never
+        # touch it (dQ is produced directly), so a token buffer stands in for the [B,H,S_q,d_qk] tensor.
+        dq_accum = torch.zeros(1, device=q.device, dtype=torch.float32)
         arrays = [q, k, v, mask, do, r, dq, dk, dv, dq_accum]
         tuner = RetBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal)
-        tuned_now = tuner.check_cache() is None
         cc = resolve(tuner, lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        if tuned_now:
-            dq_accum.zero_()                      # tuning launches accumulated into the scratch
         Runtime(device_type, cc).apply(arrays, causal=ctx.causal)
         return dq, dk, dv, None, None, None
 
 
+class RetNetDecayAttn(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, q, k, v, gamma, device_type: Arch):
+        if not (q.is_cuda and k.is_cuda and v.is_cuda):
+            raise RuntimeError("RetNetDecayAttnFunc runs on the GPU only (HIP kernels); move the tensors to a cuda device")
+        assert q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16
+        q, k, v = [x.contiguous() for x in (q, k, v)]
+        batch_size, nheads, seqlen_q, key_dim = q.shape
+        seqlen_k = k.shape[2]
+        head_dim = v.shape[-1]
+        gamma = torch.as_tensor(gamma, dtype=torch.float64).reshape(-1)
+        assert gamma.numel() == nheads and bool(((gamma >= 0.5) & (gamma <= 1.0)).all()), "one decay rate in [0.5, 1] per head"
+        assert head_dim % 64 == 0 and head_dim <= 512
+        assert key_dim % 64 == 0 and key_dim <= 256
+        lg = torch.log2(gamma).to(device=q.device, dtype=torch.float32).contiguous()
+
+        o = torch.empty(batch_size, nheads, seqlen_q, head_dim, device=q.device, dtype=torch.float16)
+        r = torch.empty(batch_size, nheads, seqlen_q, device=q.device, dtype=torch.float32)
+        arrays = [q, k, v, lg, o, r]
+        tuner = RetTunner(arch=device_type, torch_array=arrays, decay=True)
+        cc = resolve(tuner, lambda: gfx950_space.default_forward_config("ret", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+        Runtime(device_type, cc).apply(arrays, decay=True)
+        ctx.save_for_backward(q, k, v, lg, r)
+        ctx.device_type = device_type
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, lg, r = ctx.saved_tensors
+        device_type = ctx.device_type
+        key_dim, head_dim = q.shape[-1], v.shape[-1]
+        seqlen_q, seqlen_k = q.shape[2], k.shape[2]
+        do = do.contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        arrays = [q, k, v, lg, do, r, dq, dk, dv]
+        tuner = RetBwdTunner(arch=device_type, torch_array=arrays, decay=True)
+        cc = resolve(tuner, lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+        Runtime(device_type, cc).apply(arrays, decay=True)
+        return dq, dk, dv, None, None
+
+
 RetNetAttnFunc = RetNetAttn.apply
+RetNetDecayAttnFunc = RetNetDecayAttn.apply

@@ -32,7 +32,7 @@
 
 #include <stddef.h>
 
-#define AAT_ABI_VERSION 2
+#define AAT_ABI_VERSION 3
 #define AAT_ERR_SHAPE (-2)      /* Seq_q / Seq_k not divisible by the tile, or a non-positive size */
 #define AAT_ERR_WORKSPACE (-3)  /* workspace missing or smaller than workspace_size() */
 
@@ -82,6 +82,18 @@ float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half
 int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* o, float* r,
                     int B, int H, int Seq_q, int Seq_k, int causal, void* workspace,
                     size_t workspace_bytes, void* stream);
+/* The same with RetNet's decay mask built in registers instead of read from a tensor:
+ * mask[h][i][j] = gamma_h^(i + Seq_k - Seq_q - j) for j <= i + Seq_k - Seq_q, 0 above that diagonal;
+ * log2_gamma [H] fp32 holds log2(gamma_h), 0.5 <= gamma_h <= 1.  Tiles above the diagonal are skipped.
+ * No counterpart in the reference, which always streams the [H,Seq_q,Seq_k] tensor
+ * (python/ops/retnet_interface.py:26-31) and lists "causal config" and the mask stream's cost as open
+ * items (README.md:102-114). */
+float profile_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* o, float* r,
+                    int B, int H, int Seq_q, int Seq_k, void* workspace, size_t workspace_bytes,
+                    void* stream);
+int kernel_entry_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* o,
+                       float* r, int B, int H, int Seq_q, int Seq_k, void* workspace,
+                       size_t workspace_bytes, void* stream);
 
 #elif defined(AAT_OP_RET_BWD)
 /* RetNet parallel backward.  Replaces: reference csrc/kernels/retnet/bwd/profile_code.py:53 and :98.
@@ -98,6 +110,13 @@ float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half
 int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
                     aat_half* dq, aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q,
                     int Seq_k, int causal, void* workspace, size_t workspace_bytes, void* stream);
+/* Decay-mask variant of the backward (see the forward's profile_decay); no dqaccum argument. */
+float profile_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* dO, float* r,
+                    aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k,
+                    void* workspace, size_t workspace_bytes, void* stream);
+int kernel_entry_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_gamma, aat_half* dO,
+                       float* r, aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q,
+                       int Seq_k, void* workspace, size_t workspace_bytes, void* stream);
 
 #elif defined(AAT_OP_ATTN_BWD)
 /* Flash-attention backward: dq, dk, dv from q, k, v, o, dO and the forward's lse (see kernel_entry_lse).

@@ -31,7 +31,7 @@ def test_header_declares_the_reference_pair_for_every_operator():
     pair = ["abi_version", "config_string", "kernel_entry", "kernel_entry_ex", "profile", "profile_ex", "workspace_size"]
     assert _declared_symbols("AAT_OP_ATTN") == sorted(pair + ["kernel_entry_lse"])
     for macro in ("AAT_OP_RET", "AAT_OP_RET_BWD"):
-        assert _declared_symbols(macro) == pair
+        assert _declared_symbols(macro) == sorted(pair + ["kernel_entry_decay", "profile_decay"])
     # the attention backward has no reference signature to keep: only the extended entry points
     assert _declared_symbols("AAT_OP_ATTN_BWD") == ["abi_version", "config_string", "kernel_entry_ex", "profile_ex", "workspace_size"]
 
@@ -60,7 +60,7 @@ def test_shipping_set_is_built_and_exports_the_abi():
         for name in _declared_symbols(macro[cfg.operation]):
             assert hasattr(raw, name), (cfg, name)
         lib = library.load(path, cfg.operation)
-        assert lib.abi_version() == 2
+        assert lib.abi_version() == 3
         assert lib.config_string().decode() == f"{cfg.operation}:{cfg}"
         if cfg.operation == "attn_bwd":
             assert lib.workspace_size(2, 3, 256, 512) == 2 * 2 * 3 * 256 * 4      # lse2 + delta, fp32 per query row

@@ -151,3 +151,61 @@ def test_reference_signature_entry_points_bwd():
         assert ok, ex
     assert acc.abs().max().item() == 0          # the scratch is never touched
     assert lib.kernel_entry(*ptrs, 1, 2, 100, 128) == -2
+
+
+# ---------------------------------------------------------------------------------- decay mask on the fly
+def _decay_problem(b, h, sq, sk, dqk, dv, seed):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v, do = (torch.randn(*s, generator=g).half() for s in ((b, h, sq, dqk), (b, h, sk, dqk), (b, h, sk, dv), (b, h, sq, dv)))
+    gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(h, dtype=torch.float64))
+    n = torch.arange(sq, dtype=torch.float64).view(1, sq, 1) + (sk - sq)
+    m = torch.arange(sk, dtype=torch.float64).view(1, 1, sk)
+    mask = torch.where(n >= m, gamma.view(h, 1, 1) ** (n - m).clamp(min=0), torch.zeros((), dtype=torch.float64)).float()
+    return q, k, v, do, gamma, mask
+
+
+@pytest.mark.parametrize("dqk,dv", [(64, 64), (128, 128), (256, 256), (256, 512)])
+@pytest.mark.parametrize("sq,sk", [(256, 256), (128, 384)])
+def test_decay_operator_matches_oracle_with_the_exact_mask(dqk, dv, sq, sk):
+    """Oracle: the same closed forms with the decay mask evaluated in fp64 and held in fp32 (the
+    tensor-mask path rounds it to fp16; the register path does not round it at all)."""
+    q, k, v, do, gamma, mask = _decay_problem(2, 3, sq, sk, dqk, dv, seed=dqk + sq)
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = aat.RetNetDecayAttnFunc(qc, kc, vc, gamma, ARCH)
+    o.backward(do.cuda())
+    ref_o, ref_r = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    grads = ref_op.retnet_bwd_ref(q, k, v, mask, do, ref_r)
+    assert (o.detach().float().cpu() - ref_o).abs().max().item() <= 2e-3
+    for name, got, want in zip(("dq", "dk", "dv"), (qc.grad, kc.grad, vc.grad), grads):
+        err = (got.float().cpu() - want).abs()
+        assert bool((err <= 2e-3 + 1e-3 * want.abs()).all()), (name, err.max().item())
+
+
+def test_decay_operator_agrees_with_the_tensor_mask_operator_at_config_4():
+    q, k, v, do, gamma, mask = _decay_problem(4, 8, 2048, 2048, 256, 512, seed=4)
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = aat.RetNetDecayAttnFunc(qc, kc, vc, gamma, ARCH)
+    o.backward(do.cuda())
+    q2, k2, v2 = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o2 = aat.RetNetAttnFunc(q2, k2, v2, mask.half().cuda(), ARCH, True)
+    o2.backward(do.cuda())
+    # the two paths differ only in the fp16 rounding of the mask values (relative 2^-11)
+    assert (o.float() - o2.float()).abs().max().item() <= 4e-3
+    for a, b in ((qc.grad, q2.grad), (kc.grad, k2.grad), (vc.grad, v2.grad)):
+        d = (a.float() - b.float()).abs()
+        assert bool((d <= 4e-3 + 4e-3 * b.float().abs()).all()), d.max().item()
+    for b, h in ((0, 0), (3, 7)):                       # and the oracle on two (batch, head) slices
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref_o, ref_r = ref_op.retnet_ref(q[sl], k[sl], v[sl], mask[h:h + 1], return_r=True)
+        assert (o[sl].detach().float().cpu() - ref_o).abs().max().item() <= 2e-3
+        for got, want in zip((qc.grad[sl], kc.grad[sl], vc.grad[sl]), ref_op.retnet_bwd_ref(q[sl], k[sl], v[sl], mask[h:h + 1], do[sl], ref_r)):
+            err = (got.float().cpu() - want).abs()
+            assert bool((err <= 2e-3 + 1e-3 * want.abs()).all()), err.max().item()
+
+
+def test_decay_rate_must_be_one_per_head_and_in_range():
+    q = torch.zeros(1, 2, 128, 64, dtype=torch.float16, device="cuda")
+    with pytest.raises(AssertionError):
+        aat.RetNetDecayAttnFunc(q, q, q, [0.9], ARCH)
+    with pytest.raises(AssertionError):
+        aat.RetNetDecayAttnFunc(q, q, q, [0.9, 0.2], ARCH)
