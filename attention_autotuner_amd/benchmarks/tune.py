@@ -5,6 +5,7 @@ python/tests/attntuner_demo.py:186-192 and python/tests/test_retbwdtunner.py:88-
     python -m attention_autotuner_amd.benchmarks.tune ret     B H Sq Sk dqk dv [--causal]
     python -m attention_autotuner_amd.benchmarks.tune ret_bwd B H Sq Sk dqk dv [--causal]
     python -m attention_autotuner_amd.benchmarks.tune attn_bwd B H Sq Sk dqk dv [--causal]
+    python -m attention_autotuner_amd.benchmarks.tune ret|ret_bwd ... --decay      (decay mask built in registers)
 
 Writes the best configuration into the tuning cache, the per-candidate log next to it, and prints a
 one-line JSON summary.  ``--compile-only`` builds every candidate library (no GPU needed) so that a
@@ -64,7 +65,7 @@ def make_tensors(op, b, h, sq, sk, dqk, dv, device, seed=0):
 
 def flops(op, b, h, sq, sk, dqk, dv, causal):
     f = 2.0 * b * h * sq * sk * ((dqk + dv) if op in ("attn", "ret") else (3 * dqk + 2 * dv))
-    return f / 2 if (causal and op in ("attn", "attn_bwd")) else f
+    return f / 2 if (causal and op in ("attn", "attn_bwd")) else f      # RetNet rates are quoted on the dense count
 
 
 def main(argv=None):
@@ -72,6 +73,7 @@ def main(argv=None):
     ap.add_argument("op", choices=["attn", "ret", "ret_bwd", "attn_bwd"])
     ap.add_argument("dims", type=int, nargs=6, metavar="N", help="B H Sq Sk dqk dv")
     ap.add_argument("--causal", action="store_true")
+    ap.add_argument("--decay", action="store_true", help="RetNet only: decay mask built in registers from one rate per head")
     ap.add_argument("--compile-only", action="store_true")
     ap.add_argument("--log-dir", default=DEFAULT_LOG_DIR)
     args = ap.parse_args(argv)
@@ -80,7 +82,16 @@ def main(argv=None):
     cls = {"attn": AttnTunner, "ret": RetTunner, "ret_bwd": RetBwdTunner, "attn_bwd": AttnBwdTunner}[args.op]
     device = "meta" if args.compile_only else "cuda"
     arrays = make_tensors(args.op, b, h, sq, sk, dqk, dv, device)
-    tuner = cls(arch, arrays, causal=args.causal)
+    if args.decay:
+        if args.op not in ("ret", "ret_bwd"):
+            ap.error("--decay applies to ret and ret_bwd")
+        gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(h, dtype=torch.float64))
+        arrays[3] = torch.log2(gamma).float().to(device) if device != "meta" else torch.empty(h, device="meta")
+        if args.op == "ret_bwd":
+            arrays = arrays[:9]                                # no dqaccum in the decay entry points
+        tuner = cls(arch, arrays, decay=True)
+    else:
+        tuner = cls(arch, arrays, causal=args.causal)
     if args.compile_only:
         cfgs = [c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)]
         t0 = time.time()
@@ -88,7 +99,7 @@ def main(argv=None):
         print(json.dumps({"op": args.op, "candidates": len(cfgs), "built": sum(l is not None for l in libs),
                           "seconds": round(time.time() - t0, 1)}))
         return 0
-    log_dir = os.path.join(args.log_dir, f"{args.op}_b{b}h{h}q{sq}k{sk}_c{int(args.causal)}")
+    log_dir = os.path.join(args.log_dir, f"{args.op}{'_decay' if args.decay else ''}_b{b}h{h}q{sq}k{sk}_c{int(args.causal or args.decay)}")
     best = tuner.tune(log_path=log_dir, use_cache=False)
     ms = tuner.last_timings[best]
     ok = [t for t in tuner.last_timings.values() if t < 1e7]

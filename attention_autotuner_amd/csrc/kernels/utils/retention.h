@@ -41,28 +41,30 @@ AAT_DEV void apply_mask(f16v (&s)[NT], const uint32_t (&maddr)[NT * 4], int buf_
 //     D[q][kv] = gamma^(q + diag - kv)  for kv <= q + diag,   0 above the diagonal,   diag = S_kv - S_q.
 // In the transposed score layout a lane owns one index and its 16*NT registers run over the other one
 // at fixed offsets off(t, v) = 32t + 8(v/4) + 4h + v%4 from the tile origin, so with lg = log2(gamma)
-//     D = exp2(lg * base) * fac[t][v]
-// is one per-lane scalar per tile times 16*NT per-lane constants:
+//     D = exp2(lg * base) * fac(t, v)
+// is one per-lane scalar per tile times per-lane constants:
 //     OWN_Q  (lane owns q, registers run over kv):  base = (q + diag) - kv_origin,  fac = exp2(-lg * off)
 //     !OWN_Q (lane owns kv, registers run over q):  base = q_origin - (kv - diag),  fac = exp2(+lg * off)
 // Off the diagonal |lg| * tile_rows bounds the exponents, so nothing overflows for gamma >= 0.5 and
 // tiles of up to 128 rows; far below the diagonal the scalar underflows to zero, as the fp16 tensor does.
+// The offsets split as off = (32t + 8g) + (4h + e) with v = 4g + e, so the 16*NT constants are products
+// of 4*NT + 4 of them: fb[t][g] = exp2(-/+lg * (32t + 8g)), fa[e] = exp2(-/+lg * (4h + e)).
 template <int NT, bool OWN_Q>
 struct DecayMask {
-  float fac[NT][16];
+  float fa[4], fb[NT][4];
   float lg;
   int h4;
 
   AAT_DEV void init(float lg2gamma, int h) {
     lg = lg2gamma;
     h4 = 4 * h;
+    const float step = OWN_Q ? -lg : lg;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) fa[e] = fast_exp2(step * (float)(h4 + e));
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float off = (float)(32 * t + 8 * (v >> 2) + h4 + (v & 3));
-        fac[t][v] = fast_exp2((OWN_Q ? -lg : lg) * off);
-      }
+      for (int g = 0; g < 4; ++g) fb[t][g] = fast_exp2(step * (float)(32 * t + 8 * g));
   }
   // s <- s * D * extra for the tile whose origin makes `base` (see above).  DIAG: the diagonal may cross
   // this tile, entries above it are zeroed.
@@ -72,13 +74,18 @@ struct DecayMask {
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float m = tf * fac[t][v] * extra(t, v);
-        if constexpr (DIAG) {
-          const int off = 32 * t + 8 * (v >> 2) + h4 + (v & 3);
-          if ((OWN_Q ? base - off : base + off) < 0) m = 0.f;
+      for (int g = 0; g < 4; ++g) {
+        const float tg = tf * fb[t][g];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int v = 4 * g + e;
+          float m = tg * fa[e] * extra(t, v);
+          if constexpr (DIAG) {
+            const int off = 32 * t + 8 * g + h4 + e;
+            if ((OWN_Q ? base - off : base + off) < 0) m = 0.f;
+          }
+          s[t][v] *= m;
         }
-        s[t][v] *= m;
       }
   }
 };
