@@ -242,6 +242,17 @@ def retnet_measurements(aat, arch, mk, steps, warmup):
     _, ms_fb = time_launches(fb, steps, warmup)
     res["retnet_fwd_bwd_b4h8s2048_dqk256_dv512"] = {"ms": round(ms_fb, 5), "tflops": round((fwd_flops + bwd_flops) / ms_fb / 1e9, 1)}
     log(f"retnet fwd+bwd: {ms_fb:.4f} ms -> {(fwd_flops + bwd_flops) / ms_fb / 1e9:.1f} TFLOP/s (dense-mask FLOPs)")
+
+    if hasattr(aat, "RetNetDecayAttnFunc"):              # the same decay mask, built in registers from one rate per head
+        gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(h, dtype=torch.float64))
+
+        def fb_decay():
+            q.grad = k.grad = v.grad = None
+            aat.RetNetDecayAttnFunc(q, k, v, gamma, arch).backward(do)
+
+        _, ms_d = time_launches(fb_decay, steps, warmup)
+        res["retnet_decay_fwd_bwd_b4h8s2048_dqk256_dv512"] = {"ms": round(ms_d, 5), "tflops": round((fwd_flops + bwd_flops) / ms_d / 1e9, 1)}
+        log(f"retnet decay fwd+bwd: {ms_d:.4f} ms -> {(fwd_flops + bwd_flops) / ms_d / 1e9:.1f} TFLOP/s (dense-mask FLOPs)")
     return res
 
 
