@@ -1,0 +1,132 @@
+"""Export (configuration features, measured cycles) pairs for fitting a cost model of the search space.
+
+MI355X counterpart of reference python/tests/export_costmodel_config.py:1-62 and python/tests/ncu_profile.py:10-44:
+the reference runs Nsight Compute once per candidate and reads "Elapsed Cycles"; here ONE rocprofv3
+counter run (GRBM_GUI_ACTIVE, busy cycles summed over the 8 XCDs) covers every candidate, because the
+candidates are separately built libraries that one process can launch back to back.
+
+    python -m attention_autotuner_amd.benchmarks.export_costmodel_config attn 4 32 2048 2048 128 128 [--causal] [--limit N] [--out FILE]
+
+The outer invocation builds the candidate libraries, starts itself under ``rocprofv3 --pmc`` with
+``--run-candidates`` (that inner process launches every candidate twice: one warm-up, one counted),
+matches the counter rows to the candidates by dispatch order and writes a JSON list of
+
+    {"config": {...}, "cost_model_config": [[Sq, Sk, dqk, dv], [Br, Bc, BlockK, D], [wave tile of the first
+     contraction], [wave tile of the second], B, H], "cycles": int, "lds_bytes": int, "registers": int}
+
+in the tuple layout of the reference's exporter (wave tiles are (rows, columns, 16): the rows and
+columns one wave computes per step and the MFMA k depth).
+"""
+import argparse
+import csv
+import glob
+import json
+import os
+import subprocess
+import sys
+import tempfile
+
+import torch
+
+from ..arch import MI355X
+from ..autotuner import codegen, gfx950_space, library
+from .tune import make_tensors
+
+TUNERS = {"attn": "AttnTunner", "ret": "RetTunner"}
+XCDS = 8
+
+
+def candidates(op, dims, causal, limit):
+    from ..autotuner import tunner
+    b, h, sq, sk, dqk, dv = dims
+    arrays = make_tensors(op, b, h, sq, sk, dqk, dv, "meta")
+    t = getattr(tunner, TUNERS[op])(MI355X(), arrays, causal=causal)
+    cfgs = [c for c in t.get_tuned_configs() if t._fits_problem(c) and getattr(c, "kv_splits", 1) == 1]
+    return cfgs[:limit] if limit else cfgs
+
+
+def cost_model_tuple(cfg, dims):
+    b, h, sq, sk, dqk, dv = dims
+    nw = cfg.Nthreads // 64
+    if cfg.fuse_type == "shared":
+        w1n, w2n = cfg.warps_mma1_n, cfg.warps_mma_n
+    else:                                                 # register fuse: every wave owns whole rows of both contractions
+        w1n = w2n = 1
+    tile1 = (cfg.Br // (nw // w1n), cfg.Bc // w1n, 16)
+    tile2 = (cfg.Br // (nw // w2n), cfg.D // w2n, 16)
+    return [[sq, sk, dqk, dv], [cfg.Br, cfg.Bc, cfg.BlockKSmem, cfg.D], list(tile1), list(tile2), b, h]
+
+
+def run_candidates(op, dims, causal, limit):
+    """Inner mode (under rocprofv3): launch every candidate library twice."""
+    import ctypes
+    b, h, sq, sk, dqk, dv = dims
+    arrays = make_tensors(op, b, h, sq, sk, dqk, dv, "cuda")
+    ptrs = [ctypes.c_void_p(t.data_ptr()) for t in arrays]
+    extra = [ctypes.c_float(dqk ** -0.5), ctypes.c_int(int(causal))] if op == "attn" else [ctypes.c_int(int(causal))]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for cfg in candidates(op, dims, causal, limit):
+        path = codegen.library_path(cfg)
+        if not os.path.exists(path):
+            continue
+        lib = library.load(path, op)
+        for _ in range(2):
+            rc = lib.kernel_entry_ex(*ptrs, b, h, sq, sk, *extra, ctypes.c_void_p(0), ctypes.c_size_t(0), stream)
+            if rc != 0:
+                raise RuntimeError(f"{cfg}: kernel_entry_ex returned {rc}")
+        torch.cuda.synchronize()
+        print("LAUNCHED " + str(cfg), flush=True)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("op", choices=sorted(TUNERS))
+    ap.add_argument("dims", type=int, nargs=6, metavar="N", help="B H Sq Sk dqk dv")
+    ap.add_argument("--causal", action="store_true")
+    ap.add_argument("--limit", type=int, default=0, help="only the first N candidates")
+    ap.add_argument("--out", default=None)
+    ap.add_argument("--run-candidates", action="store_true", help=argparse.SUPPRESS)
+    args = ap.parse_args(argv)
+    if args.run_candidates:
+        run_candidates(args.op, args.dims, args.causal, args.limit)
+        return 0
+
+    arch = MI355X()
+    cfgs = candidates(args.op, args.dims, args.causal, args.limit)
+    libs = codegen.compile_parallel(cfgs, arch, timeout=300)
+    cfgs = [c for c, l in zip(cfgs, libs) if l is not None]
+    out_dir = tempfile.mkdtemp(prefix="aat_costmodel_", dir=os.environ.get("TMPDIR", "/tmp"))
+    inner = [sys.executable, "-m", "attention_autotuner_amd.benchmarks.export_costmodel_config", args.op,
+             *map(str, args.dims), "--run-candidates", "--limit", str(args.limit)] + (["--causal"] if args.causal else [])
+    cmd = ["rocprofv3", "--pmc", "GRBM_GUI_ACTIVE", "--output-format", "csv", "-d", out_dir, "-o", "cm", "--", *inner]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=1800)
+    launched = [l.split(" ", 1)[1] for l in res.stdout.splitlines() if l.startswith("LAUNCHED ")]
+    if res.returncode != 0 or not launched:
+        sys.stderr.write(res.stdout[-2000:] + res.stderr[-2000:])
+        raise RuntimeError("the counter run failed")
+    rows = []
+    for path in glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True):
+        with open(path) as f:
+            rows += [r for r in csv.DictReader(f) if r["Counter_Name"] == "GRBM_GUI_ACTIVE" and "aat" in r["Kernel_Name"]]
+    rows.sort(key=lambda r: int(r["Dispatch_Id"]))
+    # one kernel per launch for unsplit forward configurations: two dispatches per candidate, keep the second
+    if len(rows) != 2 * len(launched):
+        raise RuntimeError(f"{len(rows)} counted dispatches for {len(launched)} candidates")
+    by_name = {str(c): c for c in cfgs}
+    records = []
+    for i, name in enumerate(launched):
+        cfg = by_name[name]
+        records.append({"config": cfg.to_dict(), "cost_model_config": cost_model_tuple(cfg, args.dims),
+                        "cycles": int(float(rows[2 * i + 1]["Counter_Value"]) / XCDS),
+                        "lds_bytes": gfx950_space.forward_lds_bytes(cfg), "registers": gfx950_space.forward_reg_estimate(cfg)})
+    out = args.out or f"{args.op}_{args.dims[4]}_{args.dims[5]}_costmodel.json"
+    with open(out, "w") as f:
+        json.dump(records, f, indent=1)
+    best = min(records, key=lambda r: r["cycles"])
+    print(json.dumps({"candidates": len(records), "out": out, "fewest_cycles": best["cycles"],
+                      "best": str(by_name[launched[records.index(best)]])}))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
