@@ -59,24 +59,37 @@ def render(config, kind="kernel"):
     return text.format_map(fields)
 
 
-@functools.lru_cache(maxsize=1)
-def source_digest():
-    """Hash of every file that can change the machine code of a config library."""
+# kernel directories (under csrc/kernels) whose files can change the machine code of an operator's libraries;
+# csrc/kernels/utils and include/ count for every operator
+SOURCE_DIRS = {
+    "attn": ("attention/regfuse", "attention/smemfuse"),
+    "attn_bwd": ("attention/bwd",),
+    "ret": ("retnet/regfuse", "retnet/smemfuse"),
+    "ret_bwd": ("retnet/bwd",),
+    "ret_recurrent": ("retnet/recurrent",),
+}
+
+
+@functools.lru_cache(maxsize=None)
+def source_digest(operation):
+    """Hash of every file that can change the machine code of a config library of ``operation``."""
     h = hashlib.sha1()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for root in (os.path.join(CSRC_DIR, "kernels"), INCLUDE_DIR):
+    kernels = os.path.join(CSRC_DIR, "kernels")
+    roots = [os.path.join(kernels, "utils")] + [os.path.join(kernels, d) for d in SOURCE_DIRS[operation]] + [INCLUDE_DIR]
+    for root in roots:
         for dirpath, dirnames, filenames in sorted(os.walk(root)):
             dirnames.sort()
             for fn in sorted(filenames):
                 if fn.endswith((".h", ".py", ".hip")):
                     with open(os.path.join(dirpath, fn), "rb") as f:
-                        h.update(fn.encode())
+                        h.update(os.path.relpath(os.path.join(dirpath, fn), kernels).encode())
                         h.update(f.read())
     return h.hexdigest()[:10]
 
 
 def library_name(config):
-    return f"{config}-{source_digest()}.so"
+    return f"{config}-{source_digest(config.operation)}.so"
 
 
 def library_path(config, build_dir=None):

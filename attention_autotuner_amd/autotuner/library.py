@@ -53,6 +53,28 @@ def _bind(lib, op):
     return lib
 
 
+def _bind_recurrent(lib):
+    """The RetNet recurrent library: reference-named entry points instead of profile / kernel_entry."""
+    lib.abi_version.restype = _I
+    lib.abi_version.argtypes = []
+    lib.config_string.restype = ctypes.c_char_p
+    lib.config_string.argtypes = []
+    lib.workspace_size.restype = _SZ
+    lib.workspace_size.argtypes = [_I] * 4
+    dims = [_I] * 6                                   # batch, heads, kdim, vdim, l, block_kdim
+    lib.retnet_recurrent_fwd.restype = None
+    lib.retnet_recurrent_fwd.argtypes = [_VP] * 5 + dims
+    lib.retnet_recurrent_fwd_ex.restype = _I
+    lib.retnet_recurrent_fwd_ex.argtypes = [_VP] * 5 + dims + [_VP, _SZ, _VP]
+    lib.retnet_recurrent_profile.restype = _F
+    lib.retnet_recurrent_profile.argtypes = [_VP] * 5 + dims + [_VP, _SZ, _VP]
+    return lib
+
+
+def load_recurrent(path):
+    return load(path, "ret_recurrent")
+
+
 def load(path, op):
     """dlopen ``path`` once per process and set the prototypes for operator ``op``."""
     key = (path, op)
@@ -62,7 +84,7 @@ def load(path, op):
             lib = _handles.get(key)
             if lib is None:
                 try:
-                    lib = _bind(ctypes.CDLL(path), op)
+                    lib = _bind_recurrent(ctypes.CDLL(path)) if op == "ret_recurrent" else _bind(ctypes.CDLL(path), op)
                 except (OSError, AttributeError) as e:
                     raise KernelLibraryError(f"cannot load kernel library {path}: {e}") from e
                 _handles[key] = lib

@@ -104,6 +104,7 @@ def shipping_set(arch=None):
         if op == "ret":
             cfgs.append(gfx950_space.default_backward_config(dqk, dv, arch))
     cfgs += extra_configs(arch)
+    cfgs.append(supported_configs["ret_recurrent"]())
     cfgs += cached_configs()
     seen, unique = set(), []
     for c in cfgs:
@@ -134,13 +135,16 @@ def build_all(arch=None, force=True, timeout=600, verbose=True):
 def prune_stale(build_dir=None):
     """Delete libraries (and their sources / logs) built from an older revision of the kernel sources."""
     root = build_dir or codegen.DEFAULT_BUILD_DIR
-    keep = "-" + codegen.source_digest() + "."
     removed = 0
-    for dirpath, _, files in os.walk(root):
-        for fn in files:
-            if fn.endswith((".so", ".hip", ".log")) and keep not in fn:
-                os.remove(os.path.join(dirpath, fn))
-                removed += 1
+    for op in sorted(os.listdir(root)) if os.path.isdir(root) else []:
+        if op not in codegen.SOURCE_DIRS:
+            continue
+        keep = "-" + codegen.source_digest(op) + "."
+        for dirpath, _, files in os.walk(os.path.join(root, op)):
+            for fn in files:
+                if fn.endswith((".so", ".hip", ".log")) and keep not in fn:
+                    os.remove(os.path.join(dirpath, fn))
+                    removed += 1
     return removed
 
 

@@ -1,0 +1,131 @@
+"""Source text of the wrapper library for the RetNet recurrent form
+(same role as the ``extern "C" retnet_recurrent_fwd`` at the end of reference
+csrc/kernels/retnet/recurrent/recurrent.h:427-463, which the reference compiles straight into its
+benchmark, benchmarks/retnet/retnet.cu:175-215).
+
+One library holds every supported (key dims, value slice) instantiation and picks one per call, so the
+only field of the configuration record is a revision tag.
+"""
+
+global_vars = r"""
+#define AAT_OP_RET_RECURRENT 1
+#include "aat_kernel_abi.h"
+#include "kernels/retnet/recurrent/recurrent.h"
+#include "kernels/utils/host_launch.h"
+#include <mutex>
+
+namespace {{
+constexpr int kRevision = {revision};
+
+size_t factor_bytes(int heads, int l) {{ return (size_t)heads * (size_t)(l / 32) * aat::kRecFactorBytes; }}
+
+bool rec_shape_ok(int batch, int heads, int kdim, int vdim, int l, int block_kdim) {{
+  return batch > 0 && heads > 0 && l > 0 && l % 32 == 0 && l / 32 <= 4096 && (block_kdim == 64 || block_kdim == 128) &&
+         block_kdim <= kdim && vdim > 0 && vdim % 64 == 0;
+}}
+
+template <int KD, int DVS>
+hipError_t launch_one(const float* q, const float* k, const float* v, const char* factors, float* out, int batch,
+                      int heads, int kdim, int vdim, int l, hipStream_t stream) {{
+  using T = aat::RetRecurrent<KD, DVS>;
+  const auto kernel = &aat::retnet_recurrent_kernel<KD, DVS>;
+  static const hipError_t ok = aat::allow_lds(kernel, T::kSmemBytes);
+  if (ok != hipSuccess) return ok;
+  kernel<<<dim3(vdim / DVS, batch * heads), dim3(T::kThreads), T::kSmemBytes, stream>>>(q, k, v, factors, out, heads,
+                                                                                    kdim, vdim, l);
+  return hipGetLastError();
+}}
+
+// Two launches: the decay factors of every (head, chunk), then the scan.  A value slice of 128 dims per
+// block halves the traffic of q and k; 64 is taken when vdim asks for it or when 128 would leave most of
+// the compute units without a block.
+hipError_t launch(const float* q, const float* k, const float* v, const float* decay, float* out, int batch, int heads,
+                  int kdim, int vdim, int l, int block_kdim, char* factors, hipStream_t stream) {{
+  aat::retnet_recurrent_factors<<<dim3(heads), dim3(aat::kRecFactorThreads), (size_t)(l / 32) * 16, stream>>>(decay, factors, l);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const bool wide = vdim % 128 == 0 && (long)batch * heads * (vdim / 128) >= 192;
+  if (block_kdim == 128)
+    return wide ? launch_one<128, 128>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream)
+                : launch_one<128, 64>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream);
+  return wide ? launch_one<64, 128>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream)
+              : launch_one<64, 64>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream);
+}}
+
+// Workspace of the reference-signature entry point, which has no argument to bring one in: one buffer
+// per device, grown on demand, kept until the process ends.
+std::mutex g_ws_mutex;
+struct DeviceWorkspace {{ char* ptr = nullptr; size_t bytes = 0; }};
+DeviceWorkspace g_ws[64];
+
+char* cached_workspace(size_t bytes) {{
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(g_ws_mutex);
+  DeviceWorkspace& w = g_ws[dev];
+  if (w.bytes < bytes) {{
+    if (w.ptr != nullptr) {{
+      if (hipDeviceSynchronize() != hipSuccess) return nullptr;     // earlier launches may still read it
+      (void)hipFree(w.ptr);
+      w.ptr = nullptr;
+      w.bytes = 0;
+    }}
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) return nullptr;
+    w.ptr = static_cast<char*>(p);
+    w.bytes = bytes;
+  }}
+  return w.ptr;
+}}
+}}  // namespace
+"""
+
+kernel_code = global_vars + r"""
+extern "C" int abi_version(void) {{ return AAT_ABI_VERSION; }}
+extern "C" const char* config_string(void) {{ return "{config_name}"; }}
+extern "C" size_t workspace_size(int B, int H, int Seq_q, int Seq_k) {{
+  (void)B; (void)Seq_k;
+  return H > 0 && Seq_q > 0 ? factor_bytes(H, Seq_q) : 0;
+}}
+
+extern "C" int retnet_recurrent_fwd_ex(const float* q, const float* k, const float* v, const float* decay, float* out,
+                                       int batch, int heads, int kdim, int vdim, int l, int block_kdim,
+                                       void* workspace, size_t workspace_bytes, void* stream) {{
+  if (!rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim)) return AAT_ERR_SHAPE;
+  if (workspace == nullptr || workspace_bytes < factor_bytes(heads, l)) return AAT_ERR_WORKSPACE;
+  return (int)launch(q, k, v, decay, out, batch, heads, kdim, vdim, l, block_kdim, static_cast<char*>(workspace),
+                     static_cast<hipStream_t>(stream));
+}}
+
+extern "C" float retnet_recurrent_profile(const float* q, const float* k, const float* v, const float* decay, float* out,
+                                          int batch, int heads, int kdim, int vdim, int l, int block_kdim,
+                                          void* workspace, size_t workspace_bytes, void* stream) {{
+  if (!rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim)) return -1.f;
+  if (workspace == nullptr || workspace_bytes < factor_bytes(heads, l)) return -1.f;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return aat::timed_mean_ms(s, [&]() {{
+    return launch(q, k, v, decay, out, batch, heads, kdim, vdim, l, block_kdim, static_cast<char*>(workspace), s);
+  }});
+}}
+
+// The reference's own entry point: same name, same arguments, no status, null stream.  An unsupported
+// shape or a failed allocation is reported on stderr and leaves `out` untouched.
+extern "C" void retnet_recurrent_fwd(void* d_q, void* d_k, void* d_v, void* d_decay, void* d_out, int batch, int heads,
+                                     int kdim, int vdim, int l, int block_kdim) {{
+  if (!rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim)) {{
+    std::fprintf(stderr, "retnet_recurrent_fwd: unsupported shape (l %% 32 == 0, block_kdim 64 or 128, vdim %% 64 == 0)\n");
+    return;
+  }}
+  char* ws = cached_workspace(factor_bytes(heads, l));
+  if (ws == nullptr) {{
+    std::fprintf(stderr, "retnet_recurrent_fwd: cannot allocate %zu bytes of workspace\n", factor_bytes(heads, l));
+    return;
+  }}
+  const hipError_t e = launch(static_cast<const float*>(d_q), static_cast<const float*>(d_k), static_cast<const float*>(d_v),
+                              static_cast<const float*>(d_decay), static_cast<float*>(d_out), batch, heads, kdim, vdim, l,
+                              block_kdim, ws, nullptr);
+  if (e != hipSuccess) std::fprintf(stderr, "retnet_recurrent_fwd: %s\n", hipGetErrorString(e));
+}}
+"""
+
+profile_code = kernel_code

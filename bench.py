@@ -199,7 +199,31 @@ def side_measurements(aat, arch, Runtime, mk, steps, warmup):
     log(f"attention fwd long-kv: {ms:.4f} ms -> {res['attn_longkv_b1h32q256k16384d128']}")
     res.update(attention_backward_measurement(aat, arch, mk, steps, warmup))
     res.update(retnet_measurements(aat, arch, mk, steps, warmup))
+    res.update(retnet_recurrent_measurement(aat, steps, warmup))
     return res
+
+
+def retnet_recurrent_measurement(aat, steps, warmup):
+    """RetNet recurrent form at the shape of the reference's own bench (benchmarks/retnet/retnet.cu:236:
+    B 8, H 32, L 2048, 128 key and value dims, fp32).  5 flops per (position, key dim, value dim): the
+    recurrence's two multiply-adds and one multiply; fp32 MFMA peak 157.3 TFLOP/s."""
+    import torch
+    if not hasattr(aat, "retnet_recurrent_fwd"):
+        return {}
+    b, h, kd, vd, seqlen = 8, 32, 128, 128, 2048
+    g = torch.Generator(device="cuda").manual_seed(11)
+    q, k = (torch.rand(b, h, kd, seqlen, generator=g, device="cuda") * 2 - 1 for _ in range(2))
+    v = torch.rand(b, h, vd, seqlen, generator=g, device="cuda") * 2 - 1
+    decay = (1.0 - 2.0 ** (-5.0 - torch.arange(h, dtype=torch.float32, device="cuda"))).unsqueeze(1).expand(h, seqlen).contiguous()
+    out = torch.empty_like(v)
+    ws = torch.empty(h * (seqlen // 32) * 5120, dtype=torch.uint8, device="cuda")
+    _, ms = time_launches(lambda: aat.retnet_recurrent_fwd(q, k, v, decay, out=out, workspace=ws), steps, warmup)
+    flops = 5.0 * b * h * seqlen * kd * vd
+    nbytes = 4.0 * (q.numel() + k.numel() + v.numel() + out.numel())
+    res = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "frac_of_fp32_mfma_peak": round(flops / ms / 1e9 / 157.3, 3),
+           "gbps": round(nbytes / ms / 1e6, 1)}
+    log(f"retnet recurrent fwd: {ms:.4f} ms -> {res}")
+    return {"retnet_recurrent_b8h32s2048_dqk128_dv128_f32": res}
 
 
 def attention_backward_measurement(aat, arch, mk, steps, warmup):

@@ -3,7 +3,8 @@
  * The autotuner turns every candidate configuration (tile sizes, wave count, LDS buffering, fuse
  * type) into its own shared object, exactly as the reference does, and binds it with ctypes.  Each
  * such library exports the symbols declared below for ONE operator; which operator is selected at
- * compile time by defining AAT_OP_ATTN, AAT_OP_RET, AAT_OP_RET_BWD or AAT_OP_ATTN_BWD before including this header
+ * compile time by defining AAT_OP_ATTN, AAT_OP_RET, AAT_OP_RET_BWD, AAT_OP_ATTN_BWD or AAT_OP_RET_RECURRENT before
+ * including this header
  * (the generated wrapper does that, so the compiler checks the definitions against this file).
  *
  * Conventions (same as the reference unless stated):
@@ -32,7 +33,7 @@
 
 #include <stddef.h>
 
-#define AAT_ABI_VERSION 3
+#define AAT_ABI_VERSION 4
 #define AAT_ERR_SHAPE (-2)      /* Seq_q / Seq_k not divisible by the tile, or a non-positive size */
 #define AAT_ERR_WORKSPACE (-3)  /* workspace missing or smaller than workspace_size() */
 
@@ -131,6 +132,27 @@ int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, aat_half
                     aat_half* dq, aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k,
                     float softmax_scale, int causal, void* workspace, size_t workspace_bytes,
                     void* stream);
+
+#elif defined(AAT_OP_RET_RECURRENT)
+/* RetNet recurrent form, fp32:  S_n = decay[h][n] * S_{n-1} + k_n^T v_n,  out_n = q_n S_n  over the first
+ * block_kdim key dims.  q, k [batch, heads, kdim, l], v, out [batch, heads, vdim, l] (sequence contiguous),
+ * decay [heads, l]; every decay value is used as given (zero and negative ones included).
+ * Replaces: reference csrc/kernels/retnet/recurrent/recurrent.h:427 (retnet_recurrent_fwd, same name and
+ * arguments), whose only caller is benchmarks/retnet/retnet.cu:175-215.  This is ONE library for all
+ * supported shapes: l a multiple of 32 (the reference reads whole 2048-position chunks, :453-460),
+ * block_kdim 64 or 128 and <= kdim, vdim a multiple of 64.
+ * workspace_size(B, H, l, l) bytes of workspace hold the per-(head, chunk) decay factors.  The
+ * reference-signature entry point has no workspace argument: it is the one exception to "nothing is
+ * allocated by the callee" -- it keeps one buffer per device, grown on demand, until the process ends,
+ * launches on the null stream and reports errors on stderr. */
+void retnet_recurrent_fwd(void* d_q, void* d_k, void* d_v, void* d_decay, void* d_out, int batch, int heads,
+                          int kdim, int vdim, int l, int block_kdim);
+int retnet_recurrent_fwd_ex(const float* q, const float* k, const float* v, const float* decay, float* out,
+                            int batch, int heads, int kdim, int vdim, int l, int block_kdim, void* workspace,
+                            size_t workspace_bytes, void* stream);
+float retnet_recurrent_profile(const float* q, const float* k, const float* v, const float* decay, float* out,
+                               int batch, int heads, int kdim, int vdim, int l, int block_kdim, void* workspace,
+                               size_t workspace_bytes, void* stream);
 #endif
 
 #ifdef __cplusplus

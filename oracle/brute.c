@@ -1,9 +1,11 @@
-/* fp64 brute-force loops for attention forward, RetNet forward and RetNet backward.
+/* fp64 brute-force loops for attention forward, RetNet forward, RetNet backward and the RetNet recurrent form.
  *
  * TEST INFRASTRUCTURE ONLY.  This file is an independent restatement (plain loops, double
  * precision, no tiling, no library calls besides exp) used to pin oracle/ref_op.py, which in turn
  * checks the HIP kernels.  Formulas: reference python/utils/ref_op.py:2-13 and, for the gradients,
- * reference csrc/kernels/retnet/bwd/bwd_colblock.h:522-576.
+ * reference csrc/kernels/retnet/bwd/bwd_colblock.h:522-576; the recurrent form restates the scan of
+ * reference csrc/kernels/retnet/recurrent/recurrent.h:110-114 (the pair operator) and :303-330 (one scan per
+ * (key dim, value dim) pair, seeded with (0, 0), its .y component weighted by q and summed over key dims).
  *
  * All tensors are contiguous fp32: q [BH,Sq,Kd], k [BH,Sk,Kd], v [BH,Sk,D], mask [H,Sq,Sk] (the
  * head of slice b is b % H), outputs likewise.  Built by oracle/Makefile into oracle/libbrute.so.
@@ -109,4 +111,30 @@ void brute_retnet_bwd(const float* q, const float* k, const float* v, const floa
   }
   free(P);
   free(dS);
+}
+
+/* RetNet recurrent form.  q, k [BH][kdim][L], v, out [BH][vdim][L] (sequence contiguous), decay [H][L]:
+ *   S(kd, vd, n) = decay[n] * S(kd, vd, n-1) + k[kd][n] * v[vd][n],  S(., ., -1) = 0
+ *   out[vd][n]   = sum_{kd < block_kdim} q[kd][n] * S(kd, vd, n) */
+void brute_retnet_recurrent(const float* q, const float* k, const float* v, const float* decay, float* out,
+                            int BH, int H, int kdim, int vdim, int L, int block_kdim) {
+  double* acc = (double*)malloc(sizeof(double) * (size_t)L);
+  for (int b = 0; b < BH; ++b) {
+    const float* a = decay + (size_t)(b % H) * L;
+    for (int vd = 0; vd < vdim; ++vd) {
+      const float* vr = v + ((size_t)b * vdim + vd) * L;
+      for (int n = 0; n < L; ++n) acc[n] = 0;
+      for (int kd = 0; kd < block_kdim; ++kd) {
+        const float* kr = k + ((size_t)b * kdim + kd) * L;
+        const float* qr = q + ((size_t)b * kdim + kd) * L;
+        double S = 0;
+        for (int n = 0; n < L; ++n) {
+          S = (double)a[n] * S + (double)kr[n] * (double)vr[n];
+          acc[n] += (double)qr[n] * S;
+        }
+      }
+      for (int n = 0; n < L; ++n) out[((size_t)b * vdim + vd) * L + n] = (float)acc[n];
+    }
+  }
+  free(acc);
 }

@@ -62,3 +62,15 @@ def retnet_bwd(q, k, v, mask, do):
     dq, dk, dv = np.empty_like(q), np.empty_like(k), np.empty_like(v)
     _lib().brute_retnet_bwd(_p(q), _p(k), _p(v), _p(mask), _p(do), _p(dq), _p(dk), _p(dv), bh, h, sq, sk, kd, d)
     return dq, dk, dv
+
+
+def retnet_recurrent(q, k, v, decay, block_kdim=None):
+    """q, k [..., kdim, L], v [..., vdim, L], decay [H, L] -> out [..., vdim, L] (fp64 recurrence, fp32 result)."""
+    q, k, v, decay = _c(q), _c(k), _c(v), _c(decay)
+    bh = int(np.prod(q.shape[:-2]))
+    kdim, l = q.shape[-2:]
+    vdim = v.shape[-2]
+    out = np.empty(v.shape, dtype=np.float32)
+    _lib().brute_retnet_recurrent(_p(q), _p(k), _p(v), _p(decay), _p(out), bh, decay.shape[0], kdim, vdim, l,
+                                  int(block_kdim or kdim))
+    return out

@@ -19,6 +19,11 @@ reference uses as its own correctness check:
   ``dV = P^T dO``, ``dS = (dO V^T / r) * mask``, ``dK = dS^T Q``, ``dQ = dS K``.
 * ``retnet_decay_mask`` is the decay matrix of the benchmark configuration:
   ``D[h, n, m] = gamma_h^(n-m)`` for n >= m else 0, ``gamma_h = 1 - 2^(-5-h)``.
+* ``retnet_recurrent_ref`` is the closed form of the recurrent scan of reference
+  csrc/kernels/retnet/recurrent/recurrent.h:110-114,303-330 (``S_n = a_n S_{n-1} + k_n^T v_n``,
+  ``out_n = q_n S_n`` over the first ``block_kdim`` key dims, fp32 tensors laid out [B, H, dim, L]):
+  ``out = V (K^T Q * D)`` with ``D[m, n] = prod_{m<j<=n} a_j`` for m <= n, else 0, in fp64.  The products
+  are taken literally (no logarithms), so zero and negative decays mean what they mean in the scan.
 * ``attention_online_ref`` / ``retnet_online_ref`` restate the tile-by-tile recurrences sketched in
   reference README.md:81-99 and python/tests/attntuner_demo.py:59-97,122-161; they exist so a test
   can show the online form equals the one-shot form.
@@ -108,6 +113,27 @@ def retnet_decay_mask(nheads, seq_q, seq_k, dtype=torch.float16):
     gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(nheads, dtype=torch.float64)).view(nheads, 1, 1)
     d = torch.where(n >= m, gamma ** (n - m).clamp(min=0), torch.zeros((), dtype=torch.float64))
     return d.to(dtype) if dtype == torch.float64 else d.to(torch.float32).to(dtype)
+
+
+def retnet_recurrent_decay_matrix(decay):
+    """decay [H, L] -> D [H, L(m), L(n)] fp64, D[h, m, n] = prod_{m<j<=n} decay[h, j] for m <= n, 0 below."""
+    a = decay.detach().to(device="cpu", dtype=torch.float64)
+    nheads, seqlen = a.shape
+    d = torch.zeros(nheads, seqlen, seqlen, dtype=torch.float64)
+    for m in range(seqlen):
+        d[:, m, m] = 1.0
+        if m + 1 < seqlen:
+            d[:, m, m + 1:] = torch.cumprod(a[:, m + 1:], dim=-1)
+    return d
+
+
+def retnet_recurrent_ref(q, k, v, decay, block_kdim=None):
+    """q, k [B, H, kdim, L], v [B, H, vdim, L], decay [H, L] -> out [B, H, vdim, L] (fp64 math, fp32 result)."""
+    q, k, v = (x.detach().to(device="cpu", dtype=torch.float64) for x in (q, k, v))
+    kd = block_kdim or q.shape[2]
+    s = k[:, :, :kd].transpose(-1, -2) @ q[:, :, :kd]            # [B, H, L(m), L(n)]
+    p = s * retnet_recurrent_decay_matrix(decay).unsqueeze(0)
+    return (v @ p).to(torch.float32)
 
 
 def attention_online_ref(q, k, v, softmax_scale=None, causal=False, block_kv=64):

@@ -34,6 +34,9 @@ def test_header_declares_the_reference_pair_for_every_operator():
         assert _declared_symbols(macro) == sorted(pair + ["kernel_entry_decay", "profile_decay"])
     # the attention backward has no reference signature to keep: only the extended entry points
     assert _declared_symbols("AAT_OP_ATTN_BWD") == ["abi_version", "config_string", "kernel_entry_ex", "profile_ex", "workspace_size"]
+    # the recurrent form keeps the reference's own entry-point name (reference recurrent.h:427)
+    assert _declared_symbols("AAT_OP_RET_RECURRENT") == ["abi_version", "config_string", "retnet_recurrent_fwd",
+                                                         "retnet_recurrent_fwd_ex", "retnet_recurrent_profile", "workspace_size"]
 
 
 def test_wrapper_text_carries_the_configuration():
@@ -51,7 +54,8 @@ def test_wrapper_text_carries_the_configuration():
 def test_shipping_set_is_built_and_exports_the_abi():
     cfgs = prebuilt.shipping_set(ARCH)
     assert cfgs
-    macro = {"attn": "AAT_OP_ATTN", "ret": "AAT_OP_RET", "ret_bwd": "AAT_OP_RET_BWD", "attn_bwd": "AAT_OP_ATTN_BWD"}
+    macro = {"attn": "AAT_OP_ATTN", "ret": "AAT_OP_RET", "ret_bwd": "AAT_OP_RET_BWD", "attn_bwd": "AAT_OP_ATTN_BWD",
+             "ret_recurrent": "AAT_OP_RET_RECURRENT"}
     assert {c.operation for c in cfgs} == set(macro)
     for cfg in cfgs:
         path = codegen.compile_config(cfg, ARCH, timeout=600)          # already built by build(); builds if not
@@ -60,9 +64,11 @@ def test_shipping_set_is_built_and_exports_the_abi():
         for name in _declared_symbols(macro[cfg.operation]):
             assert hasattr(raw, name), (cfg, name)
         lib = library.load(path, cfg.operation)
-        assert lib.abi_version() == 3
+        assert lib.abi_version() == 4
         assert lib.config_string().decode() == f"{cfg.operation}:{cfg}"
-        if cfg.operation == "attn_bwd":
+        if cfg.operation == "ret_recurrent":
+            assert lib.workspace_size(8, 4, 2048, 2048) == 4 * (2048 // 32) * 5120    # one factor record per (head, chunk)
+        elif cfg.operation == "attn_bwd":
             assert lib.workspace_size(2, 3, 256, 512) == 2 * 2 * 3 * 256 * 4      # lse2 + delta, fp32 per query row
         elif getattr(cfg, "kv_splits", 1) == 1:
             assert lib.workspace_size(1, 1, 256, 256) == 0
@@ -145,3 +151,6 @@ def test_ops_refuse_cpu_tensors():
         aat.flash_attn_func(q, q, q, ARCH)
     with pytest.raises(RuntimeError, match="GPU only"):
         aat.RetNetAttnFunc(q, q, q, torch.zeros(1, 128, 128, dtype=torch.float16), ARCH)
+    x = torch.zeros(1, 1, 64, 32)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        aat.retnet_recurrent_fwd(x, x, x, torch.ones(1, 32))

@@ -248,3 +248,74 @@ def test_attention_bwd_closed_forms():
     # causal, first query row sees one key: P = 1 there, so dS = P (dP - delta) = 0 and dQ[0] = 0
     dqc, _, dvc = ref_op.attention_bwd_ref(q, k, v, d1, None, True)
     assert dqc[..., 0, :].abs().max() < 1e-6
+
+
+# ---------------------------------------------------------------------------------------------------
+# RetNet recurrent form: two independent statements (a sequential fp64 recurrence in C, the parallel
+# closed form in torch) pinned against each other and against what the mathematics fixes.
+def _recurrent_inputs(seed, b=2, h=3, kdim=8, vdim=5, seqlen=37, lo=-1.0, hi=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.rand(b, h, kdim, seqlen, generator=g) * 2 - 1
+    k = torch.rand(b, h, kdim, seqlen, generator=g) * 2 - 1
+    v = torch.rand(b, h, vdim, seqlen, generator=g) * 2 - 1
+    decay = torch.rand(h, seqlen, generator=g) * (hi - lo) + lo
+    return q, k, v, decay
+
+
+def test_recurrent_closed_form_matches_the_sequential_recurrence():
+    q, k, v, decay = _recurrent_inputs(0)
+    decay[0, 5] = 0.0                      # a zero cuts the history, negative values flip signs
+    decay[1, 9] = -0.75
+    closed = ref_op.retnet_recurrent_ref(q, k, v, decay)
+    scan = torch.from_numpy(brute.retnet_recurrent(q.numpy(), k.numpy(), v.numpy(), decay.numpy()))
+    assert torch.allclose(closed, scan, atol=2e-6, rtol=1e-5)
+    # only the first block_kdim key dims take part
+    part = ref_op.retnet_recurrent_ref(q, k, v, decay, block_kdim=3)
+    scan3 = torch.from_numpy(brute.retnet_recurrent(q.numpy(), k.numpy(), v.numpy(), decay.numpy(), block_kdim=3))
+    assert torch.allclose(part, scan3, atol=2e-6, rtol=1e-5)
+    assert torch.allclose(part, ref_op.retnet_recurrent_ref(q[:, :, :3], k[:, :, :3], v, decay), atol=1e-6)
+    assert not torch.allclose(part, closed, atol=1e-3)
+
+
+def test_recurrent_special_cases():
+    q, k, v, decay = _recurrent_inputs(1, seqlen=24)
+    h, seqlen = decay.shape
+    # decay 1: causal linear attention, out = V tril(K^T Q)
+    ones = torch.ones(h, seqlen)
+    s = k.transpose(-1, -2).double() @ q.double()
+    expect = (v.double() @ torch.triu(s)).float()            # [m, n] kept for m <= n
+    assert torch.allclose(ref_op.retnet_recurrent_ref(q, k, v, ones), expect, atol=1e-5)
+    assert torch.allclose(torch.from_numpy(brute.retnet_recurrent(q.numpy(), k.numpy(), v.numpy(), ones.numpy())), expect, atol=1e-5)
+    # decay 0: no history, out_n = (q_n . k_n) v_n
+    zeros = torch.zeros(h, seqlen)
+    expect0 = (q * k).sum(dim=2, keepdim=True) * v
+    assert torch.allclose(ref_op.retnet_recurrent_ref(q, k, v, zeros), expect0, atol=1e-6)
+    assert torch.allclose(torch.from_numpy(brute.retnet_recurrent(q.numpy(), k.numpy(), v.numpy(), zeros.numpy())), expect0, atol=1e-6)
+    # decay matrix entries: diagonal 1, first superdiagonal a_n, zero below the diagonal
+    d = ref_op.retnet_recurrent_decay_matrix(decay)
+    assert torch.equal(torch.diagonal(d, dim1=1, dim2=2), torch.ones(h, seqlen, dtype=torch.float64))
+    assert torch.allclose(torch.diagonal(d, offset=1, dim1=1, dim2=2), decay[:, 1:].double())
+    assert torch.equal(torch.tril(d, diagonal=-1), torch.zeros_like(d))
+    assert torch.allclose(d[:, 2, 7], decay[:, 3:8].double().prod(dim=-1))
+    # linear in v and in q
+    q2, _, v2, _ = _recurrent_inputs(2, seqlen=24)
+    lhs = ref_op.retnet_recurrent_ref(q, k, v + 2 * v2, decay)
+    assert torch.allclose(lhs, ref_op.retnet_recurrent_ref(q, k, v, decay) + 2 * ref_op.retnet_recurrent_ref(q, k, v2, decay), atol=1e-5)
+    lhs = ref_op.retnet_recurrent_ref(q - q2, k, v, decay)
+    assert torch.allclose(lhs, ref_op.retnet_recurrent_ref(q, k, v, decay) - ref_op.retnet_recurrent_ref(q2, k, v, decay), atol=1e-5)
+
+
+def test_recurrent_form_equals_parallel_retention_for_a_constant_decay():
+    """With decay[h, n] = gamma_h the scan is the numerator of parallel retention under the decay mask."""
+    b, h, seqlen, kdim, vdim = 1, 2, 32, 16, 8
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(b, h, seqlen, kdim, generator=g)
+    k = torch.randn(b, h, seqlen, kdim, generator=g)
+    v = torch.randn(b, h, seqlen, vdim, generator=g)
+    mask = ref_op.retnet_decay_mask(h, seqlen, seqlen, dtype=torch.float32)
+    o, r = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    numerator = o * r.unsqueeze(-1)                              # undo the normalisation: (q k^T * mask) v
+    gamma = 1.0 - 2.0 ** (-5.0 - torch.arange(h, dtype=torch.float32))
+    decay = gamma.unsqueeze(1).expand(h, seqlen).contiguous()
+    out = ref_op.retnet_recurrent_ref(q.transpose(-1, -2), k.transpose(-1, -2), v.transpose(-1, -2), decay)
+    assert torch.allclose(out.transpose(-1, -2), numerator, atol=2e-4, rtol=1e-4)
