@@ -62,6 +62,8 @@ def _bind_recurrent(lib):
     lib.workspace_size.restype = _SZ
     lib.workspace_size.argtypes = [_I] * 4
     dims = [_I] * 6                                   # batch, heads, kdim, vdim, l, block_kdim
+    lib.retnet_recurrent_workspace_size.restype = _SZ
+    lib.retnet_recurrent_workspace_size.argtypes = dims
     lib.retnet_recurrent_fwd.restype = None
     lib.retnet_recurrent_fwd.argtypes = [_VP] * 5 + dims
     lib.retnet_recurrent_fwd_ex.restype = _I

@@ -17,11 +17,28 @@ global_vars = r"""
 namespace {{
 constexpr int kRevision = {revision};
 
+constexpr int kMaxKdim = 256;                     // the reference's MAX_KDIM (reference recurrent.h:18)
+
 size_t factor_bytes(int heads, int l) {{ return (size_t)heads * (size_t)(l / 32) * aat::kRecFactorBytes; }}
+// More than 128 key dims are contracted in passes of 128 (or 64) whose outputs add; every pass but the
+// first writes into a second output-sized buffer behind the decay factors.
+size_t total_workspace_bytes(int batch, int heads, int vdim, int l, int block_kdim) {{
+  const size_t f = (factor_bytes(heads, l) + 255) / 256 * 256;
+  return block_kdim > 128 ? f + (size_t)batch * heads * vdim * l * sizeof(float) : f;
+}}
 
 bool rec_shape_ok(int batch, int heads, int kdim, int vdim, int l, int block_kdim) {{
-  return batch > 0 && heads > 0 && l > 0 && l % 32 == 0 && l / 32 <= 4096 && (block_kdim == 64 || block_kdim == 128) &&
-         block_kdim <= kdim && vdim > 0 && vdim % 64 == 0;
+  return batch > 0 && heads > 0 && l > 0 && l % 32 == 0 && l / 32 <= 4096 && block_kdim >= 64 && block_kdim % 64 == 0 &&
+         block_kdim <= kMaxKdim && block_kdim <= kdim && vdim > 0 && vdim % 64 == 0;
+}}
+
+__global__ void rec_add_kernel(float4* __restrict__ out, const float4* __restrict__ part, size_t n4) {{
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {{
+    float4 a = out[i];
+    const float4 b = part[i];
+    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    out[i] = a;
+  }}
 }}
 
 template <int KD, int DVS>
@@ -40,16 +57,31 @@ hipError_t launch_one(const float* q, const float* k, const float* v, const char
 // block halves the traffic of q and k; 64 is taken when vdim asks for it or when 128 would leave most of
 // the compute units without a block.
 hipError_t launch(const float* q, const float* k, const float* v, const float* decay, float* out, int batch, int heads,
-                  int kdim, int vdim, int l, int block_kdim, char* factors, hipStream_t stream) {{
+                  int kdim, int vdim, int l, int block_kdim, char* workspace, hipStream_t stream) {{
+  char* factors = workspace;
+  float* part = reinterpret_cast<float*>(workspace + (factor_bytes(heads, l) + 255) / 256 * 256);
   aat::retnet_recurrent_factors<<<dim3(heads), dim3(aat::kRecFactorThreads), (size_t)(l / 32) * 16, stream>>>(decay, factors, l);
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
   const bool wide = vdim % 128 == 0 && (long)batch * heads * (vdim / 128) >= 192;
-  if (block_kdim == 128)
-    return wide ? launch_one<128, 128>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream)
-                : launch_one<128, 64>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream);
-  return wide ? launch_one<64, 128>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream)
-              : launch_one<64, 64>(q, k, v, factors, out, batch, heads, kdim, vdim, l, stream);
+  for (int kd0 = 0; kd0 < block_kdim && e == hipSuccess; ) {{
+    const int kd = block_kdim - kd0 >= 128 ? 128 : 64;                 // key dims of this pass
+    const float* qp = q + (size_t)kd0 * l;                             // rows kd0.. of every (batch, head) slice
+    const float* kp = k + (size_t)kd0 * l;
+    float* dst = kd0 == 0 ? out : part;
+    if (kd == 128)
+      e = wide ? launch_one<128, 128>(qp, kp, v, factors, dst, batch, heads, kdim, vdim, l, stream)
+               : launch_one<128, 64>(qp, kp, v, factors, dst, batch, heads, kdim, vdim, l, stream);
+    else
+      e = wide ? launch_one<64, 128>(qp, kp, v, factors, dst, batch, heads, kdim, vdim, l, stream)
+               : launch_one<64, 64>(qp, kp, v, factors, dst, batch, heads, kdim, vdim, l, stream);
+    if (e == hipSuccess && kd0 > 0) {{
+      const size_t n4 = (size_t)batch * heads * vdim * l / 4;
+      rec_add_kernel<<<dim3(2048), dim3(256), 0, stream>>>(reinterpret_cast<float4*>(out), reinterpret_cast<const float4*>(part), n4);
+      e = hipGetLastError();
+    }}
+    kd0 += kd;
+  }}
+  return e;
 }}
 
 // Workspace of the reference-signature entry point, which has no argument to bring one in: one buffer
@@ -84,15 +116,19 @@ kernel_code = global_vars + r"""
 extern "C" int abi_version(void) {{ return AAT_ABI_VERSION; }}
 extern "C" const char* config_string(void) {{ return "{config_name}"; }}
 extern "C" size_t workspace_size(int B, int H, int Seq_q, int Seq_k) {{
-  (void)B; (void)Seq_k;
-  return H > 0 && Seq_q > 0 ? factor_bytes(H, Seq_q) : 0;
+  (void)B; (void)Seq_k;                           // up to 128 key dims; retnet_recurrent_workspace_size covers every case
+  return H > 0 && Seq_q > 0 ? (factor_bytes(H, Seq_q) + 255) / 256 * 256 : 0;
+}}
+
+extern "C" size_t retnet_recurrent_workspace_size(int batch, int heads, int kdim, int vdim, int l, int block_kdim) {{
+  return rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim) ? total_workspace_bytes(batch, heads, vdim, l, block_kdim) : 0;
 }}
 
 extern "C" int retnet_recurrent_fwd_ex(const float* q, const float* k, const float* v, const float* decay, float* out,
                                        int batch, int heads, int kdim, int vdim, int l, int block_kdim,
                                        void* workspace, size_t workspace_bytes, void* stream) {{
   if (!rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim)) return AAT_ERR_SHAPE;
-  if (workspace == nullptr || workspace_bytes < factor_bytes(heads, l)) return AAT_ERR_WORKSPACE;
+  if (workspace == nullptr || workspace_bytes < total_workspace_bytes(batch, heads, vdim, l, block_kdim)) return AAT_ERR_WORKSPACE;
   return (int)launch(q, k, v, decay, out, batch, heads, kdim, vdim, l, block_kdim, static_cast<char*>(workspace),
                      static_cast<hipStream_t>(stream));
 }}
@@ -101,7 +137,7 @@ extern "C" float retnet_recurrent_profile(const float* q, const float* k, const 
                                           int batch, int heads, int kdim, int vdim, int l, int block_kdim,
                                           void* workspace, size_t workspace_bytes, void* stream) {{
   if (!rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim)) return -1.f;
-  if (workspace == nullptr || workspace_bytes < factor_bytes(heads, l)) return -1.f;
+  if (workspace == nullptr || workspace_bytes < total_workspace_bytes(batch, heads, vdim, l, block_kdim)) return -1.f;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return aat::timed_mean_ms(s, [&]() {{
     return launch(q, k, v, decay, out, batch, heads, kdim, vdim, l, block_kdim, static_cast<char*>(workspace), s);
@@ -113,12 +149,13 @@ extern "C" float retnet_recurrent_profile(const float* q, const float* k, const 
 extern "C" void retnet_recurrent_fwd(void* d_q, void* d_k, void* d_v, void* d_decay, void* d_out, int batch, int heads,
                                      int kdim, int vdim, int l, int block_kdim) {{
   if (!rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim)) {{
-    std::fprintf(stderr, "retnet_recurrent_fwd: unsupported shape (l %% 32 == 0, block_kdim 64 or 128, vdim %% 64 == 0)\n");
+    std::fprintf(stderr, "retnet_recurrent_fwd: unsupported shape (l %% 32 == 0, block_kdim a multiple of 64 up to 256, vdim %% 64 == 0)\n");
     return;
   }}
-  char* ws = cached_workspace(factor_bytes(heads, l));
+  const size_t need = total_workspace_bytes(batch, heads, vdim, l, block_kdim);
+  char* ws = cached_workspace(need);
   if (ws == nullptr) {{
-    std::fprintf(stderr, "retnet_recurrent_fwd: cannot allocate %zu bytes of workspace\n", factor_bytes(heads, l));
+    std::fprintf(stderr, "retnet_recurrent_fwd: cannot allocate %zu bytes of workspace\n", need);
     return;
   }}
   const hipError_t e = launch(static_cast<const float*>(d_q), static_cast<const float*>(d_k), static_cast<const float*>(d_v),

@@ -18,8 +18,8 @@ from ..autotuner import codegen, library
 from ..autotuner.configs import RetRecurrentConfig
 from ..autotuner.runtime import KernelLaunchError
 
-_ERRORS = {-2: "unsupported shape: L must be a multiple of 32 (at most 131072), block_kdim 64 or 128 and <= kdim, "
-               "vdim a multiple of 64",
+_ERRORS = {-2: "unsupported shape: L must be a multiple of 32 (at most 131072), block_kdim a multiple of 64 up to 256 "
+               "and <= kdim, vdim a multiple of 64",
            -3: "workspace missing or too small"}
 
 
@@ -32,9 +32,11 @@ def _library(device_type):
     return library.load_recurrent(path)
 
 
-def workspace_size(nheads, seqlen, device_type=None):
-    """Bytes of workspace one call needs (the decay factors of every (head, 32-position chunk))."""
-    return int(_library(device_type or MI355X()).workspace_size(1, nheads, seqlen, seqlen))
+def workspace_size(nheads, seqlen, device_type=None, batch=1, kdim=128, vdim=128, block_kdim=None):
+    """Bytes of workspace one call needs: the decay factors of every (head, 32-position chunk) and, beyond 128
+    key dims, a second output-sized buffer (0 for an unsupported shape)."""
+    return int(_library(device_type or MI355X()).retnet_recurrent_workspace_size(batch, nheads, kdim, vdim, seqlen,
+                                                                                  int(block_kdim or kdim)))
 
 
 def retnet_recurrent_fwd(q, k, v, decay, device_type=None, block_kdim=None, out=None, workspace=None):
@@ -51,7 +53,7 @@ def retnet_recurrent_fwd(q, k, v, decay, device_type=None, block_kdim=None, out=
     if out is None:
         out = torch.empty_like(v)
     assert out.shape == v.shape and out.dtype == torch.float32 and out.is_contiguous() and out.device == v.device
-    need = int(lib.workspace_size(batch, nheads, seqlen, seqlen))
+    need = int(lib.retnet_recurrent_workspace_size(batch, nheads, kdim, vdim, seqlen, block_kdim))
     if workspace is None or workspace.numel() * workspace.element_size() < need:
         workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):

@@ -140,13 +140,16 @@ int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, aat_half
  * Replaces: reference csrc/kernels/retnet/recurrent/recurrent.h:427 (retnet_recurrent_fwd, same name and
  * arguments), whose only caller is benchmarks/retnet/retnet.cu:175-215.  This is ONE library for all
  * supported shapes: l a multiple of 32 (the reference reads whole 2048-position chunks, :453-460),
- * block_kdim 64 or 128 and <= kdim, vdim a multiple of 64.
- * workspace_size(B, H, l, l) bytes of workspace hold the per-(head, chunk) decay factors.  The
+ * block_kdim a multiple of 64 up to 256 (the reference's MAX_KDIM, :18) and <= kdim, vdim a multiple of 64.
+ * retnet_recurrent_workspace_size() bytes of workspace hold the per-(head, chunk) decay factors and, for
+ * more than 128 key dims (contracted in passes of 128 whose outputs add), a second output-sized buffer;
+ * workspace_size(B, H, l, l) is the same figure for up to 128 key dims.  The
  * reference-signature entry point has no workspace argument: it is the one exception to "nothing is
  * allocated by the callee" -- it keeps one buffer per device, grown on demand, until the process ends,
  * launches on the null stream and reports errors on stderr. */
 void retnet_recurrent_fwd(void* d_q, void* d_k, void* d_v, void* d_decay, void* d_out, int batch, int heads,
                           int kdim, int vdim, int l, int block_kdim);
+size_t retnet_recurrent_workspace_size(int batch, int heads, int kdim, int vdim, int l, int block_kdim);
 int retnet_recurrent_fwd_ex(const float* q, const float* k, const float* v, const float* decay, float* out,
                             int batch, int heads, int kdim, int vdim, int l, int block_kdim, void* workspace,
                             size_t workspace_bytes, void* stream);

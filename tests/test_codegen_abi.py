@@ -36,7 +36,8 @@ def test_header_declares_the_reference_pair_for_every_operator():
     assert _declared_symbols("AAT_OP_ATTN_BWD") == ["abi_version", "config_string", "kernel_entry_ex", "profile_ex", "workspace_size"]
     # the recurrent form keeps the reference's own entry-point name (reference recurrent.h:427)
     assert _declared_symbols("AAT_OP_RET_RECURRENT") == ["abi_version", "config_string", "retnet_recurrent_fwd",
-                                                         "retnet_recurrent_fwd_ex", "retnet_recurrent_profile", "workspace_size"]
+                                                         "retnet_recurrent_fwd_ex", "retnet_recurrent_profile",
+                                                         "retnet_recurrent_workspace_size", "workspace_size"]
 
 
 def test_wrapper_text_carries_the_configuration():
@@ -67,7 +68,12 @@ def test_shipping_set_is_built_and_exports_the_abi():
         assert lib.abi_version() == 4
         assert lib.config_string().decode() == f"{cfg.operation}:{cfg}"
         if cfg.operation == "ret_recurrent":
-            assert lib.workspace_size(8, 4, 2048, 2048) == 4 * (2048 // 32) * 5120    # one factor record per (head, chunk)
+            factors = 4 * (2048 // 32) * 5120                                         # one record per (head, chunk)
+            assert lib.workspace_size(8, 4, 2048, 2048) == factors
+            assert lib.retnet_recurrent_workspace_size(8, 4, 128, 64, 2048, 128) == factors
+            # beyond 128 key dims: plus a second output-sized buffer for the passes that add
+            assert lib.retnet_recurrent_workspace_size(8, 4, 256, 64, 2048, 256) == factors + 8 * 4 * 64 * 2048 * 4
+            assert lib.retnet_recurrent_workspace_size(8, 4, 256, 64, 2000, 256) == 0     # unsupported shape
         elif cfg.operation == "attn_bwd":
             assert lib.workspace_size(2, 3, 256, 512) == 2 * 2 * 3 * 256 * 4      # lse2 + delta, fp32 per query row
         elif getattr(cfg, "kv_splits", 1) == 1:

@@ -35,9 +35,10 @@ def _close(got, ref):
 
 
 # value slices of 64 and 128 dims, 64 and 128 key dims, few and many blocks (both launch shapes), ragged
-# chunk counts (odd number of 32-position chunks), a single chunk
+# chunk counts (odd number of 32-position chunks), a single chunk, more than 128 key dims (passes that add)
 @pytest.mark.parametrize("b,h,kdim,vdim,seqlen", [(1, 2, 128, 128, 256), (1, 3, 64, 256, 96), (2, 1, 128, 64, 32),
-                                                   (1, 2, 64, 64, 160), (2, 2, 64, 192, 64)])
+                                                   (1, 2, 64, 64, 160), (2, 2, 64, 192, 64), (1, 2, 256, 64, 96),
+                                                   (1, 1, 192, 128, 64)])
 def test_matches_the_closed_form(b, h, kdim, vdim, seqlen):
     q, k, v, decay = _inputs(0, b, h, kdim, vdim, seqlen, 0.5, 1.0)
     out = aat.retnet_recurrent_fwd(q.cuda(), k.cuda(), v.cuda(), decay.cuda())
@@ -106,6 +107,7 @@ def test_reference_signature_entry_point_and_error_codes():
     assert call((b, h, kdim, vdim, seqlen, kdim), ctypes.c_void_p(0), 0) == -3
     assert call((b, h, kdim, vdim, 100, kdim), ptr(ws), need) == -2         # l not a multiple of 32
     assert call((b, h, kdim, vdim, seqlen, 32), ptr(ws), need) == -2        # block_kdim
+    assert call((b, h, kdim, vdim, seqlen, 128), ptr(ws), need) == -2       # block_kdim > kdim
     assert call((b, h, kdim, 32, seqlen, kdim), ptr(ws), need) == -2        # vdim
     assert call((0, h, kdim, vdim, seqlen, kdim), ptr(ws), need) == -2
     torch.cuda.synchronize()
