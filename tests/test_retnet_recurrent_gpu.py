@@ -153,3 +153,46 @@ def test_full_size_through_size_independent_properties():
     sl = (slice(3, 4), slice(17, 18))
     ref = brute.retnet_recurrent(q[sl].cpu().numpy(), k[sl].cpu().numpy(), v[sl].cpu().numpy(), decay[17:18].cpu().numpy())
     _close(o1[sl], torch.from_numpy(ref))
+
+
+def test_long_sequence_and_side_stream():
+    """128 chunks per head (the carried product leaves its range several times), launched on a side stream."""
+    q, k, v, decay = _inputs(8, 1, 2, 64, 64, 4096, 0.6, 1.0)
+    side = torch.cuda.Stream()
+    qc, kc, vc, dc = q.cuda(), k.cuda(), v.cuda(), decay.cuda()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        out = aat.retnet_recurrent_fwd(qc, kc, vc, dc)
+    side.synchronize()
+    ref = torch.from_numpy(brute.retnet_recurrent(q.numpy(), k.numpy(), v.numpy(), decay.numpy()))
+    _close(out, ref)
+
+
+def test_graph_capture_replays():
+    """The extended entry point allocates nothing and launches two kernels: a captured graph of it replays
+    correctly with eager work and synchronisations in between, and follows new inputs written in place."""
+    b, h, kdim, vdim, seqlen = 2, 2, 128, 64, 256
+    q, k, v, decay = [t.cuda() for t in _inputs(9, b, h, kdim, vdim, seqlen, 0.8, 1.0)]
+    out = torch.empty_like(v)
+    ws = torch.empty(retnet_recurrent.workspace_size(h, seqlen, batch=b, kdim=kdim, vdim=vdim), dtype=torch.uint8, device="cuda")
+    eager = aat.retnet_recurrent_fwd(q, k, v, decay)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        aat.retnet_recurrent_fwd(q, k, v, decay, out=out, workspace=ws)          # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        aat.retnet_recurrent_fwd(q, k, v, decay, out=out, workspace=ws)
+    for rep in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        _ = (q * 2).sum().item()                                              # eager work between replays
+    q2, k2, v2, decay2 = [t.cuda() for t in _inputs(10, b, h, kdim, vdim, seqlen, 0.8, 1.0)]
+    q.copy_(q2), k.copy_(k2), v.copy_(v2), decay.copy_(decay2)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, aat.retnet_recurrent_fwd(q2, k2, v2, decay2))
