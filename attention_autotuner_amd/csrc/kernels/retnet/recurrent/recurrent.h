@@ -455,6 +455,7 @@ __global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2)))
     chunk(std::integral_constant<int, 0>{}, c);
     if (c + 1 < nchunk) chunk(std::integral_constant<int, 1>{}, c + 1);
   }
+  wait_vmcnt<0>();      // the last chunk's copy into the idle stage must not outlive the block's hold on its LDS
 }
 
 }  // namespace aat
