@@ -156,7 +156,7 @@ template <int KD, int DVS>
 struct RetRecurrent {
   static constexpr int kChunk = 32;                       // positions per step
   static constexpr int kWaves = DVS / 32;
-  static constexpr int kThreads = kWaves * 64;
+  static constexpr int kThreads = kWaves * 64 + 64;        // the matrix waves plus one wave that moves the data
   static constexpr int kKB = KD / 32;                     // State tiles per wave
   static constexpr int kGroups = KD / 8;                  // groups of 8 key dims (one (h, e) sweep of a step)
   static constexpr int kGroupsPerWave = kGroups / kWaves; // share of one wave in the S^T contraction
@@ -166,10 +166,8 @@ struct RetRecurrent {
   static constexpr int kRed = kWaves * 4096;              // one partial S^T tile per wave
   static constexpr int kOutOff = 2 * kStage + kRed;       // per wave: its 32 x 32 output tile, staged for 16-byte stores
   static constexpr int kSmemBytes = kOutOff + kWaves * 4096;
-  static constexpr int kRowsPerDma = kThreads / 8;        // tile rows one LDS-DMA instruction of the block covers
   static_assert(KD % 32 == 0 && DVS % 64 == 0 && DVS <= 256, "tile shape");
   static_assert(kGroups % kWaves == 0, "the S^T contraction must split evenly over the waves");
-  static_assert(kRowsPerDma % 16 == 0, "the per-lane part of a copy must not depend on the instruction index");
   static_assert(kFOff + kRecFactorBytes <= 65536, "tile offsets go into the 16-bit offset field of the LDS reads");
   static_assert(kSmemBytes <= 160 * 1024, "LDS");
 };
@@ -196,8 +194,14 @@ template <int N, class V> AAT_DEV void lds_wait_younger_f(V& v) {
 // the first KD key dims (the reference's block_kdim, reference recurrent.h:290,427).  Grid (vdim / DVS, B*H).
 // Compiled for two waves per SIMD's worth of registers (256): then every MFMA takes and leaves its
 // operands in vector registers and nothing has to be moved between register classes.
+//
+// Waves 0 .. DVS/32-1 do the arithmetic; the last wave of the block only moves data: it issues every
+// LDS-DMA copy of the next chunk and stores the previous chunk's output tiles from their LDS staging
+// area.  An LDS-DMA or store instruction holds its wave for 16 to 50 cycles (thousands for a burst), and a
+// matrix wave is the only one on its SIMD: whatever it spends issuing memory instructions the matrix core
+// idles.  The data wave has nothing else to do.
 template <int KD, int DVS>
-__global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2))) void retnet_recurrent_kernel(
+__global__ __launch_bounds__(DVS * 2 + 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void retnet_recurrent_kernel(
     const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
     const char* __restrict__ factors, float* __restrict__ out, int heads, int kdim, int vdim, int L) {
   using T = RetRecurrent<KD, DVS>;
@@ -212,52 +216,93 @@ __global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const char* kg = reinterpret_cast<const char*>(k + (size_t)bh * kdim * L);
   const char* vg = reinterpret_cast<const char*>(v + ((size_t)bh * vdim + (size_t)blockIdx.x * DVS) * L);
   const char* fg = factors + (size_t)h * nchunk * kRecFactorBytes;
-  float* og = out + ((size_t)bh * vdim + (size_t)blockIdx.x * DVS + wave * 32) * L;
   const int pitch = L * 4;
-  // Output: the wave's O^T tile goes through LDS so that it leaves as four 16-byte-per-lane stores (8 rows
+  // Output: a wave's O^T tile goes through LDS so that it leaves as four 16-byte-per-lane stores (8 rows
   // x 128 bytes each) instead of sixteen 4-byte ones.  Row r of the tile sits at position r ^ ((r>>2)&1):
   // the two rows a write covers (r, r+4) and the two rows a 16-lane read phase covers (2m, 2m+1) then
   // fall on different halves of the banks.
   const int orl = lane >> 3, occ = lane & 7;
-  const uint32_t out_lane = (uint32_t)((orl * L + occ * 4) * 4);          // byte offset of this lane's 16 bytes in an 8-row group
+
+  if (wave == T::kWaves) {
+    // ================================ data wave =================================================
+    // LDS-DMA of a tile of 128-byte rows: instruction i covers positions 8i .. 8i+7, lane l position
+    // 8i + l/8, chunk slot l%8.  The source row is rec_pos(position), the source chunk the slot XOR the
+    // position's slot term (whose high bit is the parity of i).  Every address below is a scalar base that
+    // moves with the chunk plus a per-lane 32-bit offset computed here once: the loop of this wave must not
+    // contain a single vector instruction -- a vector instruction has to find a gap between the fp32 MFMAs
+    // of the matrix wave that shares the SIMD, and a copy that waits for one took 175 cycles to issue.
+    constexpr int kTileOps = (KD > DVS ? KD : DVS) / 8;
+    uint32_t toff[kTileOps];
+#pragma unroll
+    for (int i = 0; i < kTileOps; ++i)
+      toff[i] = (uint32_t)((8 * i + rec_pos(orl)) * pitch + (occ ^ (((i & 1) << 2) | (orl >> 1))) * 16);
+    const uint32_t lane16off = lane * 16;
+    auto dma_one = [&](const char* g_uniform, uint32_t lane_off, char* lds) {   // written out: scalar base + lane offset form
+      const uint64_t base = (uint64_t)(uintptr_t)g_uniform;
+      const uint32_t dst = (uint32_t)(uintptr_t)(AAT_AS3 char*)lds;
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :: "v"(lane_off), "s"(base), "s"(dst) : "memory", "m0");
+    };
+    // K and Q are needed first (the partial S^T opens a chunk); V and the decay factors follow.
+    auto dma_kq = [&](int c, int stage) {
+      char* s = smem + stage * T::kStage;
+      const size_t col = (size_t)c * T::kChunk * 4;
+#pragma unroll
+      for (int i = 0; i < KD / 8; ++i) dma_one(kg + col, toff[i], s + i * 1024);
+#pragma unroll
+      for (int i = 0; i < KD / 8; ++i) dma_one(qg + col, toff[i], s + T::kQOff + i * 1024);
+    };
+    auto dma_vf = [&](int c, int stage) {
+      char* s = smem + stage * T::kStage;
+#pragma unroll
+      for (int i = 0; i < DVS / 8; ++i) dma_one(vg + (size_t)c * T::kChunk * 4, toff[i], s + T::kVOff + i * 1024);
+      const char* f = fg + (size_t)c * kRecFactorBytes;
+#pragma unroll
+      for (int i = 0; i < kRecFactorBytes / 1024; ++i) dma_one(f + i * 1024, lane16off, s + T::kFOff + i * 1024);
+    };
+    // output tiles of chunk c: one per matrix wave, four 8-row groups each; all reads first, one wait, then
+    // the stores back to back, each a scalar base plus one of 16 precomputed lane offsets
+    uint32_t ooff[T::kWaves][4];
+#pragma unroll
+    for (int w = 0; w < T::kWaves; ++w)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ooff[w][i] = (uint32_t)(((32 * w + 8 * i + orl) * L + occ * 4) * 4);
+    const char* const oread = smem + T::kOutOff + (orl ^ ((orl >> 2) & 1)) * 128 + occ * 16;
+    float* const og = out + ((size_t)bh * vdim + (size_t)blockIdx.x * DVS) * L;
+    auto store_chunk = [&](int c) {
+      f4v x[T::kWaves][4];
+#pragma unroll
+      for (int w = 0; w < T::kWaves; ++w)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[w][i] = *reinterpret_cast<const f4v*>(oread + w * 4096 + i * 1024);
+      wait_lgkm0();
+      const uint64_t base = (uint64_t)(uintptr_t)(og + (size_t)c * T::kChunk);
+#pragma unroll
+      for (int w = 0; w < T::kWaves; ++w)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) asm volatile("global_store_dwordx4 %0, %1, %2" :: "v"(ooff[w][i]), "v"(x[w][i]), "s"(base) : "memory");
+    };
+    dma_kq(0, 0);
+    dma_vf(0, 0);
+    wait_vmcnt<0>();
+    for (int c = 0; c < nchunk; ++c) {
+      const bool more = c + 1 < nchunk;
+      asm volatile("s_barrier" ::: "memory");          // chunk c is in LDS; the matrix waves are done with chunk c-1
+      if (more) dma_kq(c + 1, (c + 1) & 1);
+      if (c > 0) store_chunk(c - 1);                     // staged before this barrier, overwritten after the next one
+      asm volatile("s_barrier" ::: "memory");          // (the matrix waves' barrier in front of the S^T sum)
+      if (more) dma_vf(c + 1, (c + 1) & 1);
+      wait_vmcnt<0>();                                   // the next chunk has landed, the stores are out
+    }
+    asm volatile("s_barrier" ::: "memory");              // the last chunk's tiles are staged
+    store_chunk(nchunk - 1);
+    return;
+  }
+
+  // ================================ matrix waves ================================================
   char* const ost = smem + T::kOutOff + wave * 4096;
   char* const ow_even = ost + n * 4 + 5 * hi * 128;                         // write base for e even: position 4h + h
   char* const ow_odd = ost + n * 4 + (3 * hi + 1) * 128;                    // e odd: position 4h + (1 - h)
-  const uint32_t oread = lds_addr(ost) + (orl ^ ((orl >> 2) & 1)) * 128 + occ * 16;
-
-  // LDS-DMA: slot s = i * kThreads + tid of a tile is position s/8, chunk slot s%8; the per-lane part of
-  // the source address is the same for every instruction i because kRowsPerDma is a multiple of 16.
-  const int dp = tid >> 3, dcs = tid & 7;
-  const uint32_t dma_off = (uint32_t)(rec_pos(dp) * pitch + rec_slot(dp, dcs) * 16);
-  auto dma_one = [&](const char* g_uniform, uint32_t lane_off, char* lds) {
-    uint64_t base = (uint64_t)(uintptr_t)g_uniform;
-    asm volatile("" : "+s"(base));
-    __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)(base + lane_off), (AAT_AS3 void*)lds, 16, 0, 0);
-  };
-  // The copy of one chunk is a list of kDmaOps LDS-DMA instructions per wave (K, Q, V tiles, then the
-  // decay factors; the last one belongs to wave 0 alone).  They are issued one at a time between the
-  // matrix instructions of the previous chunk: a burst of them blocks the wave for thousands of cycles
-  // (the CU tracks only so many cache lines in flight, and every 16-byte lane piece of these column
-  // accesses is a line of its own), and with one wave per SIMD nothing else would feed the matrix core.
-  constexpr int kOpsK = KD / T::kRowsPerDma, kOpsV = DVS / T::kRowsPerDma, kOpsF = 4096 / (T::kThreads * 16);
-  constexpr int kDmaOps = 2 * kOpsK + kOpsV + kOpsF + 1;
-  auto dma_op = [&](auto op_tag, int c, int stage) {
-    constexpr int op = decltype(op_tag)::value;
-    char* s = smem + stage * T::kStage;
-    const size_t col = (size_t)c * T::kChunk * 4;
-    if constexpr (op < 2 * kOpsK + kOpsV) {
-      constexpr int tile = op < kOpsK ? 0 : (op < 2 * kOpsK ? 1 : 2);
-      constexpr int i = tile == 0 ? op : (tile == 1 ? op - kOpsK : op - 2 * kOpsK);
-      const char* g = (tile == 0 ? kg : (tile == 1 ? qg : vg)) + col;
-      dma_one(g + (size_t)i * T::kRowsPerDma * pitch, dma_off,
-              s + (tile == 0 ? 0 : (tile == 1 ? T::kQOff : T::kVOff)) + (i * T::kThreads + wave * 64) * 16);
-    } else if constexpr (op < kDmaOps - 1) {
-      constexpr int i = op - (2 * kOpsK + kOpsV);
-      dma_one(fg + (size_t)c * kRecFactorBytes + i * T::kThreads * 16, tid * 16, s + T::kFOff + (i * T::kThreads + wave * 64) * 16);
-    } else {
-      if (wave == 0) dma_one(fg + (size_t)c * kRecFactorBytes + 4096, lane * 16, s + T::kFOff + 4096);
-    }
-  };
 
   // Per-lane LDS read addresses of the current stage (moved to the other stage at the end of a chunk).
   //  row read (row 8G+4h+e, column n): the slot term of the row is the compile-time constant
@@ -307,10 +352,7 @@ __global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2)))
   constexpr int nS4 = 16 * T::kKB;                        // Q row reads of State^T Q
   constexpr int nRedG = T::kWaves;                        // per g: the other waves' partials, then D
   constexpr int jRed = nS1 + nS4, jPnl = jRed + 4 * nRedG, jFlag = jPnl + 1, jV = jFlag + 1, jW = jV + 4, jK = jW + 4;
-  constexpr int jO = jK + 2 * T::kKB;                     // output tile reads, half way through the State update
-  constexpr int nElem = jK + 4 * T::kKB + 4;
-  constexpr int kDmaEvery = (nElem * 3 / 4) / kDmaOps;      // one copy instruction every so many stream elements
-  static_assert(kDmaEvery >= 1 && kDmaEvery * (kDmaOps - 1) < jK, "every copy instruction is issued before the first output store");
+  constexpr int nElem = jK + 4 * T::kKB;
 
   auto chunk = [&](auto stage_tag, int c) {
     constexpr int S = decltype(stage_tag)::value;
@@ -341,10 +383,8 @@ __global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2)))
         vr[slot] = lds_read_f4_async(colv[j - jV], 0);
       } else if constexpr (j < jK) {
         vr[slot] = lds_read_f4_async(wbase, T::kFOff + kRecFactorW + (j - jW) * 16);
-      } else if constexpr (j >= jO && j < jO + 4) {
-        vr[slot] = lds_read_f4_async(oread, (j - jO) * 1024);
       } else {
-        constexpr int jj = j < jO ? j - jK : j - jK - 4, kb = jj / 4, g = jj % 4;
+        constexpr int kb = (j - jK) / 4, g = (j - jK) % 4;
         vr[slot] = lds_read_f4_async(colb[g], kb * 4096);
       }
     };
@@ -397,7 +437,7 @@ __global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               *reinterpret_cast<float*>((e & 1 ? ow_odd : ow_even) + (8 * g + (e & 2)) * 128) = oacc[4 * g + e];
-          asm volatile("" ::: "memory");     // the tile is written before its reads are issued
+          asm volatile("" ::: "memory");     // staged before the barrier that hands it to the data wave
         }
       } else if constexpr (j < jK) {
         lds_wait_younger_f<younger>(vr[slot]);
@@ -412,26 +452,15 @@ __global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2)))
               for (int i = 0; i < 16; ++i) st[kb][i] *= sc;
           }
         }
-      } else if constexpr (j >= jO && j < jO + 4) {
-        lds_wait_younger_f<younger>(vr[slot]);
-        uint64_t rowp = (uint64_t)(uintptr_t)(og + (size_t)(8 * (j - jO)) * L + (size_t)c * T::kChunk);
-        asm volatile("" : "+s"(rowp));
-        *reinterpret_cast<AAT_AS1 f4v*>(rowp + out_lane) = vr[slot];
       } else {
-        constexpr int jj = j < jO ? j - jK : j - jK - 4, kb = jj / 4, g = jj % 4;
+        constexpr int kb = (j - jK) / 4, g = (j - jK) % 4;
         lds_wait_younger_f<younger>(vr[slot]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) st[kb] = mfma_32x32x2_f32(vr[slot][e], wv[g][e], st[kb]);
       }
     };
 
-    // Outstanding vector-memory operations, oldest first: the copy of chunk c (issued during chunk c-1),
-    // then the 4 output stores of chunk c-1.  They retire in order, so the copy has landed once at most
-    // the stores are left.  (Chunk 0 was copied by the prologue and has no stores behind it.)
-    if (c == 0) wait_vmcnt<0>();
-    else wait_vmcnt<4>();
-    asm volatile("s_barrier" ::: "memory");   // chunk c is in LDS; every wave is done with chunk c-1
-    const int cnext = c + 1 < nchunk ? c + 1 : c;      // the last chunk re-reads itself into the idle stage
+    asm volatile("s_barrier" ::: "memory");   // chunk c is in LDS (the data wave waited for it); every wave is done with chunk c-1
     static_for<kPF>([&](auto jt) { issue(jt); });
     sched_fence();
     static_for<nElem>([&](auto jt) {
@@ -443,19 +472,18 @@ __global__ __launch_bounds__(DVS * 2) __attribute__((amdgpu_waves_per_eu(2, 2)))
         issue(std::integral_constant<int, j + kPF>{});
       }
       consume(jt);
-      if constexpr (j % kDmaEvery == 0 && j / kDmaEvery < kDmaOps) dma_op(std::integral_constant<int, j / kDmaEvery>{}, cnext, S ^ 1);
       sched_fence();
     });
 #pragma unroll
     for (int i = 0; i < kNumBases; ++i) bases[i] += (S == 0) ? T::kStage : -T::kStage;
   };
 
-  static_for<kDmaOps>([&](auto op) { dma_op(op, 0, 0); });
   for (int c = 0; c < nchunk; c += 2) {
     chunk(std::integral_constant<int, 0>{}, c);
     if (c + 1 < nchunk) chunk(std::integral_constant<int, 1>{}, c + 1);
   }
-  wait_vmcnt<0>();      // the last chunk's copy into the idle stage must not outlive the block's hold on its LDS
+  wait_lgkm0();
+  asm volatile("s_barrier" ::: "memory");     // the last chunk's output tiles are staged: the data wave stores them
 }
 
 }  // namespace aat
