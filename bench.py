@@ -46,12 +46,12 @@ def resolve_config(aat, arch, tensors, causal):
 def time_launches(fn, steps, warmup):
     """(wall ms per step, mean kernel ms from per-launch events on the launch stream)."""
     import torch
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    t0 = time.perf_counter()
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()              # nothing but this between the warm-up and the timed steps: the clock ramps
+    t0 = time.perf_counter()              # up over tens of milliseconds of load and falls back when the GPU idles
     for i in range(steps):
         starts[i].record()
         fn()
@@ -104,8 +104,8 @@ def measured_traffic(cfg):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the causal / long-kv / RetNet side measurements")
     ap.add_argument("--copy-calibration", action="store_true",
