@@ -290,8 +290,8 @@ __global__ __launch_bounds__(DVS * 2 + 64) __attribute__((amdgpu_waves_per_eu(2,
       asm volatile("s_barrier" ::: "memory");          // chunk c is in LDS; the matrix waves are done with chunk c-1
       if (more) dma_kq(c + 1, (c + 1) & 1);
       if (c > 0) store_chunk(c - 1);                     // staged before this barrier, overwritten after the next one
-      asm volatile("s_barrier" ::: "memory");          // (the matrix waves' barrier in front of the S^T sum)
       if (more) dma_vf(c + 1, (c + 1) & 1);
+      asm volatile("s_barrier" ::: "memory");          // (the matrix waves' barrier in front of the S^T sum, late in the chunk)
       wait_vmcnt<0>();                                   // the next chunk has landed, the stores are out
     }
     asm volatile("s_barrier" ::: "memory");              // the last chunk's tiles are staged
@@ -351,8 +351,13 @@ __global__ __launch_bounds__(DVS * 2 + 64) __attribute__((amdgpu_waves_per_eu(2,
   constexpr int nS1 = 8 * T::kGroupsPerWave;              // K and Q row reads of the partial S^T
   constexpr int nS4 = 16 * T::kKB;                        // Q row reads of State^T Q
   constexpr int nRedG = T::kWaves;                        // per g: the other waves' partials, then D
-  constexpr int jRed = nS1 + nS4, jPnl = jRed + 4 * nRedG, jFlag = jPnl + 1, jV = jFlag + 1, jW = jV + 4, jK = jW + 4;
-  constexpr int nElem = jK + 4 * T::kKB;
+  // Order after State^T Q: the State update comes first (it needs V, w and K only), the sum of the partial
+  // S^T tiles, P and V P sit inside it, before its last 16 matrix instructions.  Whatever a vector phase
+  // needs from the matrix pipe (O^T for its scaling, V P for the staging of the output tile) then left it a
+  // thousand cycles earlier, and the barrier in front of the partial tiles comes late in the chunk.
+  constexpr int jS4 = nS1, jFlag = jS4 + nS4, jV = jFlag + 1, jW = jV + 4, jK1 = jW + 4;
+  constexpr int jRed = jK1 + 4 * (T::kKB - 1), jPnl = jRed + 4 * nRedG, jK2 = jPnl + 1;
+  constexpr int nElem = jK2 + 4;
 
   auto chunk = [&](auto stage_tag, int c) {
     constexpr int S = decltype(stage_tag)::value;
@@ -360,32 +365,33 @@ __global__ __launch_bounds__(DVS * 2 + 64) __attribute__((amdgpu_waves_per_eu(2,
     f4v vr[kRing];
     f16v sp = zero16(), oacc = zero16(), pm;
     f4v vt[4], wv[4];
-    float ka = 0.f, pnl = 0.f;
-    f4v flag = {0.f, 0.f, 0.f, 0.f};
+    float ka = 0.f;
 
     auto issue = [&](auto jt) {
       constexpr int j = decltype(jt)::value, slot = j % kRing;
       if constexpr (j < nS1) {
         constexpr int i = j / 2, gg = i / 4, e = i % 4, p0 = 8 * gg + 4 * (e & 1) + (e & 2), sw = (p0 >> 1) & 7;
         fr[slot] = lds_read_f1_async(row1[sw], (j % 2 ? T::kQOff : 0) + p0 * 128);
-      } else if constexpr (j < jRed) {
-        constexpr int jj = j - nS1, G = jj / 4, e = jj % 4, p0 = 8 * G + 4 * (e & 1) + (e & 2), sw = (p0 >> 1) & 7;
+      } else if constexpr (j < jFlag) {
+        constexpr int jj = j - jS4, G = jj / 4, e = jj % 4, p0 = 8 * G + 4 * (e & 1) + (e & 2), sw = (p0 >> 1) & 7;
         fr[slot] = lds_read_f1_async(row4[sw], T::kQOff + p0 * 128);
+      } else if constexpr (j == jFlag) {
+        vr[slot] = lds_read_f4_async(sbase, T::kFOff + kRecFactorFlag);
+      } else if constexpr (j < jW) {
+        vr[slot] = lds_read_f4_async(colv[j - jV], 0);
+      } else if constexpr (j < jK1) {
+        vr[slot] = lds_read_f4_async(wbase, T::kFOff + kRecFactorW + (j - jW) * 16);
+      } else if constexpr (j < jRed) {
+        constexpr int kb = (j - jK1) / 4, g = (j - jK1) % 4;
+        vr[slot] = lds_read_f4_async(colb[g], kb * 4096);
       } else if constexpr (j < jPnl) {
         constexpr int g = (j - jRed) / nRedG, t = (j - jRed) % nRedG;
         if constexpr (t < T::kWaves - 1) vr[slot] = lds_read_f4_async(redo[t], g * 1024);
         else vr[slot] = lds_read_f4_async(lane16, T::kFOff + g * 1024);
       } else if constexpr (j == jPnl) {
         fr[slot] = lds_read_f1_async(pbase, T::kFOff + kRecFactorPnl);
-      } else if constexpr (j == jFlag) {
-        vr[slot] = lds_read_f4_async(sbase, T::kFOff + kRecFactorFlag);
-      } else if constexpr (j < jW) {
-        vr[slot] = lds_read_f4_async(colv[j - jV], 0);
-      } else if constexpr (j < jK) {
-        vr[slot] = lds_read_f4_async(wbase, T::kFOff + kRecFactorW + (j - jW) * 16);
       } else {
-        constexpr int kb = (j - jK) / 4, g = (j - jK) % 4;
-        vr[slot] = lds_read_f4_async(colb[g], kb * 4096);
+        vr[slot] = lds_read_f4_async(colb[j - jK2], (T::kKB - 1) * 4096);
       }
     };
 
@@ -403,10 +409,31 @@ __global__ __launch_bounds__(DVS * 2 + 64) __attribute__((amdgpu_waves_per_eu(2,
           }
           asm volatile("" ::: "memory");     // the stores stay here, far ahead of the barrier that publishes them
         }
-      } else if constexpr (j < jRed) {
-        constexpr int jj = j - nS1;
+      } else if constexpr (j < jFlag) {
+        constexpr int jj = j - jS4;
         lds_wait_younger_f<younger>(fr[slot]);
         oacc = mfma_32x32x2_f32(st[jj / 16][jj % 16], fr[slot], oacc);
+      } else if constexpr (j == jFlag) {
+        lds_wait_younger_f<younger>(vr[slot]);
+        if (__builtin_amdgcn_readfirstlane(__float_as_uint(vr[slot][0])) != 0u) {   // lambda left its range: fold it into T
+          const float sc = vr[slot][1];
+#pragma unroll
+          for (int kb = 0; kb < T::kKB; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) st[kb][i] *= sc;
+        }
+      } else if constexpr (j < jW) {
+        lds_wait_younger_f<younger>(vr[slot]);
+        vt[j - jV] = vr[slot];
+      } else if constexpr (j < jK1) {
+        lds_wait_younger_f<younger>(vr[slot]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) wv[j - jW][e] = vt[j - jW][e] * vr[slot][e];
+      } else if constexpr (j < jRed) {
+        constexpr int kb = (j - jK1) / 4, g = (j - jK1) % 4;
+        lds_wait_younger_f<younger>(vr[slot]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) st[kb] = mfma_32x32x2_f32(vr[slot][e], wv[g][e], st[kb]);
       } else if constexpr (j < jPnl) {
         constexpr int g = (j - jRed) / nRedG, t = (j - jRed) % nRedG;
         lds_wait_younger_f<younger>(vr[slot]);
@@ -417,46 +444,26 @@ __global__ __launch_bounds__(DVS * 2 + 64) __attribute__((amdgpu_waves_per_eu(2,
         }
       } else if constexpr (j == jPnl) {
         lds_wait_younger_f<younger>(fr[slot]);
-        pnl = fr[slot];
-      } else if constexpr (j == jFlag) {
-        lds_wait_younger_f<younger>(vr[slot]);
-        flag = vr[slot];
-      } else if constexpr (j < jW) {
-        lds_wait_younger_f<younger>(vr[slot]);
-        vt[j - jV] = vr[slot];
-        if constexpr (j == jW - 1) {
-          // O^T = (p_n lambda) T^T Q + V P, then out
+        // O^T = (p_n lambda) T^T Q + V P
 #pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[i] *= pnl;
+        for (int i = 0; i < 16; ++i) oacc[i] *= fr[slot];
 #pragma unroll
-          for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < 4; ++g)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) oacc = mfma_32x32x2_f32(vt[g][e], pm[4 * g + e], oacc);
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              *reinterpret_cast<float*>((e & 1 ? ow_odd : ow_even) + (8 * g + (e & 2)) * 128) = oacc[4 * g + e];
-          asm volatile("" ::: "memory");     // staged before the barrier that hands it to the data wave
-        }
-      } else if constexpr (j < jK) {
-        lds_wait_younger_f<younger>(vr[slot]);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) wv[j - jW][e] = vt[j - jW][e] * vr[slot][e];
-        if constexpr (j == jK - 1) {
-          if (__builtin_amdgcn_readfirstlane(__float_as_uint(flag[0])) != 0u) {   // lambda left its range: fold it into T
-            const float sc = flag[1];
-#pragma unroll
-            for (int kb = 0; kb < T::kKB; ++kb)
-#pragma unroll
-              for (int i = 0; i < 16; ++i) st[kb][i] *= sc;
-          }
-        }
+          for (int e = 0; e < 4; ++e) oacc = mfma_32x32x2_f32(vt[g][e], pm[4 * g + e], oacc);
       } else {
-        constexpr int kb = (j - jK) / 4, g = (j - jK) % 4;
+        constexpr int kb = T::kKB - 1, g = j - jK2;
         lds_wait_younger_f<younger>(vr[slot]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) st[kb] = mfma_32x32x2_f32(vr[slot][e], wv[g][e], st[kb]);
+        if constexpr (j == nElem - 1) {
+#pragma unroll
+          for (int gg = 0; gg < 4; ++gg)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              *reinterpret_cast<float*>((e & 1 ? ow_odd : ow_even) + (8 * gg + (e & 2)) * 128) = oacc[4 * gg + e];
+          asm volatile("" ::: "memory");     // staged before the barrier that hands it to the data wave
+        }
       }
     };
 
