@@ -76,9 +76,32 @@ static void test_regfuse_attention(const ProblemShape& ps, const Buffers& b) {
   HIP_OK(hipFuncSetAttribute((const void*)plain, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
   HIP_OK(hipFuncSetAttribute((const void*)causal, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
   const float scale = 1.f / std::sqrt((float)Kd);
+  const int items = ps.B * ps.H * ps.Sq / Br;
+  // as the library does: persistent blocks for non-causal problems with more row blocks than the chip holds
+  using TP = typename T::template Persist<WPE>;
+  int resident = 0;
+  if constexpr (TP::kOk && !PIPE) {
+    auto persist = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, false, false, false, true>;
+    int per_cu = 0, cus = 0, dev = 0;
+    HIP_OK(hipGetDevice(&dev));
+    HIP_OK(hipFuncSetAttribute((const void*)persist, hipFuncAttributeMaxDynamicSharedMemorySize, TP::kSmemBytes));
+    HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)persist, NT, TP::kSmemBytes));
+    HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    if (!ps.causal && (ps.Sk / Bc) % 2 == 0 && ps.Sk / Bc <= 14 && items > per_cu * cus) resident = per_cu * cus;
+    if (resident > 0) {
+      auto t = aat_bench::do_bench([&] {
+        persist<<<dim3(resident), dim3(NT), TP::kSmemBytes, 0>>>(b.q, b.k, b.v, b.o, nullptr, ps.H, ps.Sk, ps.Sq, scale,
+                                                                nullptr, nullptr, items);
+      }, ps.flush);
+      char name[128];
+      std::snprintf(name, sizeof name, "regfuse  Br=%d Bc=%d thr=%d bufs=%d/%d waves/SIMD=%d persistent (%d blocks)", Br, Bc, NT, NSK, NSV, WPE, resident);
+      report(name, ps, Kd, D, t);
+      return;
+    }
+  }
   auto t = aat_bench::do_bench([&] {
-    (ps.causal ? causal : plain)<<<dim3(ps.B * ps.H * ps.Sq / Br), dim3(NT), T::kSmemBytes, 0>>>(
-        b.q, b.k, b.v, b.o, nullptr, ps.H, ps.Sk, ps.Sq, scale, nullptr, nullptr);
+    (ps.causal ? causal : plain)<<<dim3(items), dim3(NT), T::kSmemBytes, 0>>>(
+        b.q, b.k, b.v, b.o, nullptr, ps.H, ps.Sk, ps.Sq, scale, nullptr, nullptr, 0);
   }, ps.flush);
   char name[128];
   std::snprintf(name, sizeof name, "regfuse  Br=%d Bc=%d thr=%d bufs=%d/%d waves/SIMD=%d%s", Br, Bc, NT, NSK, NSV, WPE, PIPE ? " pipelined" : "");

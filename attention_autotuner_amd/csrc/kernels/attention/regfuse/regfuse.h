@@ -54,6 +54,28 @@ struct AttnFwdRegfuse {
   static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
   static constexpr int kEpiBytesSplit = Br * kOStride32;
   static constexpr int kSmemBytesSplit = kMainBytes > kEpiBytesSplit ? kMainBytes : kEpiBytesSplit;
+  // Persistent blocks (PERSIST) stage their output tiles where the copies of the next row block's first kv
+  // tile do not land: behind the K/V buffers as far as the LDS budget of a block goes, then in the second K
+  // and the second V buffer (the last kv tile of a row block has parity 1, the prefetch goes to parity 0).
+  static constexpr int kStageWave = WM * kOStride;
+  template <int WPE> struct Persist {
+    static constexpr int kBlocksByRegs = (WPE * 4) / NW > 0 ? (WPE * 4) / NW : 1;   // resident blocks the registers allow
+    static constexpr int kBudget = (160 * 1024 / kBlocksByRegs) & ~2047;            // whole allocation units
+    static constexpr int kWant = kMainBytes + NW * kStageWave;
+    static constexpr int kFit = kWant < kBudget ? kWant : kBudget;
+    static constexpr int kSmemBytes = kFit > kMainBytes ? kFit : kMainBytes;
+    static constexpr int kInSpare = (kSmemBytes - kMainBytes) / kStageWave;
+    static constexpr int kInK = kKBytes / kStageWave, kInV = kVBytes / kStageWave;
+    static constexpr bool kOk = NSK == 2 && NSV == 2 && kInSpare + kInK + kInV >= NW;
+    static constexpr bool kSharesBuffers = kInSpare < NW;   // then every wave must be done with the last tile first
+    static constexpr int kOutputStores = RT * D / 16;       // 16-byte-per-lane store instructions of one output tile
+    static_assert(kOutputStores + RT < 64, "vmcnt is a 6-bit counter");
+    AAT_DEV static int stage_offset(int wave) {
+      if (wave < kInSpare) return kMainBytes + wave * kStageWave;
+      if (wave < kInSpare + kInK) return kKBytes + (wave - kInSpare) * kStageWave;
+      return NSK * kKBytes + kVBytes + (wave - kInSpare - kInK) * kStageWave;
+    }
+  };
   // The pipelined schedule copies K in whole 32-row units.
   static constexpr bool kPipeOk = NSK == 2 && NSV == 2 && KDma::kRegular && KDma::kRowsPerIter <= 32 &&
                                   32 % KDma::kRowsPerIter == 0;
@@ -88,18 +110,31 @@ template <bool CAUSAL, class F> AAT_DEV void run_tiles(F& tile, int n_full, int 
 // blocks to fill the chip).  Part s handles kv tiles [s, s+1) * n_tiles / parts and writes its own
 // normalised output (fp32) and log-sum-exp to part_o / part_lse, laid out [part][B*H*S_q][D] and
 // [part][B*H*S_q]; attn_split_merge combines them.  o and lse are not touched.
+//
+// PERSIST: the grid is as many blocks as the chip holds at once and block b works through row blocks
+// b, b + gridDim.x, ... of the n_items = B*H*S_q/Br there are.  A block that is alone on its CU otherwise
+// pays for every row block the launch of a new block, the first trip to memory for Q, K and V with nothing
+// to overlap it, and the drain of the output stores: 5.7 us of the 66 us a 256-row block of the 2048 x 2048
+// problem takes.  Here the last kv tile of a row block requests tile 0 of the next one (K, V into the
+// buffers of the other parity, Q into the fragment registers the moment the last scores are done), the
+// output tile is staged where those copies do not land, and the first tile of the next row block waits for
+// the copies only: memory operations complete in order, so "at most as many outstanding as stores were issued
+// after them" leaves the stores in flight.  Needs two K and two V buffers and an even number of kv tiles (the
+// buffer parity must wrap); plain schedule, non-causal, unsplit.
 template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int WPE = 1, bool PIPE = false,
-          bool CAUSAL = false, bool SPLIT = false>
+          bool CAUSAL = false, bool SPLIT = false, bool PERSIST = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k,
                       const half_t* __restrict__ v, half_t* __restrict__ o, float* __restrict__ lse,
                       int H, int seq_k, int seq_q, float softmax_scale, float* __restrict__ part_o = nullptr,
-                      float* __restrict__ part_lse = nullptr) {
+                      float* __restrict__ part_lse = nullptr, int n_items = 0) {
   using T = AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, WM = T::WM;
   constexpr int PF = AAT_PF;                     // operand prefetch distance, in MFMA steps
   static_assert(!PIPE || T::kPipeOk, "the pipelined schedule needs 2+2 buffers and unit-aligned K copies");
   static_assert(!(SPLIT && CAUSAL), "kv splitting is for non-causal problems");
+  using TP = typename T::template Persist<WPE>;
+  static_assert(!PERSIST || (!PIPE && !CAUSAL && !SPLIT && TP::kOk), "persistent blocks: plain schedule, 2+2 buffers, room to stage the output");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 #ifdef AAT_CLOCK_PROBE
   const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
@@ -113,33 +148,6 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   const int n = lane & 31, h = lane >> 5;
 
   const int Tr = seq_q / Br;
-  const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = tile / Tr;
-  int rb = tile % Tr;
-  if constexpr (CAUSAL) rb = Tr - 1 - rb;       // long rows first
-  const int q0 = rb * Br;
-  const int diag = seq_k - seq_q;               // kv index allowed for query i is <= i + diag
-  int n_tiles = seq_k / Bc;
-  int n_full = n_tiles;                         // tiles [0, n_full) are visible to every row of the block
-  if constexpr (CAUSAL) {
-    const int last = q0 + Br - 1 + diag;        // last visible kv index for this block
-    const int lim = last < 0 ? 0 : last / Bc + 1;
-    n_tiles = lim < n_tiles ? lim : n_tiles;
-    const int full = (q0 + diag + 1) / Bc;
-    n_full = full < 0 ? 0 : (full < n_tiles ? full : n_tiles);
-    n_full &= ~1;                               // keep the masked loop on an even tile: buffer parity 0
-  }
-
-  int tile0 = 0;                                // first kv tile of this block's range
-  if constexpr (SPLIT) {
-    const int per = n_tiles / (int)gridDim.y;   // the launcher guarantees divisibility
-    tile0 = (int)blockIdx.y * per;
-    n_tiles = per;
-    n_full = per;
-  }
-  const char* kg = reinterpret_cast<const char*>(k + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * Kd);
-  const char* vg = reinterpret_cast<const char*>(v + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * D);
-
   typename T::KDma kdma;
   typename T::VDma vdma;
   kdma.init(tid);
@@ -147,7 +155,6 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   const int wave_base = wave * 64;
 
   h8 qf[RT][KS];
-  load_q_frags<RT, KS, Kd>(qf, q + ((size_t)bh * seq_q + q0 + wave * WM + n) * Kd + 8 * h);
   uint32_t kaddr[KS], vaddr[DT];                 // this lane's operand addresses inside buffer 0
   {
     int koff[KS], voff[DT];
@@ -159,189 +166,254 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     for (int dt = 0; dt < DT; ++dt) vaddr[dt] = lds_addr(vbuf + voff[dt]);
   }
 
-  f16v oacc[RT][DT];
-  float m_run[RT], l_run[RT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    m_run[rt] = -INFINITY;
-    l_run[rt] = 0.f;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] = zero16();
-  }
   const float c2 = softmax_scale * kLog2e;
-  const int q_lim0 = q0 + wave * WM + n + diag;   // last kv index row n of row group 0 may see
+  const int diag = seq_k - seq_q;               // kv index allowed for query i is <= i + diag
 
-  if constexpr (!PIPE) {
-    // ============================ plain schedule =================================================
-    if (n_tiles > 0) {
-      kdma.issue(kg, kbuf, wave_base);
-      if constexpr (NSV == 2) vdma.issue(vg, vbuf, wave_base);
+  // One pass per row block: a single one unless PERSIST.
+  bool prefetched = false;                      // Q fragments and kv tile 0 of this row block were requested by the previous pass
+  for (int vb = blockIdx.x;; vb += gridDim.x) {
+    const int tile = PERSIST ? xcd_remap(vb, n_items) : xcd_remap(vb, (int)gridDim.x);
+    const int bh = tile / Tr;
+    int rb = tile % Tr;
+    if constexpr (CAUSAL) rb = Tr - 1 - rb;       // long rows first
+    const int q0 = rb * Br;
+    int n_tiles = seq_k / Bc;
+    int n_full = n_tiles;                         // tiles [0, n_full) are visible to every row of the block
+    if constexpr (CAUSAL) {
+      const int last = q0 + Br - 1 + diag;        // last visible kv index for this block
+      const int lim = last < 0 ? 0 : last / Bc + 1;
+      n_tiles = lim < n_tiles ? lim : n_tiles;
+      const int full = (q0 + diag + 1) / Bc;
+      n_full = full < 0 ? 0 : (full < n_tiles ? full : n_tiles);
+      n_full &= ~1;                               // keep the masked loop on an even tile: buffer parity 0
     }
-    // `parity_tag` carries j & 1 as a compile-time value so that every LDS address of the tile is a
-    // per-lane constant plus an immediate.
-    auto kv_tile = [&](const int j, auto parity_tag, auto masked_tag) {
-      constexpr int PAR = decltype(parity_tag)::value;
-      constexpr bool MASKED = decltype(masked_tag)::value;   // the causal diagonal may cross this tile
-      char* const vcur = vbuf + (NSV == 2 ? PAR * T::kVBytes : 0);
-      const bool more = (j + 1 < n_tiles);
-      if constexpr (WPE == 1) {
-        // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
-        // output accumulators in the accumulation half and the Q fragments in the vector half, or the
-        // allocator parks Q there and copies four registers back in front of every MFMA.
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
-        }
-      }
 
-      // (A) K_j (and with two V buffers V_j) has landed; every wave is past iteration j-1.
-      wait_vmcnt<0>();
-      block_sync();
-      if constexpr (NSV == 1) vdma.issue(vg + (size_t)j * T::kVBytes, vcur, wave_base);
-      if (more) {
-        if constexpr (NSK == 2) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf + (PAR ^ 1) * T::kKBytes, wave_base);
-        if constexpr (NSV == 2) vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + (PAR ^ 1) * T::kVBytes, wave_base);
-      }
-
-      f16v sacc[RT][NT];
-      qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
-
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
-        const float mc = lazy_max_step<NT, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
-        exp_tile<NT>(sacc[rt], c2, mc);
-        if constexpr (MASKED) zero_masked<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
-      }
-
-      // (B) with one buffer: V_j must have landed / K buffer must be free before K_{j+1} is fetched.
-      if constexpr (NSV == 1 || NSK == 1) {
-        if constexpr (NSV == 1) wait_vmcnt<0>();
-        block_sync();
-        if constexpr (NSK == 1) {
-          if (more) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf, wave_base);
-        }
-      }
-      h8 pf[RT][NT][2];
-      pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) pack_p_group<NT>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
-      });
-    };
-    run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
-  } else {
-    // ============================ pipelined schedule =============================================
-    // The unit of work is 32 kv rows.  While unit u is exponentiated, the MFMAs of unit u+1's scores
-    // run underneath; then O += V_u^T P_u runs with the fp16 packing of P_u underneath.  Two score
-    // tiles are live (current, next).
-    //
-    // K is copied in Bc-row tiles that are SHIFTED by one unit against the V tiles: K copy j holds kv
-    // rows [j*Bc + 32, (j+1)*Bc + 32), exactly the units whose scores are computed during iteration j
-    // (units 1..NT-1 of tile j and unit 0 of tile j+1).  So iteration j reads K buffer j&1 only, while
-    // copy j+1 streams into the other one; V tile j is read from V buffer j&1 while V_{j+1} streams
-    // in.  One barrier per Bc rows.  Rows [0, 32) are fetched on their own in the prologue.
-    constexpr int KI = T::kKInstrPerUnit;        // DMA instructions per 32 rows of K
-    f16v sbuf[2][RT][1];
-    auto issue_k_copy = [&](int jj, char* dst) { // K copy jj; the last one stops at the end of the range
-      const char* src = kg + (size_t)jj * T::kKBytes + T::kUnitK;
-      if (jj + 1 < n_tiles) kdma.issue(src, dst, wave_base);
-      else kdma.template issue_part<0, (NT - 1) * KI>(src, dst, wave_base);
-    };
-    if (n_tiles > 0) {
-      kdma.template issue_part<0, KI>(kg, kbuf + T::kKBytes + (NT - 1) * T::kUnitK, wave_base);   // rows [0, 32)
-      issue_k_copy(0, kbuf);
-      vdma.issue(vg, vbuf, wave_base);
-      wait_vmcnt<0>();
-      block_sync();
-      qk_gemm_steps<RT, 1, KS, NCK, PF>(sbuf[0], qf, kaddr, T::kKBytes + (NT - 1) * T::kUnitK, [](int) {});
-    }
-    auto kv_tile = [&](const int j, auto parity_tag, auto masked_tag) {
-      constexpr int PAR = decltype(parity_tag)::value;
-      constexpr bool MASKED = decltype(masked_tag)::value;
-      const bool last_tile = (j + 1 >= n_tiles);
-      if constexpr (WPE == 1) {
-        // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
-        // output accumulators in the accumulation half and the Q fragments in the vector half, or the
-        // allocator parks Q there and copies four registers back in front of every MFMA.
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
-        }
-      }
-      // K copy j and V_j have landed; every wave finished iteration j-1 (frees the other buffers).
-      wait_vmcnt<0>();
-      block_sync();
-      if (!last_tile) {
-        issue_k_copy(j + 1, kbuf + (PAR ^ 1) * T::kKBytes);
-        vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + (PAR ^ 1) * T::kVBytes, wave_base);
-      }
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const int cur = (PAR * NT + t) & 1;                        // which score buffer holds unit (j, t)
-        auto& scur = sbuf[cur];
-        auto& snext = sbuf[cur ^ 1];
-        const int kv0 = j * Bc + 32 * t;
-        float mc[RT];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          if constexpr (MASKED) causal_mask<1>(scur[rt], kv0, q_lim0 + rt * 32, h);
-          mc[rt] = lazy_max_step<1, DT>(scur[rt], m_run[rt], l_run[rt], oacc[rt], c2);
-        }
-        constexpr int kPerStep = (16 + KS - 1) / KS;               // exponentials per MFMA step
-        if (t + 1 < NT || !last_tile) {
-          // scores of the next unit: slot t of K buffer PAR
-          qk_gemm_steps<RT, 1, KS, NCK, PF>(snext, qf, kaddr, PAR * T::kKBytes + t * T::kUnitK, [&](int step) {
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt) exp_range<1>(scur[rt], step * kPerStep, kPerStep, c2, mc[rt]);
-          });
-        } else {
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) exp_tile<1>(scur[rt], c2, mc[rt]);
-        }
-        if constexpr (MASKED) {
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) zero_masked<1>(scur[rt], kv0, q_lim0 + rt * 32, h);
-        }
-        h8 pf[RT][1][2];
-        pv_gemm_steps<RT, 1, DT, NCV, PF>(oacc, pf, vaddr, PAR * T::kVBytes + t * T::kUnitV, [&](int g) {
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) pack_p_group<1>(pf[rt], scur[rt], g, l_run[rt]);
-        });
-      }
-    };
-    run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
-  }
-
-  // ---- epilogue: normalise, round, transpose through LDS, coalesced store ----------------------
-  wait_vmcnt<0>();
-  block_sync();                                  // every wave is done with the K/V buffers
-  float inv[RT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const float l_tot = pair_sum(l_run[rt]);
-    inv[rt] = l_tot > 0.f ? fast_rcp(l_tot) : 0.f;
-    const size_t row = (size_t)bh * seq_q + q0 + wave * WM + rt * 32 + n;
-    const float row_lse = l_tot > 0.f ? m_run[rt] * softmax_scale + __logf(l_tot) : -INFINITY;
+    int tile0 = 0;                                // first kv tile of this block's range
     if constexpr (SPLIT) {
-      if (h == 0) part_lse[(size_t)blockIdx.y * gridDim.x * Br + row] = row_lse;   // gridDim.x * Br = B*H*S_q
-    } else {
-      if (lse != nullptr && h == 0) lse[row] = row_lse;
+      const int per = n_tiles / (int)gridDim.y;   // the launcher guarantees divisibility
+      tile0 = (int)blockIdx.y * per;
+      n_tiles = per;
+      n_full = per;
     }
-  }
-  if constexpr (SPLIT) {
-    const size_t rows_total = (size_t)gridDim.x * Br;
-    store_o_tile<RT, DT, D, T::kOStride32, float>(
-        oacc, inv, smem + wave * WM * T::kOStride32,
-        part_o + ((size_t)blockIdx.y * rows_total + (size_t)bh * seq_q + q0 + wave * WM) * D, lane);
-  } else {
-    store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + wave * WM * T::kOStride,
-                                         o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+    const char* kg = reinterpret_cast<const char*>(k + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * Kd);
+    const char* vg = reinterpret_cast<const char*>(v + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * D);
+
+    if (!prefetched) load_q_frags<RT, KS, Kd>(qf, q + ((size_t)bh * seq_q + q0 + wave * WM + n) * Kd + 8 * h);
+    // PERSIST: where the next row block of this block starts (tile numbers map to (head, row block) as above)
+    const int vb_next = vb + (int)gridDim.x;
+    const bool has_next = PERSIST && vb_next < n_items;
+    const int tile_next = has_next ? xcd_remap(vb_next, n_items) : tile;
+    const size_t bh_next = (size_t)(tile_next / Tr), q0_next = (size_t)(tile_next % Tr) * Br;
+    const char* const kg_next = reinterpret_cast<const char*>(k + bh_next * seq_k * Kd);
+    const char* const vg_next = reinterpret_cast<const char*>(v + bh_next * seq_k * D);
+    const half_t* const q_next = q + (bh_next * seq_q + q0_next + wave * WM + n) * Kd + 8 * h;
+    f16v oacc[RT][DT];
+    float m_run[RT], l_run[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      m_run[rt] = -INFINITY;
+      l_run[rt] = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] = zero16();
+    }
+    const int q_lim0 = q0 + wave * WM + n + diag;   // last kv index row n of row group 0 may see
+
+    if constexpr (!PIPE) {
+      // ============================ plain schedule =================================================
+      if (n_tiles > 0 && !prefetched) {
+        kdma.issue(kg, kbuf, wave_base);
+        if constexpr (NSV == 2) vdma.issue(vg, vbuf, wave_base);
+      }
+      // `parity_tag` carries j & 1 as a compile-time value so that every LDS address of the tile is a
+      // per-lane constant plus an immediate.
+      auto kv_tile = [&](const int j, auto parity_tag, auto masked_tag) {
+        constexpr int PAR = decltype(parity_tag)::value;
+        constexpr bool MASKED = decltype(masked_tag)::value;   // the causal diagonal may cross this tile
+        char* const vcur = vbuf + (NSV == 2 ? PAR * T::kVBytes : 0);
+        const bool more = (j + 1 < n_tiles);
+        if constexpr (WPE == 1) {
+          // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
+          // output accumulators in the accumulation half and the Q fragments in the vector half, or the
+          // allocator parks Q there and copies four registers back in front of every MFMA.
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
+          }
+        }
+
+        // (A) K_j (and with two V buffers V_j) has landed; every wave is past iteration j-1.
+        if (PERSIST && j == 0 && prefetched) {     // the previous row block's output stores stay in flight
+          if (lse != nullptr) wait_vmcnt<TP::kOutputStores + RT>();
+          else wait_vmcnt<TP::kOutputStores>();
+        } else {
+          wait_vmcnt<0>();
+        }
+        block_sync();
+        if constexpr (NSV == 1) vdma.issue(vg + (size_t)j * T::kVBytes, vcur, wave_base);
+        if (more) {
+          if constexpr (NSK == 2) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf + (PAR ^ 1) * T::kKBytes, wave_base);
+          if constexpr (NSV == 2) vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + (PAR ^ 1) * T::kVBytes, wave_base);
+        }
+        if constexpr (PERSIST) {
+          if (!more && has_next) {                 // tile 0 of the next row block, into the buffers it will look in
+            kdma.issue(kg_next, kbuf + (PAR ^ 1) * T::kKBytes, wave_base);
+            vdma.issue(vg_next, vbuf + (PAR ^ 1) * T::kVBytes, wave_base);
+          }
+        }
+
+        f16v sacc[RT][NT];
+        qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
+        if constexpr (PERSIST) {
+          if (!more && has_next) load_q_frags_async<RT, KS, Kd>(qf, q_next);   // the last scores of this row block are done; waited for at (A)
+        }
+
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
+          const float mc = lazy_max_step<NT, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
+          exp_tile<NT>(sacc[rt], c2, mc);
+          if constexpr (MASKED) zero_masked<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
+        }
+
+        // (B) with one buffer: V_j must have landed / K buffer must be free before K_{j+1} is fetched.
+        if constexpr (NSV == 1 || NSK == 1) {
+          if constexpr (NSV == 1) wait_vmcnt<0>();
+          block_sync();
+          if constexpr (NSK == 1) {
+            if (more) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf, wave_base);
+          }
+        }
+        h8 pf[RT][NT][2];
+        pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) pack_p_group<NT>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
+        });
+      };
+      run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
+    } else {
+      // ============================ pipelined schedule =============================================
+      // The unit of work is 32 kv rows.  While unit u is exponentiated, the MFMAs of unit u+1's scores
+      // run underneath; then O += V_u^T P_u runs with the fp16 packing of P_u underneath.  Two score
+      // tiles are live (current, next).
+      //
+      // K is copied in Bc-row tiles that are SHIFTED by one unit against the V tiles: K copy j holds kv
+      // rows [j*Bc + 32, (j+1)*Bc + 32), exactly the units whose scores are computed during iteration j
+      // (units 1..NT-1 of tile j and unit 0 of tile j+1).  So iteration j reads K buffer j&1 only, while
+      // copy j+1 streams into the other one; V tile j is read from V buffer j&1 while V_{j+1} streams
+      // in.  One barrier per Bc rows.  Rows [0, 32) are fetched on their own in the prologue.
+      constexpr int KI = T::kKInstrPerUnit;        // DMA instructions per 32 rows of K
+      f16v sbuf[2][RT][1];
+      auto issue_k_copy = [&](int jj, char* dst) { // K copy jj; the last one stops at the end of the range
+        const char* src = kg + (size_t)jj * T::kKBytes + T::kUnitK;
+        if (jj + 1 < n_tiles) kdma.issue(src, dst, wave_base);
+        else kdma.template issue_part<0, (NT - 1) * KI>(src, dst, wave_base);
+      };
+      if (n_tiles > 0) {
+        kdma.template issue_part<0, KI>(kg, kbuf + T::kKBytes + (NT - 1) * T::kUnitK, wave_base);   // rows [0, 32)
+        issue_k_copy(0, kbuf);
+        vdma.issue(vg, vbuf, wave_base);
+        wait_vmcnt<0>();
+        block_sync();
+        qk_gemm_steps<RT, 1, KS, NCK, PF>(sbuf[0], qf, kaddr, T::kKBytes + (NT - 1) * T::kUnitK, [](int) {});
+      }
+      auto kv_tile = [&](const int j, auto parity_tag, auto masked_tag) {
+        constexpr int PAR = decltype(parity_tag)::value;
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        const bool last_tile = (j + 1 >= n_tiles);
+        if constexpr (WPE == 1) {
+          // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
+          // output accumulators in the accumulation half and the Q fragments in the vector half, or the
+          // allocator parks Q there and copies four registers back in front of every MFMA.
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
+          }
+        }
+        // K copy j and V_j have landed; every wave finished iteration j-1 (frees the other buffers).
+        wait_vmcnt<0>();
+        block_sync();
+        if (!last_tile) {
+          issue_k_copy(j + 1, kbuf + (PAR ^ 1) * T::kKBytes);
+          vdma.issue(vg + (size_t)(j + 1) * T::kVBytes, vbuf + (PAR ^ 1) * T::kVBytes, wave_base);
+        }
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const int cur = (PAR * NT + t) & 1;                        // which score buffer holds unit (j, t)
+          auto& scur = sbuf[cur];
+          auto& snext = sbuf[cur ^ 1];
+          const int kv0 = j * Bc + 32 * t;
+          float mc[RT];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            if constexpr (MASKED) causal_mask<1>(scur[rt], kv0, q_lim0 + rt * 32, h);
+            mc[rt] = lazy_max_step<1, DT>(scur[rt], m_run[rt], l_run[rt], oacc[rt], c2);
+          }
+          constexpr int kPerStep = (16 + KS - 1) / KS;               // exponentials per MFMA step
+          if (t + 1 < NT || !last_tile) {
+            // scores of the next unit: slot t of K buffer PAR
+            qk_gemm_steps<RT, 1, KS, NCK, PF>(snext, qf, kaddr, PAR * T::kKBytes + t * T::kUnitK, [&](int step) {
+#pragma unroll
+              for (int rt = 0; rt < RT; ++rt) exp_range<1>(scur[rt], step * kPerStep, kPerStep, c2, mc[rt]);
+            });
+          } else {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) exp_tile<1>(scur[rt], c2, mc[rt]);
+          }
+          if constexpr (MASKED) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) zero_masked<1>(scur[rt], kv0, q_lim0 + rt * 32, h);
+          }
+          h8 pf[RT][1][2];
+          pv_gemm_steps<RT, 1, DT, NCV, PF>(oacc, pf, vaddr, PAR * T::kVBytes + t * T::kUnitV, [&](int g) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) pack_p_group<1>(pf[rt], scur[rt], g, l_run[rt]);
+          });
+        }
+      };
+      run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
+    }
+
+    // ---- epilogue: normalise, round, store -------------------------------------------------------
+    if constexpr (!PERSIST) {
+      wait_vmcnt<0>();
+      block_sync();                                // every wave is done with the K/V buffers
+    } else if constexpr (TP::kSharesBuffers) {
+      block_sync();                                // every wave is done with the parity-1 buffers
+    }
+    float inv[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const float l_tot = pair_sum(l_run[rt]);
+      inv[rt] = l_tot > 0.f ? fast_rcp(l_tot) : 0.f;
+      const size_t row = (size_t)bh * seq_q + q0 + wave * WM + rt * 32 + n;
+      const float row_lse = l_tot > 0.f ? m_run[rt] * softmax_scale + __logf(l_tot) : -INFINITY;
+      if constexpr (SPLIT) {
+        if (h == 0) part_lse[(size_t)blockIdx.y * gridDim.x * Br + row] = row_lse;   // gridDim.x * Br = B*H*S_q
+      } else {
+        if (lse != nullptr && h == 0) lse[row] = row_lse;
+      }
+    }
+    if constexpr (SPLIT) {
+      const size_t rows_total = (size_t)gridDim.x * Br;
+      store_o_tile<RT, DT, D, T::kOStride32, float>(
+          oacc, inv, smem + wave * WM * T::kOStride32,
+          part_o + ((size_t)blockIdx.y * rows_total + (size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+    } else if constexpr (PERSIST) {
+      store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + TP::stage_offset(wave),
+                                           o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+    } else {
+      // transposed through LDS for 16-byte coalesced stores
+      store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + wave * WM * T::kOStride,
+                                           o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+    }
+    if (!has_next) break;
+    prefetched = true;
   }
 #ifdef AAT_CLOCK_PROBE
   if (lse != nullptr && tid == 0 && (blockIdx.x % 64) == 0) {

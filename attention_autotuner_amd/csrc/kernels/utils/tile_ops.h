@@ -18,6 +18,20 @@ AAT_DEV void load_q_frags(h8 (&qf)[RT][KS], const half_t* qrow) {
       qf[rt][ks] = *reinterpret_cast<const h8*>(qrow + (size_t)rt * 32 * Kd + 16 * ks);
 }
 
+// The same loads issued behind the compiler's back, into registers that already hold fragments: for a
+// prefetch that stays in flight across a loop the compiler would otherwise answer with vmcnt(0) in front of
+// every use of qf, LDS-DMA copies in flight included.  The caller waits (vmcnt) before the next use.
+template <int RT, int KS, int Kd>
+AAT_DEV void load_q_frags_async(h8 (&qf)[RT][KS], const half_t* qrow) {
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const half_t* row = qrow + (size_t)rt * 32 * Kd;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "+v"(qf[rt][ks]) : "v"(row), "n"(32 * ks) : "memory");
+  }
+}
+
 // Byte offsets, inside a Rows16-swizzled [rows][Kd] tile, of this lane's A-operand chunks for tile row n.
 template <int KS, int NCK, Swz MODE = Swz::Rows16>
 AAT_DEV void k_frag_offsets(int (&koff)[KS], int n, int h) {

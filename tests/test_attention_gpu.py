@@ -63,6 +63,9 @@ def test_config2_headline_b4_h32_s2048_d128(causal):
     assert err0 <= TOL
     again = aat.flash_attn_func(qc, kc, vc, ARCH, causal)
     assert torch.equal(o, again)                                    # deterministic
+    # one batch element at a time (the tuner may pick another tiling for that problem)
+    alone = aat.flash_attn_func(qc[2:3], kc[2:3], vc[2:3], ARCH, causal)
+    assert (alone[0].float() - o[2].float()).abs().max().item() <= 1e-3
 
 
 def test_config5_long_kv_b1_h32_sq256_sk16384_d128():
@@ -108,6 +111,49 @@ def test_every_configuration_agrees_with_the_oracle(dqk, dv):
             assert _err(o, refs[causal]) <= TOL, (cfg, causal)
         ran += 1
     assert ran >= 3
+
+
+def _persistent_ok(br, bc, nt, sq, sv, wpe, dqk, dv):
+    """Mirror of AttnFwdRegfuse::Persist<WPE>::kOk (csrc/kernels/attention/regfuse/regfuse.h)."""
+    nw = nt // 64
+    stage = (br // nw) * (dv * 2 + 16)
+    main = sq * bc * dqk * 2 + sv * bc * dv * 2
+    budget = (160 * 1024 // max(1, wpe * 4 // nw)) & ~2047
+    smem = max(min(main + nw * stage, budget), main)
+    return (sq, sv) == (2, 2) and (smem - main) // stage + bc * dqk * 2 // stage + bc * dv * 2 // stage >= nw
+
+
+@pytest.mark.parametrize("dqk,dv", PARITY_DIMS)
+def test_persistent_blocks_agree_with_the_oracle(dqk, dv):
+    """More row blocks than the chip holds at once: non-causal launches of the configurations that have a
+    persistent variant walk several row blocks per block (unevenly: 2080, 1040 or 520 row blocks)."""
+    q, k, v = _inputs(2, 130, 512, 256, dqk, dv, seed=11)
+    ref = ref_op.attention_ref(q, k, v, None, False)
+    ref_lse = torch.logsumexp(q.float() @ k.float().transpose(-1, -2) / math.sqrt(dqk), dim=-1)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    ran = 0
+    for br, bc, nt, sq, sv, wpe in CONFIGS:
+        cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+        if not gfx950_space.forward_valid(cfg, ARCH) or not _persistent_ok(br, bc, nt, sq, sv, wpe, dqk, dv):
+            continue
+        o = torch.zeros(2, 130, 512, dv, dtype=torch.float16, device="cuda")
+        lse = torch.zeros(2, 130, 512, dtype=torch.float32, device="cuda")
+        Runtime(ARCH, cfg).apply([qc, kc, vc, o], lse=lse)
+        assert _err(o, ref) <= TOL, cfg
+        assert (lse.cpu() - ref_lse).abs().max().item() <= 1e-3, cfg
+        plain_entry = torch.zeros_like(o)
+        Runtime(ARCH, cfg).apply([qc, kc, vc, plain_entry])            # without the log-sum-exp output
+        assert torch.equal(plain_entry, o), cfg
+        # one (batch, head) at a time the same library takes the one-row-block-per-block path: same bits
+        single = torch.zeros(1, 1, 512, dv, dtype=torch.float16, device="cuda")
+        for b, h in ((0, 0), (1, 77), (1, 129)):
+            Runtime(ARCH, cfg).apply([qc[b:b + 1, h:h + 1].contiguous(), kc[b:b + 1, h:h + 1].contiguous(),
+                                      vc[b:b + 1, h:h + 1].contiguous(), single])
+            assert torch.equal(single[0, 0], o[b, h]), (cfg, b, h)
+        ran += 1
+    if ran == 0 and dqk > 128:
+        pytest.skip("no valid configuration of the parity set has a persistent variant at this head size")
+    assert ran >= 1
 
 
 @pytest.mark.parametrize("dqk,dv", [(64, 64), (128, 128), (256, 512)])
