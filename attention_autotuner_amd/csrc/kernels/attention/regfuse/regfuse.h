@@ -264,18 +264,26 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
           }
         }
 
+        // A wave none of whose rows sees any kv row of this tile (above the diagonal) only keeps the block's
+        // copies and barriers going: its P would be all zeros, which changes neither O nor l nor the maximum.
+        bool wave_sees = true;
+        if constexpr (MASKED) wave_sees = j * Bc <= q0 + wave * WM + WM - 1 + diag;
+
         f16v sacc[RT][NT];
-        qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
+        if (wave_sees) {
+          qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
+        }
         if constexpr (PERSIST) {
           if (!more && has_next) load_q_frags_async<RT, KS, Kd>(qf, q_next);   // the last scores of this row block are done; waited for at (A)
         }
-
+        if (wave_sees) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
-          const float mc = lazy_max_step<NT, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
-          exp_tile<NT>(sacc[rt], c2, mc);
-          if constexpr (MASKED) zero_masked<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
+          for (int rt = 0; rt < RT; ++rt) {
+            if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
+            const float mc = lazy_max_step<NT, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
+            exp_tile<NT>(sacc[rt], c2, mc);
+            if constexpr (MASKED) zero_masked<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
+          }
         }
 
         // (B) with one buffer: V_j must have landed / K buffer must be free before K_{j+1} is fetched.
@@ -286,11 +294,13 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
             if (more) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf, wave_base);
           }
         }
-        h8 pf[RT][NT][2];
-        pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
+        if (wave_sees) {
+          h8 pf[RT][NT][2];
+          pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
 #pragma unroll
-          for (int rt = 0; rt < RT; ++rt) pack_p_group<NT>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
-        });
+            for (int rt = 0; rt < RT; ++rt) pack_p_group<NT>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
+          });
+        }
       };
       run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
     } else {
