@@ -284,3 +284,27 @@ def test_forward_replays_from_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(o, eager)
         assert _err(o, ref_op.attention_ref(q2, k2, v2, None, True)) <= TOL
+
+
+def test_persistent_forward_replays_from_a_captured_graph():
+    """The same for a launch that takes the persistent-block kernel (more row blocks than the chip holds)."""
+    cfg = AttnConfig(256, 128, 128, 128, 128, 128, 2, 2, 512, True, waves_per_eu=2).set_fuse_type("register")
+    assert _persistent_ok(256, 128, 512, 2, 2, 2, 128, 128)
+    q, k, v = (t.cuda() for t in _inputs(2, 130, 512, 256, 128, 128, seed=31))
+    rt = Runtime(ARCH, cfg)
+    o = torch.empty_like(q)
+    rt.apply([q, k, v, o])                               # first call outside capture: one-time set-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rt.apply([q, k, v, o])
+    for seed in (32, 33):
+        q2, k2, v2 = _inputs(2, 130, 512, 256, 128, 128, seed=seed)
+        q.copy_(q2.cuda()), k.copy_(k2.cuda()), v.copy_(v2.cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(o)
+        rt.apply([q, k, v, eager])
+        torch.cuda.synchronize()
+        assert torch.equal(o, eager)
+        assert _err(o, ref_op.attention_ref(q2, k2, v2, None, False)) <= TOL
