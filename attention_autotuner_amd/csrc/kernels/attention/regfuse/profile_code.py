@@ -7,6 +7,7 @@ include/aat_kernel_abi.h.  Same role as reference csrc/kernels/attention/regfuse
 
 global_vars = r"""
 #define AAT_OP_ATTN 1
+#include <atomic>
 #include "aat_kernel_abi.h"
 #include "kernels/attention/regfuse/regfuse.h"
 #include "kernels/utils/host_launch.h"
@@ -51,19 +52,21 @@ const auto kernel_persist = persistent_kernel<PersistTraits::kOk && !sw_pipeline
 
 // Blocks of the persistent kernel the current device holds at once (0: unknown, do not use it).
 int resident_blocks() {{
-  static int cached[64] = {{}};
+  static std::atomic<int> cached[64];            // per device; threads that race here compute the same value
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (cached[dev] == 0) {{
+  int blocks = cached[dev].load(std::memory_order_relaxed);
+  if (blocks == 0) {{
     int per_cu = 0, cus = 0;
     if (aat::allow_lds(kernel_persist, shared_mem_persist) != hipSuccess ||
         hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel_persist), Nthreads, shared_mem_persist) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || per_cu <= 0 || cus <= 0)
-      cached[dev] = -1;
+      blocks = -1;
     else
-      cached[dev] = per_cu * cus;
+      blocks = per_cu * cus;
+    cached[dev].store(blocks, std::memory_order_relaxed);
   }}
-  return cached[dev] > 0 ? cached[dev] : 0;
+  return blocks > 0 ? blocks : 0;
 }}
 
 size_t split_workspace_bytes(int B, int H, int Seq_q) {{
