@@ -8,18 +8,40 @@ class AttnBwdConfig(BaseConfig):
 
     Two kernels share the tile shape: a column kernel (``Br`` kv rows resident per block, q/dO tiles of
     ``Bc`` rows streamed) producing dV and dK, and a row kernel (``Br`` q rows resident, k/v tiles of
-    ``Bc`` rows streamed) producing dQ.  ``num_stages_qk`` is the number of LDS buffers of the stream."""
+    ``Bc`` rows streamed) producing dQ.  ``num_stages_qk`` is the number of LDS buffers of the stream.
+    ``row_waves_per_eu`` is the register budget (resident waves per SIMD) the row kernel is compiled for: with
+    one output instead of two it fits 256 registers where the column kernel needs the whole file, and two
+    waves per SIMD overlap one wave's matrix work with the other's exponentials."""
     operation = "attn_bwd"
     kernel_subdir = "attention/bwd"
     _fields = ("Br", "Bc", "Kd", "D", "Nthreads", "num_stages_qk")
 
-    def __init__(self, Br, Bc, Kd, D, Nthreads=256, num_stages_qk=3, waves_per_eu=1):
+    def __init__(self, Br, Bc, Kd, D, Nthreads=256, num_stages_qk=3, waves_per_eu=1, row_waves_per_eu=None):
         super().__init__(Br, Bc, Kd, D, Kd, num_stages_qk, Nthreads, True)
         self.waves_per_eu = waves_per_eu
+        self.row_waves_per_eu = row_waves_per_eu or waves_per_eu
         self.fuse_type = "bwd"
 
+    @classmethod
+    def from_dict(cls, dd):
+        cfg = super().from_dict(dd)
+        if "row_waves_per_eu" not in dd:                       # records written before the knob existed
+            cfg.row_waves_per_eu = cfg.waves_per_eu
+        return cfg
+
+    def _extras(self):
+        out = super()._extras()
+        if self.row_waves_per_eu != self.waves_per_eu:
+            out.append(f"rw{self.row_waves_per_eu}")
+        return out
+
     def __repr__(self):
-        return "AttnBwdConfig(" + ", ".join(f"{f}={getattr(self, f)}" for f in self._fields) + ")"
+        body = ", ".join(f"{f}={getattr(self, f)}" for f in self._fields)
+        if self.waves_per_eu != 1:
+            body += f", waves_per_eu={self.waves_per_eu}"
+        if self.row_waves_per_eu != self.waves_per_eu:
+            body += f", row_waves_per_eu={self.row_waves_per_eu}"
+        return f"AttnBwdConfig({body})"
 
     def __str__(self):
         return "_".join([self.operation] + [str(getattr(self, f)) for f in self._fields] + self._extras())

@@ -301,10 +301,26 @@ def attn_backward_valid(cfg, arch):
             return False
     if attn_backward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
         return False
+    row_wpe = getattr(cfg, "row_waves_per_eu", cfg.waves_per_eu)
+    if row_wpe != cfg.waves_per_eu:
+        if cfg.waves_per_eu != 1 or row_wpe != 2 or nw > 8:
+            return False
+        if attn_backward_row_reg_estimate(cfg) > arch.register_per_thread // 2:
+            return False
+        if attn_backward_lds_bytes(cfg) * max(1, 8 // nw) > arch.smem_cap:
+            return False
     vec, acc = attn_backward_reg_estimate(cfg)
     if cfg.waves_per_eu == 1:
         return vec <= 256 and acc <= 256
     return vec + acc <= arch.register_per_thread // cfg.waves_per_eu
+
+
+def attn_backward_row_reg_estimate(cfg):
+    """Registers of the row kernel (resident Q and dO fragments, the dQ accumulators, S and dP, the fp16
+    operand of the second contraction, addresses): 206 measured at 128/128 with 32-row tiles, 238 with 64."""
+    rt = cfg.Br // _waves(cfg) // MFMA_M
+    nt = cfg.Bc // 32
+    return rt * ((cfg.Kd + cfg.D) // 16) * 4 + rt * (cfg.Kd // 32) * 16 + rt * nt * 32 + rt * nt * 8 + 48
 
 
 def attn_backward_candidates(br, bc, dim_qk, dim_v):
@@ -313,6 +329,7 @@ def attn_backward_candidates(br, bc, dim_qk, dim_v):
         for stages in (2, 3):
             for wpe in (1, 2):
                 out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=wpe))
+            out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=1, row_waves_per_eu=2))
     return out
 
 
@@ -320,7 +337,8 @@ def default_attn_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
     for br, bc, nt, st, wpe in ((128, 32, 256, 3, 1), (128, 32, 256, 2, 1), (64, 32, 128, 3, 1), (64, 32, 128, 2, 1), (64, 32, 128, 2, 2)):
         if any(s and (s % br or s % bc) for s in (seq_q, seq_k)):
             continue
-        cfg = AttnBwdConfig(br, bc, dim_qk, dim_v, nt, st, waves_per_eu=wpe)
-        if attn_backward_valid(cfg, arch):
-            return cfg
+        for row_wpe in ((2, wpe) if wpe == 1 else (wpe,)):            # the row kernel at two waves per SIMD where it fits
+            cfg = AttnBwdConfig(br, bc, dim_qk, dim_v, nt, st, waves_per_eu=wpe, row_waves_per_eu=row_wpe)
+            if attn_backward_valid(cfg, arch):
+                return cfg
     raise ValueError(f"no default attn_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")

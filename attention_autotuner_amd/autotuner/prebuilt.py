@@ -61,7 +61,10 @@ def extra_configs(arch=None):
         for seq in (None, 128, 64):
             out.append(gfx950_space.default_attn_backward_config(*dims, arch, seq, seq))
     for br, bc, nt, st in ATTN_BWD_TILES:
-        out.append(AttnBwdConfig(br, bc, 128, 128, nt, st))
+        for row_wpe in (1, 2):
+            cfg = AttnBwdConfig(br, bc, 128, 128, nt, st, row_waves_per_eu=row_wpe)
+            if gfx950_space.attn_backward_valid(cfg, arch):
+                out.append(cfg)
     for dqk, dv in PARITY_DIMS:
         for br, bc, nt, sq, sv, wpe in PARITY_TILES:
             cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")

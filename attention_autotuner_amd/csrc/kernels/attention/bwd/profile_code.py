@@ -21,12 +21,13 @@ constexpr int D = {D};
 constexpr int Nthreads = {Nthreads};
 constexpr int num_stages = {num_stages_qk};      // LDS buffers of the streamed tiles
 constexpr int waves_per_eu = {waves_per_eu};
+constexpr int row_waves_per_eu = {row_waves_per_eu};   // register budget of the row kernel (one output: fits 256 registers)
 
 using aat::AttnBwdPass;
 using TC = aat::AttnBwdChain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Col>;
 using TR = aat::AttnBwdChain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Row>;
 const auto kernel_col = &aat::attn_bwd_chain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Col, waves_per_eu>;
-const auto kernel_row = &aat::attn_bwd_chain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Row, waves_per_eu>;
+const auto kernel_row = &aat::attn_bwd_chain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Row, row_waves_per_eu>;
 
 bool bwd_shape_ok(int B, int H, int Seq_q, int Seq_k) {{
   // every sequence length plays both roles (resident rows in one kernel, streamed rows in the other)
