@@ -3,6 +3,8 @@ import os
 import re
 
 import pytest
+
+from attention_autotuner_amd.autotuner import gfx950_space
 import torch
 
 from attention_autotuner_amd.arch import A100, RTX4090, MI355X
@@ -101,6 +103,21 @@ def test_config_text_forms_and_roundtrip():
         assert back.template_dir and os.path.isdir(back.template_dir)
     w = AttnConfig(128, 64, 128, 128, 128, 64, 2, 2, 256, True, waves_per_eu=2).set_fuse_type("register")
     assert str(w).endswith("_w2") and "waves_per_eu=2" in repr(w)
+    # attention backward: the row kernel's own register budget is part of the key and of the log line,
+    # and records written before the knob existed read back with both kernels on the same budget
+    from attention_autotuner_amd.autotuner.configs import AttnBwdConfig
+    a = AttnBwdConfig(128, 64, 128, 128, 256, 2, row_waves_per_eu=2)
+    assert str(a) == "attn_bwd_128_64_128_128_256_2_rw2" and repr(a).endswith("num_stages_qk=2, row_waves_per_eu=2)")
+    back = AttnBwdConfig.from_dict(a.to_dict())
+    assert back == a and str(back) == str(a) and back.row_waves_per_eu == 2
+    plain = AttnBwdConfig(128, 64, 128, 128, 256, 2)
+    assert str(plain) == "attn_bwd_128_64_128_128_256_2" and plain.row_waves_per_eu == 1
+    old = {k: v for k, v in plain.to_dict().items() if k != "row_waves_per_eu"}
+    assert AttnBwdConfig.from_dict(old) == plain
+    arch = MI355X()
+    assert gfx950_space.attn_backward_valid(a, arch)
+    assert not gfx950_space.attn_backward_valid(AttnBwdConfig(128, 64, 128, 128, 256, 3, row_waves_per_eu=2), arch)   # two 99 KB blocks
+    assert not gfx950_space.attn_backward_valid(AttnBwdConfig(128, 32, 256, 256, 256, 2, row_waves_per_eu=2), arch)  # registers
 
 
 def test_mi355x_space_is_valid_and_nonempty():
