@@ -3,12 +3,10 @@ import os
 import re
 
 import pytest
-
-from attention_autotuner_amd.autotuner import gfx950_space
 import torch
 
 from attention_autotuner_amd.arch import A100, RTX4090, MI355X
-from attention_autotuner_amd.autotuner import AttnTunner, RetTunner, RetBwdTunner, AttnConfig, RetConfig, RetBwdConfig
+from attention_autotuner_amd.autotuner import AttnTunner, RetTunner, RetBwdTunner, AttnConfig, RetConfig, RetBwdConfig, gfx950_space
 from attention_autotuner_amd.autotuner.configs import balanced_wave_split, supported_configs
 
 GOLD = os.path.join(os.path.dirname(__file__), "golden", "tuning_logs")
