@@ -35,11 +35,11 @@ constexpr int shared_mem_split = Traits::kSmemBytesSplit;
 // Persistent variant (a block walks several row blocks, prefetching across them): exists for two K and two V
 // buffers, the plain schedule and a tile shape that leaves room to stage the output beside the prefetched
 // tiles; used for non-causal problems with an even number of kv tiles and more row blocks than the chip holds
-// at once -- and with fewer than 16 kv tiles per row block.  Measured with the Br=256 Bc=128 512-thread
+// at once -- and with fewer than 2048 kv rows.  Measured with the Br=256 Bc=128 512-thread
 // configuration under sustained load (300 launches back to back): +10 % at S=512 (B 16, H 32), +3 % at S=1024,
 // +-0 at S=2048, -1.5 % at S=4096: what it removes is the 5.7 us a block spends per row block on start-up and
 // drain, and on long rows the kernel runs at the chip's power limit, where idle time is not what bounds it.
-constexpr int kPersistMaxTiles = 14;
+constexpr int kPersistMaxKv = 1792;
 using PersistTraits = Traits::Persist<waves_per_eu>;
 constexpr int shared_mem_persist = PersistTraits::kSmemBytes;
 template <bool OK> auto persistent_kernel() {{
@@ -91,7 +91,7 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int
     return hipGetLastError();
   }}
   const int items = B * H * (Seq_q / Br);
-  if (kernel_persist != nullptr && !causal && (Seq_k / Bc) % 2 == 0 && Seq_k / Bc <= kPersistMaxTiles) {{
+  if (kernel_persist != nullptr && !causal && (Seq_k / Bc) % 2 == 0 && Seq_k <= kPersistMaxKv) {{
     const int resident = resident_blocks();
     if (resident > 0 && items > resident) {{
       kernel_persist<<<dim3(resident), dim3(Nthreads), shared_mem_persist, stream>>>(
