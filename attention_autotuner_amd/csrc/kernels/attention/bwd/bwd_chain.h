@@ -261,37 +261,53 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
     qk_gemm_steps<RT, NT, KS, NCK, PF, kVacc>(s, x1f, y1addr, off, [](int) {});
     qk_gemm_steps<RT, NT, DS, NCD, PF, kVacc>(dp, x2f, y2addr, off, [](int) {});
 
-    // P = exp2(s*c2 - lse2[q]),  dS = P * (dP - delta[q]);  register v of tile t is streamed row 32t + 8(v/4) + 4h + v%4
+    // P = exp2(s*c2 - lse2[q]),  dS = P * (dP - delta[q]);  register v of tile t is streamed row 32t + 8(v/4) + 4h + v%4.
+    // Only a tile the diagonal crosses runs the masking code.  COL: the statistics of the streamed rows come
+    // from LDS four rows at a time, read by hand one group ahead (a tracked read here is answered with a
+    // full lgkmcnt(0) per group: eight exposed LDS round trips per tile for the only wave of the SIMD).
     const bool diag_tile = causal && (COL ? (x0 + BX - 1 > j * BY + diag) : ((j + 1) * BY - 1 > x0 + diag));
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      const int xrow = x0 + wave * WM + rt * 32 + n;             // resident row of this lane
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          f4v l2, dl;
-          if constexpr (COL) {
-            l2 = *reinterpret_cast<AAT_AS3 const f4v*>((uintptr_t)(stat_addr + off + (32 * t + 8 * g) * 4));
-            dl = *reinterpret_cast<AAT_AS3 const f4v*>((uintptr_t)(stat_addr + off + (BY + 32 * t + 8 * g) * 4));
-          }
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int v = 4 * g + e;
-            const float lrow = COL ? l2[e] : lse_row[rt];
-            const float drow = COL ? dl[e] : delta_row[rt];
-            float p = fast_exp2(s[rt][t][v] * c2 - lrow);
-            if (diag_tile) {
-              const int yrow = j * BY + 32 * t + 8 * g + 4 * h + e;   // streamed row
-              const int qi = COL ? yrow : xrow, ki = COL ? xrow : yrow;
-              if (ki > qi + diag) p = 0.f;
-            }
-            s[rt][t][v] = p;
-            dp[rt][t][v] = p * (dp[rt][t][v] - drow);
+    auto softmax_part = [&](auto masked_tag) {
+      constexpr bool MASKED = decltype(masked_tag)::value;
+      constexpr int G = RT * NT * 4;                                 // groups of four streamed rows
+      f4v l2r[2], dlr[2];
+      auto read_stats = [&](auto it) {
+        constexpr int i = decltype(it)::value, tg = i % (NT * 4);    // the statistics do not depend on rt
+        l2r[i % 2] = lds_read_f4_async(stat_addr, off + (32 * (tg / 4) + 8 * (tg % 4)) * 4);
+        dlr[i % 2] = lds_read_f4_async(stat_addr, off + (BY + 32 * (tg / 4) + 8 * (tg % 4)) * 4);
+      };
+      if constexpr (COL) read_stats(std::integral_constant<int, 0>{});
+      static_for<G>([&](auto it) {
+        constexpr int i = decltype(it)::value, rt = i / (NT * 4), t = (i / 4) % NT, g = i % 4;
+        f4v l2 = l2r[i % 2], dl = dlr[i % 2];
+        if constexpr (COL) {
+          if constexpr (i + 1 < G) {
+            read_stats(std::integral_constant<int, i + 1>{});
+            lds_wait_younger<2>(l2, dl);
+          } else {
+            lds_wait_younger<0>(l2, dl);
           }
         }
-      }
-    }
+        // The score of resident row x and streamed row y = j*BY + c + 4h (c = 32t + 8g + e, a constant) is masked
+        // when kv > q + diag: COL (x is kv) x - diag - j*BY - 4h > c, ROW (x is q) c > x + diag - j*BY - 4h.
+        const int xrow = x0 + wave * WM + rt * 32 + n;               // resident row of this lane
+        const int lim = (COL ? xrow - diag : xrow + diag) - j * BY - 4 * h;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          constexpr int vbase = 4 * g, cbase = 32 * t + 8 * g;
+          const int v = vbase + e;
+          const float lrow = COL ? l2[e] : lse_row[rt];
+          const float drow = COL ? dl[e] : delta_row[rt];
+          float p = fast_exp2(s[rt][t][v] * c2 - lrow);
+          if constexpr (MASKED) {
+            if (COL ? lim > cbase + e : cbase + e > lim) p = 0.f;
+          }
+          s[rt][t][v] = p;
+          dp[rt][t][v] = p * (dp[rt][t][v] - drow);
+        }
+      });
+    };
+    if (diag_tile) softmax_part(std::true_type{});
+    else softmax_part(std::false_type{});
 
     // second contractions: COL  dV^T += dO^T P  and  dK^T += Q^T dS;   ROW  dQ^T += K^T dS
     h8 ef[RT][NT][2];

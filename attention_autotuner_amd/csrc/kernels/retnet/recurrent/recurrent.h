@@ -180,11 +180,6 @@ AAT_DEV float lds_read_f1_async(uint32_t base, int imm) {
   asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(base), "i"(imm));
   return v;
 }
-AAT_DEV f4v lds_read_f4_async(uint32_t base, int imm) {
-  f4v v;
-  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(base), "i"(imm));
-  return v;
-}
 template <int N, class V> AAT_DEV void lds_wait_younger_f(V& v) {
   static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));

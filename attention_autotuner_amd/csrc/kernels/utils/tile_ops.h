@@ -95,6 +95,18 @@ template <int N> AAT_DEV void lds_wait_younger(h8& v) {
   asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(v) : "n"(N));
 }
 
+// Four consecutive floats, issued the same way (per-row statistics that travel with a streamed tile).
+AAT_DEV f4v lds_read_f4_async(uint32_t base, int imm) {
+  f4v v;
+  const uint32_t hi = (uint32_t)imm & ~0xffffu;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(base + hi), "i"(imm & 0xffff));
+  return v;
+}
+template <int N> AAT_DEV void lds_wait_younger(f4v& a, f4v& b) {
+  static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+
 // MFMA with its accumulator forced into vector registers.  A kernel that owns more than 256 registers
 // gets every compiler-issued MFMA in the form that accumulates in the 256 accumulation registers; when
 // the output accumulators fill those, the short-lived score tile has to live in vector registers, which
