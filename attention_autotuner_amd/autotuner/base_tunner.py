@@ -86,7 +86,8 @@ class BaseTunner:
         if ns > 1 and (s["Sk"] // config.Bc) % ns:
             return False
         if config.operation in ("ret_bwd", "attn_bwd"):   # both lengths are resident in one pass, streamed in another
-            return all(s[n] % config.Br == 0 and s[n] % config.Bc == 0 for n in ("Sq", "Sk"))
+            return all(s[n] % config.Br == 0 and s[n] % config.Bc == 0 for n in ("Sq", "Sk")) and \
+                s["Sk"] % getattr(config, "row_Bc", config.Bc) == 0
         return s["Sq"] % config.Br == 0 and s["Sk"] % config.Bc == 0
 
     def get_tuned_configs(self):

@@ -302,12 +302,19 @@ def attn_backward_valid(cfg, arch):
     if attn_backward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
         return False
     row_wpe = getattr(cfg, "row_waves_per_eu", cfg.waves_per_eu)
+    row_bc = getattr(cfg, "row_Bc", cfg.Bc)
+    if row_bc != cfg.Bc:                                     # a tile height of its own only with a budget of its own
+        if row_wpe == cfg.waves_per_eu or row_bc % 32 or row_bc > 128:
+            return False
+        if any((row_bc * cols // 8) % cfg.Nthreads for cols in (cfg.Kd, cfg.D)):
+            return False
     if row_wpe != cfg.waves_per_eu:
         if cfg.waves_per_eu != 1 or row_wpe != 2 or nw > 8:
             return False
         if attn_backward_row_reg_estimate(cfg) > arch.register_per_thread // 2:
             return False
-        if attn_backward_lds_bytes(cfg) * max(1, 8 // nw) > arch.smem_cap:
+        row_lds = max(cfg.num_stages_qk * row_bc * (cfg.Kd + cfg.D) * 2, cfg.Br * (cfg.Kd * 2 + 16))
+        if row_lds * max(1, 8 // nw) > arch.smem_cap:
             return False
     vec, acc = attn_backward_reg_estimate(cfg)
     if cfg.waves_per_eu == 1:
@@ -319,7 +326,7 @@ def attn_backward_row_reg_estimate(cfg):
     """Registers of the row kernel (resident Q and dO fragments, the dQ accumulators, S and dP, the fp16
     operand of the second contraction, addresses): 206 measured at 128/128 with 32-row tiles, 238 with 64."""
     rt = cfg.Br // _waves(cfg) // MFMA_M
-    nt = cfg.Bc // 32
+    nt = getattr(cfg, "row_Bc", cfg.Bc) // 32
     return rt * ((cfg.Kd + cfg.D) // 16) * 4 + rt * (cfg.Kd // 32) * 16 + rt * nt * 32 + rt * nt * 8 + 48
 
 
@@ -329,7 +336,8 @@ def attn_backward_candidates(br, bc, dim_qk, dim_v):
         for stages in (2, 3):
             for wpe in (1, 2):
                 out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=wpe))
-            out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=1, row_waves_per_eu=2))
+            for row_bc in (32, 64):
+                out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=1, row_waves_per_eu=2, row_Bc=row_bc))
     return out
 
 

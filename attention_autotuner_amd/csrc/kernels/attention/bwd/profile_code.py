@@ -15,7 +15,8 @@ global_vars = r"""
 
 namespace {{
 constexpr int Br = {Br};                 // block-resident rows of both kernels
-constexpr int Bc = {Bc};                 // streamed rows per step of both kernels
+constexpr int Bc = {Bc};                 // streamed rows per step of the column kernel
+constexpr int BcRow = {row_Bc};          // streamed rows per step of the row kernel
 constexpr int Kd = {Kd};
 constexpr int D = {D};
 constexpr int Nthreads = {Nthreads};
@@ -25,13 +26,13 @@ constexpr int row_waves_per_eu = {row_waves_per_eu};   // register budget of the
 
 using aat::AttnBwdPass;
 using TC = aat::AttnBwdChain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Col>;
-using TR = aat::AttnBwdChain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Row>;
+using TR = aat::AttnBwdChain<Kd, D, Br, BcRow, Nthreads, num_stages, AttnBwdPass::Row>;
 const auto kernel_col = &aat::attn_bwd_chain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Col, waves_per_eu>;
-const auto kernel_row = &aat::attn_bwd_chain<Kd, D, Br, Bc, Nthreads, num_stages, AttnBwdPass::Row, row_waves_per_eu>;
+const auto kernel_row = &aat::attn_bwd_chain<Kd, D, Br, BcRow, Nthreads, num_stages, AttnBwdPass::Row, row_waves_per_eu>;
 
 bool bwd_shape_ok(int B, int H, int Seq_q, int Seq_k) {{
   // every sequence length plays both roles (resident rows in one kernel, streamed rows in the other)
-  return aat::shape_ok(B, H, Seq_q, Seq_k, Br, Br) && aat::shape_ok(B, H, Seq_q, Seq_k, Bc, Bc);
+  return aat::shape_ok(B, H, Seq_q, Seq_k, Br, Br) && aat::shape_ok(B, H, Seq_q, Seq_k, Bc, BcRow);   // q rows stream through the column kernel, kv rows through the row kernel
 }}
 size_t stats_bytes(int B, int H, int Seq_q) {{ return (size_t)2 * B * H * Seq_q * sizeof(float); }}
 

@@ -105,6 +105,21 @@ def test_tile_variants_agree(br, bc, nt, st, row_wpe):
         assert ok, (cfg, name, worst)
 
 
+def test_row_kernel_with_its_own_tile_height():
+    """Column kernel on 64-row streamed tiles, row kernel (two waves per SIMD) on 32-row ones."""
+    q, k, v, do = _inputs(1, 2, 256, 384, 128, 128, seed=6)
+    o_ref, lse_ref = ref_op.attention_ref(q, k, v, 0.11, True, return_lse=True)
+    cfg = AttnBwdConfig(64, 64, 128, 128, 128, 2, row_waves_per_eu=2, row_Bc=32)
+    assert str(cfg) == "attn_bwd_64_64_128_128_128_2_rw2_rb32" and gfx950_space.attn_backward_valid(cfg, ARCH)
+    arrays = [t.cuda() for t in (q, k, v, o_ref.half(), do, lse_ref)]
+    grads = [torch.empty_like(arrays[0]), torch.empty_like(arrays[1]), torch.empty_like(arrays[2])]
+    Runtime(ARCH, cfg).apply(arrays + grads, softmax_scale=0.11, causal=True)
+    ref = ref_op.attention_bwd_ref(q, k, v, do, 0.11, True)
+    for name, g, r in zip(("dq", "dk", "dv"), grads, ref):
+        ok, worst = _close(g, r)
+        assert ok, (cfg, name, worst)
+
+
 def test_abi_error_paths_and_stream():
     cfg = gfx950_space.default_attn_backward_config(128, 128, ARCH, 128, 128)
     lib = library.load(codegen.compile_config(cfg, ARCH), "attn_bwd")

@@ -108,9 +108,13 @@ def test_config_text_forms_and_roundtrip():
     assert str(a) == "attn_bwd_128_64_128_128_256_2_rw2" and repr(a).endswith("num_stages_qk=2, row_waves_per_eu=2)")
     back = AttnBwdConfig.from_dict(a.to_dict())
     assert back == a and str(back) == str(a) and back.row_waves_per_eu == 2
+    mixed = AttnBwdConfig(128, 64, 128, 128, 256, 2, row_waves_per_eu=2, row_Bc=32)
+    assert str(mixed) == "attn_bwd_128_64_128_128_256_2_rw2_rb32" and repr(mixed).endswith("row_waves_per_eu=2, row_Bc=32)")
+    assert AttnBwdConfig.from_dict(mixed.to_dict()) == mixed and gfx950_space.attn_backward_valid(mixed, MI355X())
+    assert not gfx950_space.attn_backward_valid(AttnBwdConfig(128, 64, 128, 128, 256, 2, row_Bc=32), MI355X())   # only with a budget of its own
     plain = AttnBwdConfig(128, 64, 128, 128, 256, 2)
     assert str(plain) == "attn_bwd_128_64_128_128_256_2" and plain.row_waves_per_eu == 1
-    old = {k: v for k, v in plain.to_dict().items() if k != "row_waves_per_eu"}
+    old = {k: v for k, v in plain.to_dict().items() if k not in ("row_waves_per_eu", "row_Bc")}
     assert AttnBwdConfig.from_dict(old) == plain
     arch = MI355X()
     assert gfx950_space.attn_backward_valid(a, arch)
