@@ -48,29 +48,33 @@ AAT_DEV void apply_mask(f16v (&s)[NT], const uint32_t (&maddr)[NT * 4], int buf_
 // Off the diagonal |lg| * tile_rows bounds the exponents, so nothing overflows for gamma >= 0.5 and
 // tiles of up to 128 rows; far below the diagonal the scalar underflows to zero, as the fp16 tensor does.
 // The offsets split as off = (32t + 8g) + (4h + e) with v = 4g + e, so the 16*NT constants are products
-// of 4*NT + 4 of them: fb[t][g] = exp2(-/+lg * (32t + 8g)), fa[e] = exp2(-/+lg * (4h + e)).
+// of 4*NT + 4 of them: fb[t][g] = exp2(-/+lg * (32t + 8g)), fa[e] = exp2(-/+lg * e), all of them the same in
+// every lane, with the half-wave's share exp2(-/+lg * 4h) folded into the per-tile scalar.
 template <int NT, bool OWN_Q>
 struct DecayMask {
   float fa[4], fb[NT][4];
   float lg;
   int h4;
 
+  // The rate belongs to the head, so lg and the 4*NT factors fb are the same in every lane: passed through
+  // readfirstlane they live in scalar registers (a two-wave kernel at the 256-register limit has none to spare).
+  AAT_DEV static float uniform(float x) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(x))); }
   AAT_DEV void init(float lg2gamma, int h) {
-    lg = lg2gamma;
+    lg = uniform(lg2gamma);
     h4 = 4 * h;
     const float step = OWN_Q ? -lg : lg;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) fa[e] = fast_exp2(step * (float)(h4 + e));
+    for (int e = 0; e < 4; ++e) fa[e] = uniform(fast_exp2(step * (float)e));   // the half-wave's 4h goes into the tile scalar
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) fb[t][g] = fast_exp2(step * (float)(32 * t + 8 * g));
+      for (int g = 0; g < 4; ++g) fb[t][g] = uniform(fast_exp2(step * (float)(32 * t + 8 * g)));
   }
   // s <- s * D * extra for the tile whose origin makes `base` (see above).  DIAG: the diagonal may cross
   // this tile, entries above it are zeroed.
   template <bool DIAG, class Extra>
   AAT_DEV void apply(f16v (&s)[NT], int base, Extra&& extra) const {
-    const float tf = fast_exp2(lg * (float)base);
+    const float tf = fast_exp2(lg * (float)(OWN_Q ? base - h4 : base + h4));
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
