@@ -101,13 +101,29 @@ def hipcc_command(src, out, arch):
     return [hipcc_exe(), *HIPCC_FLAGS, f"--offload-arch={target}", f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", src, "-o", out]
 
 
+class MissingLibraryError(RuntimeError):
+    """A library would have to be compiled and compiling is switched off (AAT_NO_JIT=1)."""
+
+
+def jit_allowed():
+    """AAT_NO_JIT=1 forbids spawning hipcc from this process: a measurement or profiler run must never
+    time a compile, and a process whose GPU a profiler has already initialised must not start children
+    that inherit its preloaded libraries.  Build ahead of time with
+    ``python -m attention_autotuner_amd.autotuner.prebuilt``."""
+    return os.environ.get("AAT_NO_JIT", "0") in ("", "0")
+
+
 def compile_config(config, arch, build_dir=None, timeout=None, force=False):
-    """Build the library for ``config``; returns its path, or None if hipcc failed or timed out."""
+    """Build the library for ``config``; returns its path, or None if hipcc failed or timed out.
+    Raises MissingLibraryError instead of compiling when AAT_NO_JIT=1."""
     if getattr(arch, "platform", "ROCm") != "ROCm":
         return None
     out = library_path(config, build_dir)
     if os.path.exists(out) and not force:
         return out
+    if not jit_allowed():
+        raise MissingLibraryError(f"{out} is not built and AAT_NO_JIT=1 forbids compiling it here; "
+                                  "run `python -m attention_autotuner_amd.autotuner.prebuilt` first")
     os.makedirs(os.path.dirname(out), exist_ok=True)
     src = out[:-3] + ".hip"
     try:

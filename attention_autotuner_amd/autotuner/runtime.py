@@ -83,5 +83,38 @@ class Runtime:
         return rc
 
 
+    def bind(self, torch_array, softmax_scale=None, causal=False, workspace=None):
+        """A zero-argument callable that enqueues one launch of ``kernel_entry_ex`` on ``torch_array``:
+        pointers, sizes, the workspace and the stream (the one current NOW) are converted once, so a
+        call costs one foreign-function call -- what a serving loop that launches the same problem
+        repeatedly would keep.  The tensors (and the returned callable's workspace) must stay alive."""
+        q, k = torch_array[0], torch_array[1]
+        if not q.is_cuda:
+            raise KernelLaunchError("kernel libraries run on the GPU only; got CPU tensors")
+        B, H, Sq, Sk = int(q.shape[0]), int(q.shape[1]), int(q.shape[2]), int(k.shape[2])
+        op = self.config.operation
+        lib = library.load(self._path(), op)
+        need = int(lib.workspace_size(B, H, Sq, Sk))
+        if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        args = [ctypes.c_void_p(t.data_ptr()) for t in torch_array] + [B, H, Sq, Sk]
+        if op in library.SCALED_OPS:
+            args.append(ctypes.c_float(softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])))
+        args += [ctypes.c_int(int(bool(causal))),
+                 ctypes.c_void_p(workspace.data_ptr() if workspace is not None else 0),
+                 ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0)]
+        with torch.cuda.device(q.device):
+            args.append(ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        entry, keep, name = lib.kernel_entry_ex, (list(torch_array), workspace), f"{op}:{self.config}"
+
+        def launch():
+            rc = entry(*args)
+            if rc != 0:
+                raise KernelLaunchError(f"{name} failed with code {rc}: {_ERRORS.get(rc, 'HIP error')}")
+
+        launch.keep_alive = keep
+        return launch
+
+
 def compile_parallel(configs, arch, tmp_dir=None):
     return codegen.compile_parallel(configs, arch, tmp_dir)

@@ -43,23 +43,15 @@ def resolve_config(aat, arch, tensors, causal):
     return cfg
 
 
-def time_launches(fn, steps, warmup):
-    """(wall ms per step, mean kernel ms from per-launch events on the launch stream)."""
-    import torch
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()              # nothing but this between the warm-up and the timed steps: the clock ramps
-    t0 = time.perf_counter()              # up over tens of milliseconds of load and falls back when the GPU idles
-    for i in range(steps):
-        starts[i].record()
-        fn()
-        stops[i].record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    kern_ms = sum(s.elapsed_time(e) for s, e in zip(starts, stops)) / steps
-    return wall_ms, kern_ms
+MIN_WARMUP_MS = 100.0         # wall time of back-to-back launches before anything is timed, whatever --warmup says
+
+
+def time_launches(fn, steps, warmup, before_each=None, flush_l2=False):
+    """Timing of `steps` calls after at least MIN_WARMUP_MS of back-to-back calls plus `warmup` more:
+    the shader clock needs tens of milliseconds of load to settle, so a warm-up counted in launches
+    measures the ramp (a 0.3 ms kernel timed after 5 launches runs 15-20 % below its settled rate)."""
+    from attention_autotuner_amd.benchmarks.do_bench import LaunchTimer
+    return LaunchTimer(MIN_WARMUP_MS).measure(fn, calls=steps, warmup_calls=warmup, before_each=before_each, flush_l2=flush_l2)
 
 
 def cpu_baseline(heads=8):
@@ -101,6 +93,19 @@ def measured_traffic(cfg):
         return None
 
 
+def extra(ms_timing, flops, peak=PEAK_TFLOPS, issued_ratio=None, **more):
+    """One side measurement: median per-call GPU time and its roofline fraction on the algorithmic count."""
+    ms = ms_timing.median
+    out = {"ms": round(ms, 5), "p20_ms": round(ms_timing.quantile(0.2), 5), "p80_ms": round(ms_timing.quantile(0.8), 5),
+           "tflops": round(flops / ms / 1e9, 1),
+           "roofline": {"bound": "mfma", "achieved": round(flops / ms / 1e9, 1), "peak": peak, "unit": "TFLOP/s",
+                        "frac": round(flops / ms / 1e9 / peak, 4), "algorithmic_flops": flops}}
+    if issued_ratio is not None:                  # matrix work the kernels issue / the algorithmic count
+        out["roofline"]["issued_over_algorithmic"] = issued_ratio
+    out.update(more)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -108,6 +113,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the causal / long-kv / RetNet side measurements")
+    ap.add_argument("--no-flush-pass", action="store_true", help="skip the second headline measurement (L2 flushed before each launch)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain 256 MiB device copies, so a profiler's HBM byte counters can be scaled by a known transfer")
     args = ap.parse_args()
@@ -115,6 +121,7 @@ def main():
         log("bench.py measures one GPU: the path has no cross-GPU component (batch x head slices are independent); run with --gpus 1")
         sys.exit(2)
 
+    os.environ.setdefault("AAT_NO_JIT", "1")     # a missing library is an error here, never a compile inside a measurement
     import torch
     import attention_autotuner_amd as aat
     from attention_autotuner_amd.autotuner import Runtime
@@ -144,11 +151,24 @@ def main():
     cfg = resolve_config(aat, arch, [q, k, v, o], False)
     rt = Runtime(arch, cfg)
     log(f"config: {cfg!r}")
-    wall_ms, kern_ms = time_launches(lambda: rt.apply([q, k, v, o], softmax_scale=scale, causal=False), args.steps, args.warmup)
+
+    step = rt.bind([q, k, v, o], softmax_scale=scale, causal=False)     # one kernel_entry_ex call per step
+
+    hot = time_launches(step, args.steps, args.warmup)
+    from attention_autotuner_amd.benchmarks.do_bench import gpu_state_under_load
+    hot.sclk_mhz, hot.power_w = gpu_state_under_load(step)
     flops = attn_flops(B, H, S, S, D, D)
-    value = flops / (wall_ms * 1e-3) / 1e12
-    achieved = flops / (kern_ms * 1e-3) / 1e12
-    log(f"attention fwd non-causal: {wall_ms:.4f} ms/step wall, {kern_ms:.4f} ms/launch (events) -> {achieved:.1f} TFLOP/s = {100 * achieved / PEAK_TFLOPS:.1f}% of peak")
+    value = flops / (hot.wall_ms_per_call * 1e-3) / 1e12
+    achieved = flops / (hot.mean * 1e-3) / 1e12
+    log(f"attention fwd non-causal: {hot.wall_ms_per_call:.4f} ms/step wall, {hot.mean:.4f} ms/launch mean "
+        f"(median {hot.median:.4f}, p20 {hot.quantile(0.2):.4f}, p80 {hot.quantile(0.8):.4f}; warm-up {hot.warmup_calls} launches / {hot.warmup_ms:.0f} ms; "
+        f"sclk {hot.sclk_mhz and round(hot.sclk_mhz)} MHz, {hot.power_w and round(hot.power_w)} W) -> {achieved:.1f} TFLOP/s = {100 * achieved / PEAK_TFLOPS:.1f}% of peak")
+    timing = {"hot_l2": hot.summary()}
+    if not args.no_flush_pass:
+        cold = time_launches(step, args.steps, args.warmup, flush_l2=True)
+        timing["l2_flushed"] = dict(cold.summary(), tflops_median=round(flops / cold.median / 1e9, 1))
+        log(f"  with a 256 MB write before each launch: median {cold.median:.4f} ms (p20 {cold.quantile(0.2):.4f}, p80 {cold.quantile(0.8):.4f}) "
+            f"-> {flops / cold.median / 1e9:.1f} TFLOP/s")
 
     extras = {}
     if not args.no_extras:
@@ -160,14 +180,16 @@ def main():
     out = {
         "metric": "attention fwd TFLOP/s (B4 H32 S2048 D128 fp16, non-causal)",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(hot.wall_ms_per_call, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp16", "data": "synthetic",
         "config": {"workload": "configs[1]: flash-attention forward q,k,v [4,32,2048,128] fp16 N(0,1), scale 1/sqrt(128), non-causal",
-                   "kernel_config": str(cfg), "pct_of_fp16_mfma_peak": round(100 * value / PEAK_TFLOPS, 2)},
+                   "kernel_config": str(cfg), "pct_of_fp16_mfma_peak": round(100 * value / PEAK_TFLOPS, 2),
+                   "min_warmup_ms": MIN_WARMUP_MS},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": measured_traffic(cfg),
                      "kernel": "flashattn_fwd_" + ("regfuse" if cfg.fuse_type == "register" else "smemfuse"),
-                     "launch_ms": round(kern_ms, 5), "algorithmic_flops_per_launch": flops},
+                     "launch_ms": round(hot.mean, 5), "algorithmic_flops_per_launch": flops},
+        "timing": timing,
         "extras": extras,
     }
     if not args.no_cpu_baseline:
@@ -184,27 +206,28 @@ def side_measurements(aat, arch, Runtime, mk, steps, warmup):
     o = torch.empty_like(q)
     cfg = resolve_config(aat, arch, [q, k, v, o], True)
     rt = Runtime(arch, cfg)
-    _, ms = time_launches(lambda: rt.apply([q, k, v, o], causal=True), steps, warmup)
-    res["attn_causal_b4h32s2048d128"] = {"ms": round(ms, 5), "tflops": round(attn_flops(B, H, S, S, D, D, True) / ms / 1e9, 1), "config": str(cfg)}
-    log(f"attention fwd causal: {ms:.4f} ms -> {res['attn_causal_b4h32s2048d128']['tflops']} TFLOP/s")
+    t = time_launches(lambda: rt.apply([q, k, v, o], causal=True), steps, warmup)
+    res["attn_causal_b4h32s2048d128"] = extra(t, attn_flops(B, H, S, S, D, D, True), config=str(cfg))
+    log(f"attention fwd causal: {t.median:.4f} ms -> {res['attn_causal_b4h32s2048d128']['tflops']} TFLOP/s")
 
     q5, k5, v5 = mk(1, 32, 256, D), mk(1, 32, 16384, D), mk(1, 32, 16384, D)
     o5 = torch.empty_like(q5)
     cfg5 = resolve_config(aat, arch, [q5, k5, v5, o5], False)
     rt5 = Runtime(arch, cfg5)
-    _, ms = time_launches(lambda: rt5.apply([q5, k5, v5, o5]), steps, warmup)
+    t = time_launches(lambda: rt5.apply([q5, k5, v5, o5]), steps, warmup)
     bytes5 = 2 * (q5.numel() + k5.numel() + v5.numel() + o5.numel())
-    res["attn_longkv_b1h32q256k16384d128"] = {"ms": round(ms, 5), "tflops": round(attn_flops(1, 32, 256, 16384, D, D) / ms / 1e9, 1),
-                                              "gbps": round(bytes5 / ms / 1e6, 1), "config": str(cfg5)}
-    log(f"attention fwd long-kv: {ms:.4f} ms -> {res['attn_longkv_b1h32q256k16384d128']}")
+    e5 = extra(t, attn_flops(1, 32, 256, 16384, D, D), config=str(cfg5), gbps=round(bytes5 / t.median / 1e6, 1))
+    e5["roofline"] = {"bound": "hbm", "achieved": round(bytes5 / t.median / 1e6, 1), "peak": 8000.0, "unit": "GB/s",
+                      "frac": round(bytes5 / t.median / 1e6 / 8000.0, 4), "algorithmic_bytes": bytes5}
+    res["attn_longkv_b1h32q256k16384d128"] = e5
+    log(f"attention fwd long-kv: {t.median:.4f} ms -> {e5['tflops']} TFLOP/s, {e5['gbps']} GB/s")
     # shorter rows with the headline configuration: the wrapper takes its persistent-block kernel there
     qs, ks, vs = mk(16, H, 512, D), mk(16, H, 512, D), mk(16, H, 512, D)
     os_ = torch.empty_like(qs)
     rts = Runtime(arch, resolve_config(aat, arch, [q, k, v, o], False))
-    _, ms = time_launches(lambda: rts.apply([qs, ks, vs, os_]), steps, warmup)
-    res["attn_short_rows_b16h32s512d128"] = {"ms": round(ms, 5), "tflops": round(attn_flops(16, H, 512, 512, D, D) / ms / 1e9, 1),
-                                             "config": str(rts.config)}
-    log(f"attention fwd S=512 B=16: {ms:.4f} ms -> {res['attn_short_rows_b16h32s512d128']['tflops']} TFLOP/s")
+    t = time_launches(lambda: rts.apply([qs, ks, vs, os_]), steps, warmup)
+    res["attn_short_rows_b16h32s512d128"] = extra(t, attn_flops(16, H, 512, 512, D, D), config=str(rts.config))
+    log(f"attention fwd S=512 B=16: {t.median:.4f} ms -> {res['attn_short_rows_b16h32s512d128']['tflops']} TFLOP/s")
     res.update(attention_backward_measurement(aat, arch, mk, steps, warmup))
     res.update(retnet_measurements(aat, arch, mk, steps, warmup))
     res.update(retnet_recurrent_measurement(aat, steps, warmup))
@@ -225,12 +248,12 @@ def retnet_recurrent_measurement(aat, steps, warmup):
     decay = (1.0 - 2.0 ** (-5.0 - torch.arange(h, dtype=torch.float32, device="cuda"))).unsqueeze(1).expand(h, seqlen).contiguous()
     out = torch.empty_like(v)
     ws = torch.empty(h * (seqlen // 32) * 5120, dtype=torch.uint8, device="cuda")
-    _, ms = time_launches(lambda: aat.retnet_recurrent_fwd(q, k, v, decay, out=out, workspace=ws), steps, warmup)
+    t = time_launches(lambda: aat.retnet_recurrent_fwd(q, k, v, decay, out=out, workspace=ws), steps, warmup)
     flops = 5.0 * b * h * seqlen * kd * vd
     nbytes = 4.0 * (q.numel() + k.numel() + v.numel() + out.numel())
-    res = {"ms": round(ms, 5), "tflops": round(flops / ms / 1e9, 1), "frac_of_fp32_mfma_peak": round(flops / ms / 1e9 / 157.3, 3),
-           "gbps": round(nbytes / ms / 1e6, 1)}
-    log(f"retnet recurrent fwd: {ms:.4f} ms -> {res}")
+    res = extra(t, flops, peak=157.3, gbps=round(nbytes / t.median / 1e6, 1))
+    res["frac_of_fp32_mfma_peak"] = res["roofline"]["frac"]
+    log(f"retnet recurrent fwd: {t.median:.4f} ms -> {res['tflops']} TFLOP/s ({res['gbps']} GB/s)")
     return {"retnet_recurrent_b8h32s2048_dqk128_dv128_f32": res}
 
 
@@ -240,13 +263,22 @@ def attention_backward_measurement(aat, arch, mk, steps, warmup):
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
     fwd, bwd = attn_flops(B, H, S, S, D, D), 2.0 * B * H * S * S * (3 * D + 2 * D)
 
-    def fb():
+    def reset():
         q.grad = k.grad = v.grad = None
-        aat.flash_attn_func(q, k, v, arch).backward(do)
 
-    _, ms = time_launches(fb, steps, warmup)
-    log(f"attention fwd+bwd: {ms:.4f} ms -> {(fwd + bwd) / ms / 1e9:.1f} TFLOP/s")
-    return {"attn_fwd_bwd_b4h32s2048d128": {"ms": round(ms, 5), "tflops": round((fwd + bwd) / ms / 1e9, 1)}}
+    t = time_launches(lambda: aat.flash_attn_func(q, k, v, arch).backward(do), steps, warmup, before_each=reset)
+    log(f"attention fwd+bwd: {t.median:.4f} ms -> {(fwd + bwd) / t.median / 1e9:.1f} TFLOP/s")
+    # the column and the row kernel both evaluate S and dP: 7 contractions issued for the 5 counted, plus the forward's 2
+    return {"attn_fwd_bwd_b4h32s2048d128": extra(t, fwd + bwd, issued_ratio=round((2 + 7) / (2 + 5), 3))}
+
+
+def retnet_decay_mask(heads, seq_q, seq_k, device):
+    """D[h, n, m] = gamma_h^(n - m) for n >= m, else 0, gamma_h = 1 - 2^(-5-h); fp32 closed form rounded to fp16."""
+    import torch
+    gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(heads, dtype=torch.float32, device=device))
+    dist = (torch.arange(seq_q, device=device).unsqueeze(1) - torch.arange(seq_k, device=device).unsqueeze(0)).float()
+    mask = torch.pow(gamma.view(-1, 1, 1), dist.clamp(min=0).unsqueeze(0)) * (dist >= 0).unsqueeze(0)
+    return mask.half()
 
 
 def retnet_measurements(aat, arch, mk, steps, warmup):
@@ -255,36 +287,34 @@ def retnet_measurements(aat, arch, mk, steps, warmup):
     res = {}
     if not hasattr(gfx950_space, "default_backward_config"):
         return res
-    from oracle import ref_op
     b, h, s, dqk, dv = 4, 8, 2048, 256, 512
     q, k, v, do = mk(b, h, s, dqk), mk(b, h, s, dqk), mk(b, h, s, dv), mk(b, h, s, dv)
-    mask = ref_op.retnet_decay_mask(h, s, s).cuda()
+    mask = retnet_decay_mask(h, s, s, "cuda")
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
     fwd_flops = 2.0 * b * h * s * s * (dqk + dv)
     bwd_flops = 2.0 * b * h * s * s * (3 * dqk + 2 * dv)
     with torch.no_grad():
-        _, ms_f = time_launches(lambda: aat.RetNetAttnFunc(q, k, v, mask, arch), steps, warmup)
-    res["retnet_fwd_b4h8s2048_dqk256_dv512"] = {"ms": round(ms_f, 5), "tflops": round(fwd_flops / ms_f / 1e9, 1)}
-    log(f"retnet fwd: {ms_f:.4f} ms -> {fwd_flops / ms_f / 1e9:.1f} TFLOP/s")
+        t = time_launches(lambda: aat.RetNetAttnFunc(q, k, v, mask, arch), steps, warmup)
+    res["retnet_fwd_b4h8s2048_dqk256_dv512"] = extra(t, fwd_flops)
+    log(f"retnet fwd: {t.median:.4f} ms -> {fwd_flops / t.median / 1e9:.1f} TFLOP/s")
 
-    def fb():
+    def reset():
         q.grad = k.grad = v.grad = None
-        aat.RetNetAttnFunc(q, k, v, mask, arch).backward(do)
 
-    _, ms_fb = time_launches(fb, steps, warmup)
-    res["retnet_fwd_bwd_b4h8s2048_dqk256_dv512"] = {"ms": round(ms_fb, 5), "tflops": round((fwd_flops + bwd_flops) / ms_fb / 1e9, 1)}
-    log(f"retnet fwd+bwd: {ms_fb:.4f} ms -> {(fwd_flops + bwd_flops) / ms_fb / 1e9:.1f} TFLOP/s (dense-mask FLOPs)")
+    # the three backward passes evaluate dO V^T twice: 3 (d_qk + d_v) issued for the 3 d_qk + 2 d_v counted
+    issued = round(((dqk + dv) + 3 * (dqk + dv)) / ((dqk + dv) + 3 * dqk + 2 * dv), 3)
+    t = time_launches(lambda: aat.RetNetAttnFunc(q, k, v, mask, arch).backward(do), steps, warmup, before_each=reset)
+    res["retnet_fwd_bwd_b4h8s2048_dqk256_dv512"] = extra(t, fwd_flops + bwd_flops, issued_ratio=issued)
+    log(f"retnet fwd+bwd: {t.median:.4f} ms -> {(fwd_flops + bwd_flops) / t.median / 1e9:.1f} TFLOP/s (dense-mask FLOPs)")
 
     if hasattr(aat, "RetNetDecayAttnFunc"):              # the same decay mask, built in registers from one rate per head
         gamma = 1.0 - torch.pow(2.0, -5.0 - torch.arange(h, dtype=torch.float64))
-
-        def fb_decay():
-            q.grad = k.grad = v.grad = None
-            aat.RetNetDecayAttnFunc(q, k, v, gamma, arch).backward(do)
-
-        _, ms_d = time_launches(fb_decay, steps, warmup)
-        res["retnet_decay_fwd_bwd_b4h8s2048_dqk256_dv512"] = {"ms": round(ms_d, 5), "tflops": round((fwd_flops + bwd_flops) / ms_d / 1e9, 1)}
-        log(f"retnet decay fwd+bwd: {ms_d:.4f} ms -> {(fwd_flops + bwd_flops) / ms_d / 1e9:.1f} TFLOP/s (dense-mask FLOPs)")
+        t = time_launches(lambda: aat.RetNetDecayAttnFunc(q, k, v, gamma, arch).backward(do), steps, warmup, before_each=reset)
+        # tiles above the diagonal are skipped: about half of the dense count is issued
+        # tiles above the diagonal are skipped: the roofline fraction is taken on half the dense count
+        res["retnet_decay_fwd_bwd_b4h8s2048_dqk256_dv512"] = extra(t, (fwd_flops + bwd_flops) / 2, flops_counted="causal half of the dense-mask count",
+                                                                   tflops_dense_count=round((fwd_flops + bwd_flops) / t.median / 1e9, 1))
+        log(f"retnet decay fwd+bwd: {t.median:.4f} ms -> {(fwd_flops + bwd_flops) / t.median / 1e9:.1f} TFLOP/s (dense-mask FLOPs)")
     return res
 
 
