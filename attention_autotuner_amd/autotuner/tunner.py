@@ -1,18 +1,26 @@
 """Per-operator tuners (reference python/autotuner/tunner.py:13-225).
 
-Each tuner picks its search space from the architecture's platform: "ROCm" uses the gfx950 space,
-"CUDA" uses the restated reference space (enumeration only -- those configurations cannot be built
-here and ``tune`` refuses to try).
+Each tuner enumerates the gfx950 space for a ROCm descriptor.  A descriptor of another platform may bring
+its own space along (``arch.search_space``: a module with ``forward_candidates`` / ``forward_valid`` /
+``backward_candidates`` / ``backward_valid``); such configurations can be enumerated, which is how the
+test suite replays the reference's published NVIDIA tuning logs, but not built: ``tune`` refuses.
 """
 import ctypes
 import math
 
-from . import gfx950_space, legacy_space
+from . import gfx950_space
 from .base_tunner import BaseTunner
 
 
 def _is_rocm(arch):
     return getattr(arch, "platform", "") == "ROCm"
+
+
+def _foreign_space(arch):
+    space = getattr(arch, "search_space", None)
+    if space is None:
+        raise RuntimeError(f"{arch.name}: no search space for platform {getattr(arch, 'platform', '?')!r}")
+    return space
 
 
 class _ForwardTunner(BaseTunner):
@@ -24,7 +32,7 @@ class _ForwardTunner(BaseTunner):
 
     def generate_configs(self, Br, Bc, dim_qk, dim_v):
         if not _is_rocm(self.arch):
-            return legacy_space.forward_candidates(self.operation, Br, Bc, dim_qk, dim_v)
+            return _foreign_space(self.arch).forward_candidates(self.operation, Br, Bc, dim_qk, dim_v)
         return gfx950_space.forward_candidates(self.operation, Br, Bc, dim_qk, dim_v, with_splits=self._wants_splits(Br))
 
     def _wants_splits(self, Br):
@@ -34,7 +42,7 @@ class _ForwardTunner(BaseTunner):
         return self.operation == "attn" and not self.causal and blocks < 2 * self.arch.compute_max_core
 
     def _validate(self, config):
-        space = gfx950_space if _is_rocm(self.arch) else legacy_space
+        space = gfx950_space if _is_rocm(self.arch) else _foreign_space(self.arch)
         return space.forward_valid(config, self.arch)
 
     validate_register_fuse = _validate
@@ -78,12 +86,12 @@ class RetBwdTunner(BaseTunner):
     def generate_configs(self, Br, Bc, dim_qk, dim_v):
         if _is_rocm(self.arch):
             return gfx950_space.backward_candidates(Br, Bc, dim_qk, dim_v)
-        return legacy_space.backward_candidates(Br, Bc, dim_qk, dim_v)
+        return _foreign_space(self.arch).backward_candidates(Br, Bc, dim_qk, dim_v)
 
     def validate_kernel(self, config):
         if _is_rocm(self.arch):
             return gfx950_space.backward_valid(config, self.arch)
-        return legacy_space.backward_valid(config, self.arch)
+        return _foreign_space(self.arch).backward_valid(config, self.arch)
 
     def tune(self, *a, **kw):
         if not _is_rocm(self.arch):

@@ -136,9 +136,6 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   using TP = typename T::template Persist<WPE>;
   static_assert(!PERSIST || (!PIPE && !CAUSAL && !SPLIT && TP::kOk), "persistent blocks: plain schedule, 2+2 buffers, room to stage the output");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-#ifdef AAT_CLOCK_PROBE
-  const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
-#endif
   char* const kbuf = smem;
   char* const vbuf = smem + NSK * T::kKBytes;
 
@@ -425,12 +422,6 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     if (!has_next) break;
     prefetched = true;
   }
-#ifdef AAT_CLOCK_PROBE
-  if (lse != nullptr && tid == 0 && (blockIdx.x % 64) == 0) {
-    lse[2 * (blockIdx.x / 64)] = (float)(clock64() - probe_c0);
-    lse[2 * (blockIdx.x / 64) + 1] = (float)(wall_clock64() - probe_w0);
-  }
-#endif
 }
 
 // Combine the parts of a kv split: O = sum_s exp(lse_s - lse) O_s with lse = log sum_s exp(lse_s).

@@ -106,20 +106,24 @@ template <int NT> AAT_DEV void exp_range(f16v (&s)[NT], int e0, int count, float
 }
 
 // Round 16 kv rows (group g: score tile g/2, registers 8*(g%2) .. +7) of P to one fp16 MFMA operand and
-// add their sum to `sum`.  The sum is taken over the ROUNDED values (v_dot2_f32_f16 against ones, fp32
-// accumulate), i.e. over exactly the weights the second contraction applies, at half the instruction
-// count of fp32 adds.
+// add their sum to `sum`.  The sum is taken in fp32 over the unrounded values with plain adds (two
+// interleaved chains).  v_dot2_f32_f16 against a vector of ones would halve the instruction count, but on
+// gfx950 the dot instructions share the matrix pipe's issue path: next to a wave that streams MFMAs each
+// v_dot2c_f32_f16 of the other wave of the SIMD was measured at ~90 cycles instead of 4.5 (8 of them turned
+// a 450-cycle stretch of exponentials and conversions into 1150 cycles), and a wave's own MFMAs wait for them too.
 template <int NT> AAT_DEV void pack_p_group(h8 (&pf)[NT][2], const f16v (&s)[NT], int g, float& sum) {
-  const h2 ones = {(half_t)1.f, (half_t)1.f};
   const int t = g >> 1, half = g & 1;
   h8 r;
+  float s0 = s[t][8 * half] + s[t][8 * half + 1], s1 = s[t][8 * half + 2] + s[t][8 * half + 3];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const h2 pr = pack_rne(s[t][8 * half + 2 * i], s[t][8 * half + 2 * i + 1]);
     r[2 * i] = pr[0];
     r[2 * i + 1] = pr[1];
-    sum = __builtin_amdgcn_fdot2(pr, ones, sum, false);
   }
+  s0 += s[t][8 * half + 4] + s[t][8 * half + 5];
+  s1 += s[t][8 * half + 6] + s[t][8 * half + 7];
+  sum += s0 + s1;
   pf[t][half] = r;
 }
 

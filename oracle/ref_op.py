@@ -16,7 +16,9 @@ reference uses as its own correctness check:
   ``r = clamp(sum|S|, min=1)`` detached, ``o = (S / r) v``) and also returns ``r``.
 * ``retnet_bwd_ref``  is the closed form the backward kernel evaluates, reference
   csrc/kernels/retnet/bwd/bwd_colblock.h:522-576: with r constant, ``P = S / r``,
-  ``dV = P^T dO``, ``dS = (dO V^T / r) * mask``, ``dK = dS^T Q``, ``dQ = dS K``.
+  ``dV = P^T dO``, ``dS = (dO V^T / r) * mask``, ``dK = dS^T Q``, ``dQ = dS K``; with
+  ``operand_dtype=torch.float16`` P and dS are rounded where the reference kernel rounds them (:509, :551);
+  ``retnet_bwd_rounding_bound`` is the worst case that rounding can move each gradient entry by.
 * ``retnet_decay_mask`` is the decay matrix of the benchmark configuration:
   ``D[h, n, m] = gamma_h^(n-m)`` for n >= m else 0, ``gamma_h = 1 - 2^(-5-h)``.
 * ``retnet_recurrent_ref`` is the closed form of the recurrent scan of reference
@@ -92,19 +94,40 @@ def retnet_ref(q, k, v, mask, return_r=False):
     return (o, r.squeeze(-1)) if return_r else o
 
 
-def retnet_bwd_ref(q, k, v, mask, do, r=None):
-    """Gradients of ``retnet_ref`` w.r.t. q, k, v with r treated as a constant."""
+def retnet_bwd_ref(q, k, v, mask, do, r=None, operand_dtype=None):
+    """Gradients of ``retnet_ref`` w.r.t. q, k, v with r treated as a constant.
+
+    ``operand_dtype=torch.float16`` restates the reference kernel's arithmetic instead of the exact closed
+    form: P and dS are rounded to fp16 before the contraction that consumes them (reference
+    csrc/kernels/retnet/bwd/bwd_colblock.h:509 and :551), everything else stays fp32.  The two differ by at
+    most 2^-11 * sum_j |term_j| per gradient entry (tests/test_oracle.py pins that bound)."""
     q, k, v, mask, do = _f32(q), _f32(k), _f32(v), _f32(mask), _f32(do)
     s = (q @ k.transpose(-1, -2)) * mask
     if r is None:
         r = s.abs().sum(dim=-1).clamp(min=1.0)
     r = _f32(r).unsqueeze(-1)
     p = s / r
-    dv = p.transpose(-1, -2) @ do
     ds = ((do @ v.transpose(-1, -2)) / r) * mask
+    if operand_dtype is not None:
+        p, ds = p.to(operand_dtype).float(), ds.to(operand_dtype).float()
+    dv = p.transpose(-1, -2) @ do
     dk = ds.transpose(-1, -2) @ q
     dq = ds @ k
     return dq, dk, dv
+
+
+def retnet_bwd_rounding_bound(q, k, v, mask, do, r=None):
+    """Per-entry bound on |rounded-operand form - exact form| of ``retnet_bwd_ref``: rounding P or dS to fp16
+    moves each entry by at most 2^-11 of its magnitude, so a gradient entry moves by at most
+    2^-11 * sum_j |operand_j| |other factor_j|.  Returns that sum (without the 2^-11) for dq, dk, dv."""
+    q, k, v, mask, do = _f32(q), _f32(k), _f32(v), _f32(mask), _f32(do)
+    s = (q @ k.transpose(-1, -2)) * mask
+    if r is None:
+        r = s.abs().sum(dim=-1).clamp(min=1.0)
+    r = _f32(r).unsqueeze(-1)
+    p = (s / r).abs()
+    ds = (((do @ v.transpose(-1, -2)) / r) * mask).abs()
+    return ds @ k.abs(), ds.transpose(-1, -2) @ q.abs(), p.transpose(-1, -2) @ do.abs()
 
 
 def retnet_decay_mask(nheads, seq_q, seq_k, dtype=torch.float16):

@@ -1,0 +1,57 @@
+"""Tile / wave / buffer variants the GPU parity suite runs to show that every configuration computes the
+same thing.  ``parity_configs()`` lists them so the build step can compile them ahead of time (nothing is
+compiled inside a GPU test)."""
+from attention_autotuner_amd.arch import MI355X
+from attention_autotuner_amd.autotuner import gfx950_space
+from attention_autotuner_amd.autotuner.configs import AttnBwdConfig, AttnConfig, RetConfig
+
+# attention forward, register-fused: (Br, Bc, Nthreads, K buffers, V buffers, waves per SIMD) for every head-size pair below
+PARITY_TILES = [
+    (128, 64, 256, 2, 2, 2), (128, 64, 256, 1, 1, 2), (128, 64, 256, 2, 1, 1), (128, 64, 256, 1, 2, 1),
+    (128, 32, 256, 2, 2, 2), (128, 128, 256, 1, 1, 1), (64, 64, 128, 2, 2, 2), (128, 64, 128, 1, 1, 1),
+    (256, 64, 512, 2, 2, 2), (128, 32, 256, 2, 2, 3), (128, 64, 256, 1, 1, 3),
+]
+PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
+# attention forward, LDS-fused: (Br, Bc, Nthreads, K bufs, V bufs, W1N, W2N, waves/SIMD)
+SHARED_TILES = [(128, 64, 256, 2, 2, 1, 4, 2), (64, 64, 256, 1, 1, 2, 4, 2), (64, 64, 256, 2, 1, 2, 2, 2), (64, 64, 256, 1, 1, 2, 4, 1)]
+SHARED_DIMS = [(64, 64), (128, 128), (256, 512)]
+# attention backward: head-size pairs run at their defaults, and (Br, Bc, Nthreads, buffers) variants at 128/128
+ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (256, 128), (256, 256)]
+ATTN_BWD_TILES = [(64, 32, 128, 2), (64, 64, 128, 2), (128, 64, 256, 3), (128, 32, 256, 2)]
+# kv-splitting variants: (d_qk, d_v, splits)
+SPLIT_VARIANTS = [(128, 128, 4), (128, 128, 8), (64, 64, 2)]
+
+
+def parity_configs(arch=None):
+    arch = arch or MI355X()
+    out = []
+    # RetNet forward variants at 128/128 (register and both wave grids of the LDS-fused kernel)
+    for fuse, extra in (("register", {}), ("shared", dict(warps_mma1_n=1, warps_mma_n=4)), ("shared", dict(warps_mma1_n=2, warps_mma_n=2))):
+        for st in ((1, 1), (2, 2)):
+            cfg = RetConfig(128 if fuse == "register" else 64, 64, 128, 128, 128, 64, st[0], st[0], st[1], 256, True, waves_per_eu=1, **extra)
+            cfg.fuse_type = fuse
+            if gfx950_space.forward_valid(cfg, arch):
+                out.append(cfg)
+    for br, bc, nt, st in ATTN_BWD_TILES:
+        for row_wpe in (1, 2):
+            cfg = AttnBwdConfig(br, bc, 128, 128, nt, st, row_waves_per_eu=row_wpe)
+            if gfx950_space.attn_backward_valid(cfg, arch):
+                out.append(cfg)
+    for dqk, dv in PARITY_DIMS:
+        for br, bc, nt, sq, sv, wpe in PARITY_TILES:
+            cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+            if gfx950_space.forward_valid(cfg, arch):
+                out.append(cfg)
+            if (sq, sv) == (2, 2):
+                piped = AttnConfig(br, bc, dqk, dv, dqk, bc, 2, 2, nt, True, waves_per_eu=wpe, sw_pipeline=1).set_fuse_type("register")
+                if gfx950_space.forward_valid(piped, arch):
+                    out.append(piped)
+    for dqk, dv, ns in SPLIT_VARIANTS:
+        out.append(AttnConfig(128, 64, dqk, dv, dqk, 64, 2, 2, 256, True, waves_per_eu=2, kv_splits=ns).set_fuse_type("register"))
+    for dqk, dv in SHARED_DIMS:
+        for br, bc, nt, sq, sv, w1n, w2n, wpe in SHARED_TILES:
+            cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, w1n, w2n, waves_per_eu=wpe)
+            cfg.fuse_type = "shared"
+            if gfx950_space.forward_valid(cfg, arch):
+                out.append(cfg)
+    return out

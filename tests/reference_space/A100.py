@@ -1,6 +1,8 @@
 """NVIDIA A100 limits.  Kept only so the search-space enumeration can be checked against the
 reference's published tuning logs; nothing is compiled or run for this descriptor."""
-from .arch_base import Arch
+from attention_autotuner_amd.arch import Arch
+
+from . import legacy_space
 
 
 class A100(Arch):
@@ -16,6 +18,7 @@ class A100(Arch):
     compute_capability = "80"
     register_per_thread = 255
     cutlass_mma = (16, 8, 16)
+    search_space = legacy_space        # the tuners enumerate a non-ROCm descriptor with the space it brings along
 
     def __init__(self):
         super().__init__()

@@ -1,5 +1,7 @@
 """NVIDIA RTX 4090 limits (enumeration checks only, see A100.py)."""
-from .arch_base import Arch
+from attention_autotuner_amd.arch import Arch
+
+from . import legacy_space
 
 
 class RTX4090(Arch):
@@ -15,6 +17,7 @@ class RTX4090(Arch):
     compute_capability = "89"
     register_per_thread = 255
     cutlass_mma = (16, 8, 16)
+    search_space = legacy_space        # the tuners enumerate a non-ROCm descriptor with the space it brings along
 
     def __init__(self):
         super().__init__()

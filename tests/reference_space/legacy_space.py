@@ -8,7 +8,7 @@ module reproduces them line by line.
 Rules restated from reference python/autotuner/tunner.py:13-225 (``generate_configs``,
 ``validate_register_fuse``, ``validate_shared_fuse``, ``validate_kernel``).
 """
-from .configs import AttnConfig, RetConfig, RetBwdConfig, balanced_wave_split
+from attention_autotuner_amd.autotuner.configs import AttnConfig, RetConfig, RetBwdConfig, balanced_wave_split
 
 _THREADS = (128, 256)
 

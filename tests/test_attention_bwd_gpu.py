@@ -1,8 +1,8 @@
 """GPU parity of the attention backward (dq, dk, dv) against the CPU oracle, through the operator and
 through the C ABI.
 
-Tolerance: |err| <= 2e-3 + 1e-3 * |ref| on fp16 gradients versus the fp32 oracle on the same seeded
-inputs (a gradient entry above 4 in magnitude has half an fp16 ulp of 2e-3 already); the forward's
+Tolerance (oracle/tolerance.py): max |err| <= 2e-3 on fp16 gradients versus the fp32 oracle on the same
+seeded inputs wherever |ref| < 4, one fp16 unit in the last place of the reference above; the forward's
 log-sum-exp is compared at 1e-3 absolute.
 """
 import ctypes
@@ -15,7 +15,8 @@ import attention_autotuner_amd as aat
 from attention_autotuner_amd.arch import MI355X
 from attention_autotuner_amd.autotuner import Runtime, codegen, gfx950_space, library, prebuilt
 from attention_autotuner_amd.autotuner.configs import AttnBwdConfig
-from oracle import ref_op
+import parity_matrix
+from oracle import ref_op, tolerance
 
 pytestmark = pytest.mark.gpu
 ARCH = MI355X()
@@ -31,8 +32,9 @@ def _inputs(b, h, sq, sk, dqk, dv, seed=0):
 
 
 def _close(got, ref):
-    err = (got.float().cpu() - ref).abs()
-    return bool((err <= 2e-3 + 1e-3 * ref.abs()).all()), err.max().item()
+    ok, worst_small, worst_large, n_large = tolerance.check(got, ref)
+    print(f"  max |err| {worst_small:.3e} (|ref| < 4), {worst_large:.2f} ulp over {n_large} entries with |ref| >= 4")
+    return ok, (worst_small, worst_large)
 
 
 def _op_grads(q, k, v, do, causal, scale=None):
@@ -43,7 +45,7 @@ def _op_grads(q, k, v, do, causal, scale=None):
 
 
 @pytest.mark.parametrize("causal", [False, True])
-@pytest.mark.parametrize("dqk,dv", prebuilt.ATTN_BWD_DIMS)
+@pytest.mark.parametrize("dqk,dv", parity_matrix.ATTN_BWD_DIMS)
 @pytest.mark.parametrize("sq,sk", [(256, 256), (128, 384), (384, 128)])
 def test_operator_backward_matches_oracle(dqk, dv, sq, sk, causal):
     q, k, v, do = _inputs(2, 3, sq, sk, dqk, dv, seed=sq + dqk)
@@ -87,7 +89,7 @@ def test_config2_backward_b4_h32_s2048_d128(causal):
 
 
 @pytest.mark.parametrize("row_wpe", [1, 2])
-@pytest.mark.parametrize("br,bc,nt,st", prebuilt.ATTN_BWD_TILES)
+@pytest.mark.parametrize("br,bc,nt,st", parity_matrix.ATTN_BWD_TILES)
 def test_tile_variants_agree(br, bc, nt, st, row_wpe):
     """Tile shapes of the parity set, the row kernel compiled for one and for two waves per SIMD."""
     q, k, v, do = _inputs(1, 2, 256, 256, 128, 128, seed=5)

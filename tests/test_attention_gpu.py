@@ -90,7 +90,7 @@ def test_scaled_inputs_like_the_reference_tuner_demo():
     assert _err(o, ref_op.attention_ref(q, k, v)) <= 3 * TOL      # |v| is 3x larger
 
 
-from attention_autotuner_amd.autotuner.prebuilt import PARITY_DIMS, PARITY_TILES as CONFIGS
+from parity_matrix import PARITY_DIMS, PARITY_TILES as CONFIGS
 
 
 @pytest.mark.parametrize("dqk,dv", PARITY_DIMS)
@@ -158,7 +158,7 @@ def test_persistent_blocks_agree_with_the_oracle(dqk, dv):
 
 @pytest.mark.parametrize("dqk,dv", [(64, 64), (128, 128), (256, 512)])
 def test_lds_fused_variants_agree_with_the_oracle(dqk, dv):
-    from attention_autotuner_amd.autotuner.prebuilt import SHARED_TILES
+    from parity_matrix import SHARED_TILES
     q, k, v = _inputs(1, 2, 128, 256, dqk, dv, seed=8)
     refs = {c: ref_op.attention_ref(q, k, v, None, c) for c in (False, True)}
     qc, kc, vc = q.cuda(), k.cuda(), v.cuda()

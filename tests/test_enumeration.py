@@ -5,7 +5,8 @@ import re
 import pytest
 import torch
 
-from attention_autotuner_amd.arch import A100, RTX4090, MI355X
+from attention_autotuner_amd.arch import MI355X
+from reference_space import A100, RTX4090
 from attention_autotuner_amd.autotuner import AttnTunner, RetTunner, RetBwdTunner, AttnConfig, RetConfig, RetBwdConfig, gfx950_space
 from attention_autotuner_amd.autotuner.configs import balanced_wave_split, supported_configs
 

@@ -192,6 +192,55 @@ def test_retnet_bwd_linearity_and_zero_mask():
         assert g.abs().max() == 0
 
 
+def test_retnet_bwd_rounded_operands_stay_within_the_rounding_bound():
+    """The variant that rounds P and dS to fp16 where the reference kernel does differs from the exact closed
+    form by at most half an fp16 ulp per rounded entry: |delta| <= 2^-11 * sum_j |operand_j| |other_j|, and it is
+    the exact form again once P and dS are representable (a one-hot mask row with power-of-two data)."""
+    q, k, v = _rand(1, 2, 16, 64, seed=43), _rand(1, 2, 16, 64, seed=44), _rand(1, 2, 16, 128, seed=45)
+    mask, do = ref_op.retnet_decay_mask(2, 16, 16), _rand(1, 2, 16, 128, seed=46)
+    exact = ref_op.retnet_bwd_ref(q, k, v, mask, do)
+    rounded = ref_op.retnet_bwd_ref(q, k, v, mask, do, operand_dtype=torch.float16)
+    bounds = ref_op.retnet_bwd_rounding_bound(q, k, v, mask, do)
+    differs = False
+    for e, g, b in zip(exact, rounded, bounds):
+        assert ((e - g).abs() <= 2.0 ** -11 * b * 1.001 + 1e-7).all()
+        differs |= bool((e != g).any())
+    assert differs                                      # the rounding is really applied
+    eye = torch.eye(16).expand(2, 16, 16)                # P = +-1 and dS = (dO v) / |q k| on the diagonal only
+    q2 = torch.zeros(1, 2, 16, 64); q2[..., 0] = 2.0
+    k2 = torch.zeros(1, 2, 16, 64); k2[..., 0] = 4.0    # S_ii = 8, r = 8
+    v2 = torch.zeros(1, 2, 16, 128); v2[..., 1] = 0.5
+    d2 = torch.zeros(1, 2, 16, 128); d2[..., 1] = 16.0  # dO v = 8 -> dS = 1
+    for e, g in zip(ref_op.retnet_bwd_ref(q2, k2, v2, eye, d2),
+                    ref_op.retnet_bwd_ref(q2, k2, v2, eye, d2, operand_dtype=torch.float16)):
+        assert torch.equal(e, g)
+    dq, dk, dv = ref_op.retnet_bwd_ref(q2, k2, v2, eye, d2, operand_dtype=torch.float16)
+    assert dq[0, 0, 3, 0] == 4.0 and dk[0, 0, 3, 0] == 2.0 and dv[0, 0, 3, 1] == 16.0
+
+
+# ------------------------------------------------------------------------------------ the parity bound
+def test_tolerance_rule_accepts_and_rejects_what_it_says():
+    from oracle import tolerance
+    ref = torch.tensor([0.5, 1.5, 3.0, 5.0, 100.0])
+    assert torch.equal(tolerance.fp16_ulp(ref), torch.tensor([2.0 ** -11, 2.0 ** -10, 2.0 ** -9, 2.0 ** -8, 2.0 ** -4]))
+    ok, small, large, n = tolerance.check(ref + torch.tensor([1.9e-3, -1.9e-3, 1.9e-3, 3.9e-3, -0.06]), ref)
+    assert ok and n == 2 and abs(small - 1.9e-3) < 1e-6 and 0.9 < large <= 1.0
+    assert not tolerance.check(ref + torch.tensor([0.0, 0.0, 2.1e-3, 0.0, 0.0]), ref)[0]          # 2e-3 is literal below 4
+    assert not tolerance.check(ref + torch.tensor([0.0, 0.0, 0.0, 4.0e-3, 0.0]), ref)[0]          # one ulp at 5 is 3.9e-3
+    assert not tolerance.check(ref + torch.tensor([0.0, 0.0, 0.0, 0.0, 0.07]), ref)[0]
+    assert not tolerance.check(torch.tensor([float("nan")]), torch.tensor([0.0]))[0]
+    # the rounded-operand rule: half an ulp of the result plus 2^-11 of the given sum of term magnitudes
+    terms = torch.tensor([1.0, 2.0, 4.0, 8.0, 100.0])
+    edge = 0.5 * tolerance.fp16_ulp(ref) + 2.0 ** -11 * terms
+    assert tolerance.check_rounded_operand(ref + edge, ref, terms)[0]
+    for i in range(5):
+        bad = ref.clone()
+        bad[i] -= 1.1 * edge[i] + 1e-4
+        assert not tolerance.check_rounded_operand(bad, ref, terms)[0]
+    with pytest.raises(AssertionError):
+        tolerance.assert_close(ref + 0.01, ref, "rejects")
+
+
 # ---------------------------------------------------------------------------------- attention backward
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("sq,sk", [(8, 8), (6, 10)])

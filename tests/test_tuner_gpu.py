@@ -5,6 +5,8 @@ import json
 import os
 
 import pytest
+
+import parity_matrix
 import torch
 
 from attention_autotuner_amd.arch import MI355X
@@ -18,7 +20,7 @@ ARCH = MI355X()
 
 def _prebuilt_attention_candidates(dqk, dv):
     out = []
-    for br, bc, nt, sq, sv, wpe in prebuilt.PARITY_TILES[:4]:
+    for br, bc, nt, sq, sv, wpe in parity_matrix.PARITY_TILES[:4]:
         cfg = AttnConfig(br, bc, dqk, dv, dqk, bc, sq, sv, nt, True, waves_per_eu=wpe).set_fuse_type("register")
         if gfx950_space.forward_valid(cfg, ARCH) and os.path.exists(codegen.library_path(cfg)):
             out.append(cfg)
