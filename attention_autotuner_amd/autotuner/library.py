@@ -70,6 +70,8 @@ def _bind_recurrent(lib):
     lib.retnet_recurrent_fwd_ex.argtypes = [_VP] * 5 + dims + [_VP, _SZ, _VP]
     lib.retnet_recurrent_profile.restype = _F
     lib.retnet_recurrent_profile.argtypes = [_VP] * 5 + dims + [_VP, _SZ, _VP]
+    lib.retnet_recurrent_fwd_noalloc.restype = _I
+    lib.retnet_recurrent_fwd_noalloc.argtypes = [_VP] * 5 + dims + [_VP]
     return lib
 
 

@@ -109,6 +109,36 @@ char* cached_workspace(size_t bytes) {{
   }}
   return w.ptr;
 }}
+
+// The entry point that allocates nothing keeps its decay factors in device memory that is part of this
+// library's code object: one copy of `scratch` per device that loads the library, held until the process ends.
+constexpr size_t kNoAllocScratchBytes = (size_t)AAT_RECURRENT_NOALLOC_MAX_RECORDS * aat::kRecFactorBytes;
+}}  // namespace
+
+static __device__ __align__(256) char scratch[kNoAllocScratchBytes];
+
+namespace {{
+// In host code `scratch` is only a handle for hipGetSymbolAddress; the device address differs per device
+// and is looked up once for each, with that device current.
+std::mutex g_scratch_mutex;
+char* g_scratch_ptr[64];
+
+hipError_t scratch_of_current_device(char** ptr) {{
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {{
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (p == nullptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = static_cast<char*>(p);
+  }}
+  *ptr = g_scratch_ptr[dev];
+  return hipSuccess;
+}}
 }}  // namespace
 """
 
@@ -142,6 +172,19 @@ extern "C" float retnet_recurrent_profile(const float* q, const float* k, const 
   return aat::timed_mean_ms(s, [&]() {{
     return launch(q, k, v, decay, out, batch, heads, kdim, vdim, l, block_kdim, static_cast<char*>(workspace), s);
   }});
+}}
+
+// No hipMalloc, no hipFree, no workspace argument: the decay factors go into `scratch`.  The factor kernel
+// writes every byte of every record the scan reads, so nothing of an earlier call survives into this one
+// and nothing has to be cleared.
+extern "C" int retnet_recurrent_fwd_noalloc(const float* q, const float* k, const float* v, const float* decay, float* out,
+                                            int batch, int heads, int kdim, int vdim, int l, int block_kdim, void* stream) {{
+  if (!rec_shape_ok(batch, heads, kdim, vdim, l, block_kdim)) return AAT_ERR_SHAPE;
+  if (block_kdim > 128 || (size_t)heads * (size_t)(l / 32) > (size_t)AAT_RECURRENT_NOALLOC_MAX_RECORDS) return AAT_ERR_LIMIT;
+  char* ws = nullptr;
+  const hipError_t e = scratch_of_current_device(&ws);
+  if (e != hipSuccess) return (int)e;
+  return (int)launch(q, k, v, decay, out, batch, heads, kdim, vdim, l, block_kdim, ws, static_cast<hipStream_t>(stream));
 }}
 
 // The reference's own entry point: same name, same arguments, no status, null stream.  An unsupported

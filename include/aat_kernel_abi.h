@@ -36,6 +36,7 @@
 #define AAT_ABI_VERSION 4
 #define AAT_ERR_SHAPE (-2)      /* Seq_q / Seq_k not divisible by the tile, or a non-positive size */
 #define AAT_ERR_WORKSPACE (-3)  /* workspace missing or smaller than workspace_size() */
+#define AAT_ERR_LIMIT (-4)      /* a valid shape beyond the fixed capacity of an entry point that cannot allocate */
 
 typedef unsigned short aat_half; /* raw IEEE binary16 bits */
 
@@ -158,6 +159,18 @@ int retnet_recurrent_fwd_ex(const float* q, const float* k, const float* v, cons
 float retnet_recurrent_profile(const float* q, const float* k, const float* v, const float* decay, float* out,
                                int batch, int heads, int kdim, int vdim, int l, int block_kdim, void* workspace,
                                size_t workspace_bytes, void* stream);
+/* retnet_recurrent_fwd_ex without the workspace and without any allocation.  No counterpart in the
+ * reference; it is for callers that cannot allocate device memory at the time of the call (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  The decay factors go into a
+ * static device array inside the library, AAT_RECURRENT_NOALLOC_MAX_RECORDS records of 5120 bytes (15 MiB,
+ * held by every GPU the library runs on until the process ends), so heads * (l / 32) must not exceed that
+ * number and block_kdim must not exceed 128: AAT_ERR_LIMIT otherwise, AAT_ERR_SHAPE for what
+ * retnet_recurrent_fwd_ex rejects too, 0 on success, a positive hipError_t from the runtime.  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress); make that call outside a capture.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU race. */
+#define AAT_RECURRENT_NOALLOC_MAX_RECORDS 3072
+int retnet_recurrent_fwd_noalloc(const float* q, const float* k, const float* v, const float* decay, float* out,
+                                 int batch, int heads, int kdim, int vdim, int l, int block_kdim, void* stream);
 #endif
 
 #ifdef __cplusplus

@@ -36,8 +36,9 @@ def test_header_declares_the_reference_pair_for_every_operator():
     assert _declared_symbols("AAT_OP_ATTN_BWD") == ["abi_version", "config_string", "kernel_entry_ex", "profile_ex", "workspace_size"]
     # the recurrent form keeps the reference's own entry-point name (reference recurrent.h:427)
     assert _declared_symbols("AAT_OP_RET_RECURRENT") == ["abi_version", "config_string", "retnet_recurrent_fwd",
-                                                         "retnet_recurrent_fwd_ex", "retnet_recurrent_profile",
-                                                         "retnet_recurrent_workspace_size", "workspace_size"]
+                                                         "retnet_recurrent_fwd_ex", "retnet_recurrent_fwd_noalloc",
+                                                         "retnet_recurrent_profile", "retnet_recurrent_workspace_size",
+                                                         "workspace_size"]
 
 
 def test_wrapper_text_carries_the_configuration():
