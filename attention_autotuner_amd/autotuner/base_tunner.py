@@ -23,6 +23,7 @@ import torch
 
 from . import codegen, library, verify
 from .configs import supported_configs
+from .gfx950_space import NoValidConfigError
 
 _PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
 DEFAULT_CACHE_DIR = os.environ.get("AAT_CACHE_DIR", os.path.join(_PKG, "cache"))
@@ -185,7 +186,7 @@ class BaseTunner:
                 return cached
         configs = [c for c in self.get_tuned_configs() if self._fits_problem(c)]
         if not configs:
-            raise RuntimeError(f"no valid {self.op_name} configuration for {self.problem_key} {self.problem_shape}")
+            raise NoValidConfigError(f"no valid {self.op_name} configuration for {self.problem_key} {self.problem_shape}")
         if self.verbose:
             print("Configs to be tuned: ")
             for c in configs:

@@ -8,6 +8,11 @@ all resident blocks) and a per-lane register estimate (512 / waves_per_eu).
 """
 from .configs import AttnConfig, RetConfig, RetBwdConfig, AttnBwdConfig
 
+
+class NoValidConfigError(ValueError):
+    """No configuration of the gfx950 space fits the problem (head sizes beyond what one wave's registers or
+    the LDS hold, a sequence length no tile divides)."""
+
 WAVE = 64
 MFMA_M = 32
 BR_LIST = (64, 128, 256)
@@ -174,7 +179,7 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
         cfg.fuse_type = "shared"
         if forward_valid(cfg, arch):
             return cfg
-    raise ValueError(f"no default {op} configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
+    raise NoValidConfigError(f"no default {op} configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
 
 
 # ---- backward (RetNet) ---------------------------------------------------------------------------------
@@ -262,7 +267,7 @@ def default_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
                            num_stages_mask=sy, num_stages_dv=sz, waves_per_eu=wpe)
         if backward_valid(cfg, arch):
             return cfg
-    raise ValueError(f"no default ret_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
+    raise NoValidConfigError(f"no default ret_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
 
 
 # ---- backward (attention) ------------------------------------------------------------------------------
@@ -349,4 +354,4 @@ def default_attn_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
             cfg = AttnBwdConfig(br, bc, dim_qk, dim_v, nt, st, waves_per_eu=wpe, row_waves_per_eu=row_wpe)
             if attn_backward_valid(cfg, arch):
                 return cfg
-    raise ValueError(f"no default attn_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")
+    raise NoValidConfigError(f"no default attn_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")

@@ -66,7 +66,7 @@ class MultiHeadAttnFunc(torch.autograd.Function):
         tuner = AttnBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal, softmax_scale=ctx.softmax_scale)
         try:
             cc = resolve(tuner, lambda: gfx950_space.default_attn_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        except (ValueError, RuntimeError) as e:
+        except gfx950_space.NoValidConfigError as e:      # e.g. d_v = 512: dK and dV do not fit one wave's registers
             raise NotImplementedError(f"attention backward: {e}") from e
         Runtime(device_type, cc).apply(arrays, softmax_scale=ctx.softmax_scale, causal=ctx.causal)
         return dq, dk, dv, None, None, None

@@ -88,16 +88,18 @@ def test_config2_backward_b4_h32_s2048_d128(causal):
         assert (2 * g1.float() - g2.float()).abs().max().item() <= 4e-3 + 2e-3 * g2.float().abs().max().item()
 
 
-@pytest.mark.parametrize("row_wpe", [1, 2])
-@pytest.mark.parametrize("br,bc,nt,st", parity_matrix.ATTN_BWD_TILES)
+# every tile shape of the parity set with the row kernel at one wave per SIMD, and at two where two blocks fit a CU's LDS
+TILE_CASES = [(br, bc, nt, st, wpe) for br, bc, nt, st in parity_matrix.ATTN_BWD_TILES for wpe in (1, 2)
+              if gfx950_space.attn_backward_valid(AttnBwdConfig(br, bc, 128, 128, nt, st, row_waves_per_eu=wpe), ARCH)]
+assert len(TILE_CASES) > len(parity_matrix.ATTN_BWD_TILES)
+
+
+@pytest.mark.parametrize("br,bc,nt,st,row_wpe", TILE_CASES)
 def test_tile_variants_agree(br, bc, nt, st, row_wpe):
     """Tile shapes of the parity set, the row kernel compiled for one and for two waves per SIMD."""
     q, k, v, do = _inputs(1, 2, 256, 256, 128, 128, seed=5)
     o_ref, lse_ref = ref_op.attention_ref(q, k, v, 0.11, True, return_lse=True)
     cfg = AttnBwdConfig(br, bc, 128, 128, nt, st, row_waves_per_eu=row_wpe)
-    if row_wpe == 2 and not gfx950_space.attn_backward_valid(cfg, ARCH):
-        pytest.skip("two blocks of this tile shape do not fit a CU's LDS")
-    assert gfx950_space.attn_backward_valid(cfg, ARCH)
     arrays = [t.cuda() for t in (q, k, v, o_ref.half(), do, lse_ref)]
     grads = [torch.empty_like(arrays[0]), torch.empty_like(arrays[1]), torch.empty_like(arrays[2])]
     Runtime(ARCH, cfg).apply(arrays + grads, softmax_scale=0.11, causal=True)

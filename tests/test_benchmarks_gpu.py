@@ -1,0 +1,62 @@
+"""The stand-alone benchmark programs (counterparts of reference benchmarks/attention.cu and the recurrent part of
+benchmarks/retnet/retnet.cu) run on the GPU and agree with the Python-side timing of the same kernels."""
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+import attention_autotuner_amd as aat
+from attention_autotuner_amd.autotuner import AttnConfig, Runtime
+from attention_autotuner_amd.benchmarks.do_bench import LaunchTimer
+
+pytestmark = pytest.mark.gpu
+ARCH = aat.MI355X()
+BENCH_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "attention_autotuner_amd", "csrc", "benchmarks")
+LINE = re.compile(r"^(regfuse|smemfuse)\s+Br=(\d+) Bc=(\d+) thr=(\d+) bufs=(\d+)/(\d+) (?:grid=\S+ )?waves/SIMD=(\d+)(.*?)\s+mean ([\d.]+) ms\s+median ([\d.]+)")
+
+
+def _run(binary, *args):
+    path = os.path.join(BENCH_DIR, binary)
+    assert os.path.exists(path), f"{binary} is built by __graft_entry__.build()"
+    done = subprocess.run([path, *args], capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stdout + done.stderr
+    assert "HIP error" not in done.stdout
+    return done.stdout
+
+
+def test_attention_bench_agrees_with_the_library_timing_within_ten_percent():
+    out = _run("attention_bench", "4", "32", "2048", "2048", "--no-flush")
+    print(out)
+    rows = [LINE.match(l) for l in out.splitlines()]
+    rows = [m for m in rows if m]
+    assert len(rows) >= 6, out                                  # every configuration of the list produced a line
+    times = {(m[1], int(m[2]), int(m[3]), int(m[4]), int(m[7]), m[8].strip()): float(m[10]) for m in rows}
+    best_key = min(times, key=times.get)
+    assert best_key[0] == "regfuse"
+    # the same kernel through the config library's launcher, timed by the Python-side timer
+    fuse, br, bc, nt, wpe, tag = best_key
+    assert "pipelined" not in tag
+    cfg = AttnConfig(br, bc, 128, 128, 128, bc, 2, 2, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v = (torch.randn(4, 32, 2048, 128, device="cuda", generator=g).half() for _ in range(3))
+    o = torch.empty_like(q)
+    launch = Runtime(ARCH, cfg).bind([q, k, v, o], causal=False)
+    lib_ms = LaunchTimer(min_warmup_ms=50).measure(launch, calls=200).median
+    print(f"attention_bench best: {best_key} {times[best_key]:.4f} ms; library launcher: {lib_ms:.4f} ms")
+    assert abs(times[best_key] - lib_ms) <= 0.10 * lib_ms
+    # and the figure is a sane one for this problem: 0.275 TFLOP at 30% .. 60% of the 2.5 PFLOP/s peak
+    assert 0.18 <= times[best_key] <= 0.37
+
+
+def test_retnet_recurrent_bench_checks_one_slice_and_reports():
+    """Calls retnet_recurrent_fwd as the reference's benchmark does; the program verifies one (batch, head)
+    slice against the plain recurrence on the host before it times anything."""
+    from attention_autotuner_amd.autotuner import codegen
+    from attention_autotuner_amd.autotuner.configs import RetRecurrentConfig
+    lib = codegen.compile_config(RetRecurrentConfig(), ARCH)
+    out = _run("retnet_recurrent_bench", lib, "2", "4", "512", "128", "128", "--no-flush")
+    print(out)
+    assert "-> ok" in out and "MISMATCH" not in out
+    assert re.search(r"median [\d.]+ .* TFLOP/s", out)

@@ -161,3 +161,47 @@ def test_ops_refuse_cpu_tensors():
     x = torch.zeros(1, 1, 64, 32)
     with pytest.raises(RuntimeError, match="GPU only"):
         aat.retnet_recurrent_fwd(x, x, x, torch.ones(1, 32))
+
+
+# ------------------------------------------------------------------------------ the tuning loop's guard
+def test_verify_reference_math_matches_the_oracle_and_rejects_a_perturbed_output():
+    """verify.py is torch math on whatever device its tensors live on: on the CPU its reference outputs agree
+    with the oracle, an output equal to them passes, and one wrong element, a NaN or a scaled tensor fails."""
+    from attention_autotuner_amd.autotuner import verify
+    from oracle import ref_op
+    g = torch.Generator().manual_seed(5)
+    q, k = torch.randn(1, 2, 64, 64, generator=g).half(), torch.randn(1, 2, 96, 64, generator=g).half()
+    v, do = torch.randn(1, 2, 96, 128, generator=g).half(), torch.randn(1, 2, 64, 128, generator=g).half()
+    mask = torch.randn(2, 64, 96, generator=g).half()
+    for causal in (False, True):
+        want = ref_op.attention_ref(q, k, v, 0.2, causal)
+        ref = verify.reference_outputs("attn", [q, k, v, None], scale=0.2, causal=causal)
+        torch.testing.assert_close(ref[3], want, rtol=1e-5, atol=1e-5)
+        arrays = [q, k, v, want.half()]
+        assert verify.outputs_match(arrays, ref)
+        for spoil in ("element", "nan", "scale"):
+            bad = want.clone()
+            if spoil == "element":
+                bad[0, 1, 63, 5] += 0.05
+            elif spoil == "nan":
+                bad[0, 0, 0, 0] = float("nan")
+            else:
+                bad *= 1.05
+            assert not verify.outputs_match([q, k, v, bad.half()], ref), (causal, spoil)
+    o_ref, r_ref = ref_op.retnet_ref(q, k, v, mask, return_r=True)
+    ref = verify.reference_outputs("ret", [q, k, v, mask, None, None])
+    torch.testing.assert_close(ref[4], o_ref, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(ref[5], r_ref, rtol=1e-5, atol=1e-5)
+    grads = ref_op.retnet_bwd_ref(q, k, v, mask, do, r_ref, operand_dtype=torch.float16)
+    ref = verify.reference_outputs("ret_bwd", [q, k, v, mask, do, r_ref, None, None, None, None])
+    for idx, gr in zip((6, 7, 8), grads):
+        torch.testing.assert_close(ref[idx], gr, rtol=1e-5, atol=1e-5)
+    outs = [q, k, v, mask, do, r_ref] + [t.half() for t in grads]
+    assert verify.outputs_match(outs, ref)
+    outs[7] = (grads[1] + 0.05 * (torch.arange(grads[1].numel()).view_as(grads[1]) == 77)).half()
+    assert not verify.outputs_match(outs, ref)
+    # the decay variant builds its mask from log2(gamma): gamma^(i + sk - sq - j) on and below the diagonal
+    lg = torch.log2(torch.tensor([0.9, 0.5]))
+    d = verify.decay_mask(lg, 4, 6)
+    assert d.shape == (2, 4, 6) and d[0, 0, 2] == 1.0 and d[0, 0, 3] == 0.0 and abs(d[0, 3, 2].item() - 0.9 ** 3) < 1e-6
+    assert abs(d[1, 2, 0].item() - 0.5 ** 4) < 1e-7
