@@ -4,7 +4,7 @@
 //   hipcc --offload-arch=gfx950 -O3 -fno-math-errno -ffp-contract=fast -fno-honor-nans \
 //         -Xclang -target-feature -Xclang -packed-fp32-ops -I attention_autotuner_amd/csrc \
 //         attention_autotuner_amd/csrc/benchmarks/attention.hip -o attention_bench
-//   ./attention_bench [B H Sq Sk] [--causal] [--no-flush]
+//   ./attention_bench [B H Sq Sk] [--dim 64|128] [--causal] [--no-flush]
 //
 // Inputs are N(0,1) fp16 (Box-Muller on the host from a fixed seed).  Prints mean / median / p20 / p80
 // milliseconds and TFLOP/s (2*B*H*Sq*Sk*(d_qk+d_v), halved when causal) per configuration.
@@ -33,6 +33,7 @@
 struct ProblemShape {
   int B, H, Sq, Sk;
   bool causal, flush;
+  int dim = 128;
 };
 
 static aat::half_t* device_randn(size_t n, unsigned seed) {
@@ -133,6 +134,7 @@ int main(int argc, char** argv) {
   for (int i = 1; i < argc; ++i) {
     if (!std::strcmp(argv[i], "--causal")) ps.causal = true;
     else if (!std::strcmp(argv[i], "--no-flush")) ps.flush = false;
+    else if (!std::strcmp(argv[i], "--dim") && i + 1 < argc) ps.dim = std::atoi(argv[++i]);
     else {
       int v = std::atoi(argv[i]);
       if (pos == 0) ps.B = v; else if (pos == 1) ps.H = v; else if (pos == 2) ps.Sq = v; else if (pos == 3) ps.Sk = v;
@@ -141,9 +143,22 @@ int main(int argc, char** argv) {
   }
   hipDeviceProp_t prop;
   HIP_OK(hipGetDeviceProperties(&prop, 0));
-  std::printf("%s  %d CUs  LDS/block %zu KB   problem B=%d H=%d Sq=%d Sk=%d d_qk=d_v=128 fp16 %s %s\n", prop.gcnArchName,
-              prop.multiProcessorCount, prop.sharedMemPerBlockOptin / 1024, ps.B, ps.H, ps.Sq, ps.Sk,
+  if (ps.dim != 64 && ps.dim != 128) {
+    std::printf("--dim must be 64 or 128\n");
+    return 2;
+  }
+  std::printf("%s  %d CUs  LDS/block %zu KB   problem B=%d H=%d Sq=%d Sk=%d d_qk=d_v=%d fp16 %s %s\n", prop.gcnArchName,
+              prop.multiProcessorCount, prop.sharedMemPerBlockOptin / 1024, ps.B, ps.H, ps.Sq, ps.Sk, ps.dim,
               ps.causal ? "causal" : "non-causal", ps.flush ? "(cache flushed before every launch)" : "(hot cache)");
+  if (ps.dim == 64) {
+    Buffers b = make_buffers<64, 64>(ps);
+    test_regfuse_attention<64, 64, 128, 64, 256, 2, 2, 2, false>(ps, b);
+    test_regfuse_attention<64, 64, 128, 32, 256, 2, 2, 2, false>(ps, b);
+    test_regfuse_attention<64, 64, 64, 64, 128, 2, 2, 2, false>(ps, b);
+    test_smemfuse_attention<64, 64, 64, 64, 256, 2, 2, 2, 2, 2>(ps, b);
+    HIP_OK(hipFree(b.q)); HIP_OK(hipFree(b.k)); HIP_OK(hipFree(b.v)); HIP_OK(hipFree(b.o));
+    return 0;
+  }
   Buffers b = make_buffers<128, 128>(ps);
   test_regfuse_attention<128, 128, 256, 64, 512, 2, 2, 3, false>(ps, b);
   test_regfuse_attention<128, 128, 256, 64, 512, 2, 2, 2, false>(ps, b);

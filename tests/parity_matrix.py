@@ -20,11 +20,16 @@ ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (256, 128), (256, 2
 ATTN_BWD_TILES = [(64, 32, 128, 2), (64, 64, 128, 2), (128, 64, 256, 3), (128, 32, 256, 2)]
 # kv-splitting variants: (d_qk, d_v, splits)
 SPLIT_VARIANTS = [(128, 128, 4), (128, 128, 8), (64, 64, 2)]
+# register-fused configurations the stand-alone attention benchmark times (csrc/benchmarks/attention.hip): (d, Br, Bc, threads, waves/SIMD)
+STANDALONE_BENCH_TILES = [(64, 128, 64, 256, 2), (64, 128, 32, 256, 2), (64, 64, 64, 128, 2), (128, 256, 64, 512, 3),
+                          (128, 256, 64, 512, 2), (128, 128, 64, 256, 3), (128, 128, 32, 256, 3)]
 
 
 def parity_configs(arch=None):
     arch = arch or MI355X()
     out = []
+    for d, br, bc, nt, wpe in STANDALONE_BENCH_TILES:
+        out.append(AttnConfig(br, bc, d, d, d, bc, 2, 2, nt, True, waves_per_eu=wpe).set_fuse_type("register"))
     # RetNet forward variants at 128/128 (register and both wave grids of the LDS-fused kernel)
     for fuse, extra in (("register", {}), ("shared", dict(warps_mma1_n=1, warps_mma_n=4)), ("shared", dict(warps_mma1_n=2, warps_mma_n=2))):
         for st in ((1, 1), (2, 2)):

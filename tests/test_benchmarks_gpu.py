@@ -26,28 +26,28 @@ def _run(binary, *args):
     return done.stdout
 
 
-def test_attention_bench_agrees_with_the_library_timing_within_ten_percent():
-    out = _run("attention_bench", "4", "32", "2048", "2048", "--no-flush")
+# the small plumbing shape (d = 64) and the headline shape (d = 128) of the benchmark configurations
+@pytest.mark.parametrize("b,h,s,dim,min_lines", [(2, 8, 512, 64, 4), (4, 32, 2048, 128, 6)])
+def test_attention_bench_agrees_with_the_library_timing_within_ten_percent(b, h, s, dim, min_lines):
+    out = _run("attention_bench", str(b), str(h), str(s), str(s), "--dim", str(dim), "--no-flush")
     print(out)
-    rows = [LINE.match(l) for l in out.splitlines()]
-    rows = [m for m in rows if m]
-    assert len(rows) >= 6, out                                  # every configuration of the list produced a line
+    rows = [m for m in (LINE.match(l) for l in out.splitlines()) if m]
+    assert len(rows) >= min_lines, out                          # every configuration of the list produced a line
     times = {(m[1], int(m[2]), int(m[3]), int(m[4]), int(m[7]), m[8].strip()): float(m[10]) for m in rows}
-    best_key = min(times, key=times.get)
-    assert best_key[0] == "regfuse"
+    regfuse = {key: t for key, t in times.items() if key[0] == "regfuse" and "pipelined" not in key[5]}
+    best_key = min(regfuse, key=regfuse.get)
     # the same kernel through the config library's launcher, timed by the Python-side timer
     fuse, br, bc, nt, wpe, tag = best_key
-    assert "pipelined" not in tag
-    cfg = AttnConfig(br, bc, 128, 128, 128, bc, 2, 2, nt, True, waves_per_eu=wpe).set_fuse_type("register")
+    cfg = AttnConfig(br, bc, dim, dim, dim, bc, 2, 2, nt, True, waves_per_eu=wpe).set_fuse_type("register")
     g = torch.Generator(device="cuda").manual_seed(0)
-    q, k, v = (torch.randn(4, 32, 2048, 128, device="cuda", generator=g).half() for _ in range(3))
+    q, k, v = (torch.randn(b, h, s, dim, device="cuda", generator=g).half() for _ in range(3))
     o = torch.empty_like(q)
     launch = Runtime(ARCH, cfg).bind([q, k, v, o], causal=False)
     lib_ms = LaunchTimer(min_warmup_ms=50).measure(launch, calls=200).median
     print(f"attention_bench best: {best_key} {times[best_key]:.4f} ms; library launcher: {lib_ms:.4f} ms")
-    assert abs(times[best_key] - lib_ms) <= 0.10 * lib_ms
-    # and the figure is a sane one for this problem: 0.275 TFLOP at 30% .. 60% of the 2.5 PFLOP/s peak
-    assert 0.18 <= times[best_key] <= 0.37
+    assert abs(times[best_key] - lib_ms) <= max(0.10 * lib_ms, 0.002)      # 2 us floor: the small shape runs a few microseconds
+    if dim == 128:      # a sane figure for the headline problem: 0.275 TFLOP at 30% .. 60% of the 2.5 PFLOP/s peak
+        assert min(times.values()) == times[best_key] and 0.18 <= times[best_key] <= 0.37
 
 
 def test_retnet_recurrent_bench_checks_one_slice_and_reports():
