@@ -170,9 +170,12 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   bool prefetched = false;                      // Q fragments and kv tile 0 of this row block were requested by the previous pass
   for (int vb = blockIdx.x;; vb += gridDim.x) {
     const int tile = PERSIST ? xcd_remap(vb, n_items) : xcd_remap(vb, (int)gridDim.x);
-    const int bh = tile / Tr;
-    int rb = tile % Tr;
-    if constexpr (CAUSAL) rb = Tr - 1 - rb;       // long rows first
+    int bh = tile / Tr, rb = tile % Tr;
+    if constexpr (CAUSAL) {                       // long rows first, over all heads of the XCD
+      const TileId t = causal_tile(vb, (int)gridDim.x, Tr, true);
+      bh = t.bh;
+      rb = t.blk;
+    }
     const int q0 = rb * Br;
     int n_tiles = seq_k / Bc;
     int n_full = n_tiles;                         // tiles [0, n_full) are visible to every row of the block

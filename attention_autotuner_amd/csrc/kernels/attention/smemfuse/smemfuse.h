@@ -63,9 +63,12 @@ flashattn_fwd_smemfuse(const half_t* __restrict__ q, const half_t* __restrict__ 
 
   const int Tr = seq_q / Br;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = tile / Tr;
-  int rb = tile % Tr;
-  if constexpr (CAUSAL) rb = Tr - 1 - rb;
+  int bh = tile / Tr, rb = tile % Tr;
+  if constexpr (CAUSAL) {
+    const TileId t = causal_tile(blockIdx.x, gridDim.x, Tr, true);
+    bh = t.bh;
+    rb = t.blk;
+  }
   const int q0 = rb * Br;
   const int diag = seq_k - seq_q;
   int n_tiles = seq_k / Bc;

@@ -98,9 +98,12 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
 
   const int Tx = seq_x / BX;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = tile / Tx;
-  int xb = tile % Tx;
-  if (causal && !COL) xb = Tx - 1 - xb;           // query blocks near the end walk the most kv tiles: start them first
+  int bh = tile / Tx, xb = tile % Tx;
+  if (causal) {                                   // longest blocks first: the last query blocks, the first kv blocks
+    const TileId t = causal_tile(blockIdx.x, gridDim.x, Tx, !COL);
+    bh = t.bh;
+    xb = t.blk;
+  }
   const int x0 = xb * BX;
   const int dz0 = blockIdx.y * DZB;               // first output column of this block
   const int diag = seq_k - seq_q;                 // mask[q][kv] may be non-zero only for kv <= q + diag

@@ -66,9 +66,12 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
 
   const int Tr = seq_q / Br;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = tile / Tr;
-  int rb = tile % Tr;
-  if (causal) rb = Tr - 1 - rb;
+  int bh = tile / Tr, rb = tile % Tr;
+  if (causal) {
+    const TileId t = causal_tile(blockIdx.x, gridDim.x, Tr, true);
+    bh = t.bh;
+    rb = t.blk;
+  }
   const int q0 = rb * Br;
   int n_tiles = seq_k / Bc;
   if (causal) {

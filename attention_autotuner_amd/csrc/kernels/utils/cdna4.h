@@ -292,4 +292,27 @@ AAT_DEV int xcd_remap(int wg, int grid) {
   return (wg % kXcd) * (grid / kXcd) + wg / kXcd;
 }
 
+// (batch*head, block) of a workgroup in a causal walk with T blocks per head.  A block's length grows
+// linearly with its position in the head (row blocks: the last one is the longest; kv blocks of a
+// column pass: the first one), and the chip holds only part of the grid at a time, so the order in which
+// blocks are dealt out decides the tail of the launch.  Longest first *within each head* is not enough:
+// the CUs that finish a head's short blocks early are handed the next head's longest ones.  The blocks of
+// all heads that share an XCD are therefore dealt out in one sequence sorted by length, longest first,
+// which lets every CU end up with about the same total (a head still stays on one XCD and one L2).
+struct TileId {
+  int bh, blk;
+};
+AAT_DEV TileId causal_tile(int wg, int grid, int T, bool last_is_longest) {
+  const int tile = xcd_remap(wg, grid);
+  const int per_xcd = grid / 8;
+  int bh = tile / T, pos = tile % T;
+  if (grid % 8 == 0 && per_xcd % T == 0) {
+    const int heads = per_xcd / T;                // heads per XCD
+    const int l = tile % per_xcd;
+    bh = (tile / per_xcd) * heads + l % heads;
+    pos = l / heads;
+  }
+  return {bh, last_is_longest ? T - 1 - pos : pos};
+}
+
 }  // namespace aat
