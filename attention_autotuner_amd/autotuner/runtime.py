@@ -64,7 +64,7 @@ class Runtime:
             scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])
             extra = [ctypes.c_float(scale), ctypes.c_int(int(bool(causal)))]
         else:
-            extra = [ctypes.c_int(int(bool(causal)))]
+            extra = [ctypes.c_int(mask_mode(causal))]
         with torch.cuda.device(q.device):
             stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
             ptrs = [ctypes.c_void_p(t.data_ptr()) for t in torch_array]
@@ -100,7 +100,7 @@ class Runtime:
         args = [ctypes.c_void_p(t.data_ptr()) for t in torch_array] + [B, H, Sq, Sk]
         if op in library.SCALED_OPS:
             args.append(ctypes.c_float(softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])))
-        args += [ctypes.c_int(int(bool(causal))),
+        args += [ctypes.c_int(int(bool(causal)) if op in library.SCALED_OPS else mask_mode(causal)),
                  ctypes.c_void_p(workspace.data_ptr() if workspace is not None else 0),
                  ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0)]
         with torch.cuda.device(q.device):
@@ -114,6 +114,18 @@ class Runtime:
 
         launch.keep_alive = keep
         return launch
+
+
+MASK_MODES = {"dense": 0, "causal": 1, "scan": 2, "scanned": 3}
+
+
+def mask_mode(causal):
+    """The integer the *_ex entry points take as ``causal``: False / True, or for the RetNet operators one of
+    "dense", "causal", "scan" (scan the mask tensor for all-zero tiles first, into the workspace) and
+    "scanned" (the workspace holds that scan already)."""
+    if isinstance(causal, str):
+        return MASK_MODES[causal]
+    return int(bool(causal))
 
 
 def compile_parallel(configs, arch, tmp_dir=None):

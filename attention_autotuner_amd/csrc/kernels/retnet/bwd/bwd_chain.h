@@ -29,6 +29,7 @@
 #include <type_traits>
 
 #include "../../utils/cdna4.h"
+#include "../../utils/mask_extents.h"
 #include "../../utils/retention.h"
 #include "../../utils/tile_ops.h"
 
@@ -79,7 +80,8 @@ template <int KX, int DZ, int DZB, int BX, int BY, int Nthreads, int NSY, int NS
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const half_t* __restrict__ z,
               const half_t* __restrict__ mask, const float* __restrict__ r, half_t* __restrict__ out, int H,
-              int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr) {
+              int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr,
+              const int* __restrict__ extents = nullptr) {
   if constexpr (DECAY) causal = 1;
   using T = RetBwdChain<KX, DZ, DZB, BX, BY, Nthreads, NSY, NSZ, PASS>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCY = T::NCY, NCZ = T::NCZ, NCM = T::NCM, WM = T::WM;
@@ -99,7 +101,7 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   const int Tx = seq_x / BX;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
   int bh = tile / Tx, xb = tile % Tx;
-  if (causal) {                                   // longest blocks first: the last query blocks, the first kv blocks
+  if (causal || extents != nullptr) {             // longest blocks first: the last query blocks, the first kv blocks
     const TileId t = causal_tile(blockIdx.x, gridDim.x, Tx, !COL);
     bh = t.bh;
     xb = t.blk;
@@ -108,7 +110,13 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   const int dz0 = blockIdx.y * DZB;               // first output column of this block
   const int diag = seq_k - seq_q;                 // mask[q][kv] may be non-zero only for kv <= q + diag
   int j_begin = 0, j_end = seq_y / BY;
-  if (causal) {
+  if (extents != nullptr) {                       // the streamed tiles in which the mask has a non-zero entry for these rows
+    const MaskExtents e = mask_extents_at(extents, H, seq_q, seq_k);
+    int lo, hi;
+    if constexpr (COL) mask_col_range(e, bh % H, seq_k, x0, BX, lo, hi);
+    else mask_row_range(e, bh % H, seq_q, x0, BX, lo, hi);
+    mask_tile_range(lo, hi, BY, j_end, j_begin, j_end);
+  } else if (causal) {
     if constexpr (COL) {                          // q tiles that reach kv >= x0:  q >= x0 - diag
       const int first = x0 - diag;
       j_begin = first <= 0 ? 0 : first / BY;

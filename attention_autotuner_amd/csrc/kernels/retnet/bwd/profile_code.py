@@ -44,7 +44,8 @@ bool bwd_shape_ok(int B, int H, int Seq_q, int Seq_k) {{
 }}
 
 hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
-                  aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k, int causal, hipStream_t stream) {{
+                  aat_half* dk, aat_half* dv, int B, int H, int Seq_q, int Seq_k, int mask_mode, void* workspace,
+                  hipStream_t stream) {{
   static const hipError_t ok1 = aat::allow_lds(kernel_dv, TV::kSmemBytes);
   static const hipError_t ok2 = aat::allow_lds(kernel_dk, TK::kSmemBytes);
   static const hipError_t ok3 = aat::allow_lds(kernel_dq, TQ::kSmemBytes);
@@ -54,12 +55,16 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_hal
   using H16 = aat::half_t;
   const H16 *Q = reinterpret_cast<const H16*>(q), *K = reinterpret_cast<const H16*>(k), *V = reinterpret_cast<const H16*>(v),
             *M = reinterpret_cast<const H16*>(mask), *G = reinterpret_cast<const H16*>(dO);
+  aat::MaskWalk walk;
+  const hipError_t scanned = aat::prepare_mask_walk(mask_mode, M, H, Seq_q, Seq_k, workspace, stream, &walk);
+  if (scanned != hipSuccess) return scanned;
+  const int causal = walk.causal;
   kernel_dv<<<dim3(B * H * (Seq_k / Br), D / DVB), dim3(Nthreads), TV::kSmemBytes, stream>>>(
-      K, Q, G, M, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, causal, nullptr);
+      K, Q, G, M, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, causal, nullptr, walk.extents);
   kernel_dk<<<dim3(B * H * (Seq_k / Br), Kd / DKB), dim3(Nthreads), TK::kSmemBytes, stream>>>(
-      V, G, Q, M, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, causal, nullptr);
+      V, G, Q, M, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, causal, nullptr, walk.extents);
   kernel_dq<<<dim3(B * H * (Seq_q / Br), Kd / DKB), dim3(Nthreads), TQ::kSmemBytes, stream>>>(
-      G, V, K, M, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, causal, nullptr);
+      G, V, K, M, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, causal, nullptr, walk.extents);
   return hipGetLastError();
 }}
 // Decay-mask variant: the mask is gamma_h^(q + Seq_k - Seq_q - kv) below the diagonal, zero above it.
@@ -75,27 +80,33 @@ hipError_t launch_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2
   const H16 *Q = reinterpret_cast<const H16*>(q), *K = reinterpret_cast<const H16*>(k), *V = reinterpret_cast<const H16*>(v),
             *G = reinterpret_cast<const H16*>(dO);
   decay_dv<<<dim3(B * H * (Seq_k / Br), D / DVB), dim3(Nthreads), TV::kSmemBytes, stream>>>(
-      K, Q, G, nullptr, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, 1, log2_gamma);
+      K, Q, G, nullptr, r, reinterpret_cast<H16*>(dv), H, Seq_k, Seq_q, 1, log2_gamma, nullptr);
   decay_dk<<<dim3(B * H * (Seq_k / Br), Kd / DKB), dim3(Nthreads), TK::kSmemBytes, stream>>>(
-      V, G, Q, nullptr, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, 1, log2_gamma);
+      V, G, Q, nullptr, r, reinterpret_cast<H16*>(dk), H, Seq_k, Seq_q, 1, log2_gamma, nullptr);
   decay_dq<<<dim3(B * H * (Seq_q / Br), Kd / DKB), dim3(Nthreads), TQ::kSmemBytes, stream>>>(
-      G, V, K, nullptr, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, 1, log2_gamma);
+      G, V, K, nullptr, r, reinterpret_cast<H16*>(dq), H, Seq_k, Seq_q, 1, log2_gamma, nullptr);
   return hipGetLastError();
 }}
 }}  // namespace
 
 extern "C" int abi_version(void) {{ return AAT_ABI_VERSION; }}
 extern "C" const char* config_string(void) {{ return "{config_name}"; }}
-extern "C" size_t workspace_size(int, int, int, int) {{ return 0; }}
+// Needed for the scanning mask modes only (AAT_MASK_SCAN / AAT_MASK_SCANNED); the same layout as the forward's.
+extern "C" size_t workspace_size(int, int H, int Seq_q, int Seq_k) {{
+  return H > 0 && Seq_q > 0 && Seq_k > 0 ? aat::mask_extent_bytes(H, Seq_q, Seq_k) : 0;
+}}
+static_assert(AAT_MASK_DENSE == aat::kMaskDense && AAT_MASK_CAUSAL == aat::kMaskCausal && AAT_MASK_SCAN == aat::kMaskScan &&
+              AAT_MASK_SCANNED == aat::kMaskScanned, "mask modes of the header and of the kernels");
 """
 
 profile_func = r"""
 extern "C" float profile_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
-                            aat_half* dk, aat_half* dv, float*, int B, int H, int Seq_q, int Seq_k, int causal, void*,
-                            size_t, void* stream) {{
+                            aat_half* dk, aat_half* dv, float*, int B, int H, int Seq_q, int Seq_k, int causal,
+                            void* workspace, size_t workspace_bytes, void* stream) {{
   if (!bwd_shape_ok(B, H, Seq_q, Seq_k)) return -1.f;
+  if (!aat::mask_mode_ok(causal, workspace, workspace_bytes, H, Seq_q, Seq_k)) return -1.f;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return aat::timed_mean_ms(s, [&] {{ return launch(q, k, v, mask, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, causal, s); }});
+  return aat::timed_mean_ms(s, [&] {{ return launch(q, k, v, mask, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, causal, workspace, s); }});
 }}
 extern "C" float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
                          aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q, int Seq_k) {{
@@ -106,9 +117,10 @@ extern "C" float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, 
 kernel_entry = r"""
 extern "C" int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
                                aat_half* dq, aat_half* dk, aat_half* dv, float*, int B, int H, int Seq_q, int Seq_k,
-                               int causal, void*, size_t, void* stream) {{
-  if (!bwd_shape_ok(B, H, Seq_q, Seq_k)) return AAT_ERR_SHAPE;
-  return (int)launch(q, k, v, mask, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, causal, static_cast<hipStream_t>(stream));
+                               int causal, void* workspace, size_t workspace_bytes, void* stream) {{
+  if (!bwd_shape_ok(B, H, Seq_q, Seq_k) || causal < 0 || causal > AAT_MASK_SCANNED) return AAT_ERR_SHAPE;
+  if (!aat::mask_mode_ok(causal, workspace, workspace_bytes, H, Seq_q, Seq_k)) return AAT_ERR_WORKSPACE;
+  return (int)launch(q, k, v, mask, dO, r, dq, dk, dv, B, H, Seq_q, Seq_k, causal, workspace, static_cast<hipStream_t>(stream));
 }}
 extern "C" int kernel_entry(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r, aat_half* dq,
                             aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_k, int Seq_q) {{

@@ -11,6 +11,7 @@
 #include <type_traits>
 
 #include "../../utils/cdna4.h"
+#include "../../utils/mask_extents.h"
 #include "../../utils/retention.h"
 #include "../../utils/tile_ops.h"
 
@@ -49,7 +50,8 @@ template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int NSM
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, const half_t* __restrict__ v,
                 const half_t* __restrict__ mask, half_t* __restrict__ o, float* __restrict__ r, int H,
-                int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr) {
+                int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr,
+                const int* __restrict__ extents = nullptr) {
   if constexpr (DECAY) causal = 1;
   using T = RetFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV, NSM>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, NCM = T::NCM, WM = T::WM;
@@ -67,14 +69,18 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
   const int Tr = seq_q / Br;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
   int bh = tile / Tr, rb = tile % Tr;
-  if (causal) {
+  if (causal || extents != nullptr) {             // a scanned mask is taken to be of the causal kind: later rows see more
     const TileId t = causal_tile(blockIdx.x, gridDim.x, Tr, true);
     bh = t.bh;
     rb = t.blk;
   }
   const int q0 = rb * Br;
   int n_tiles = seq_k / Bc;
-  if (causal) {
+  if (extents != nullptr) {                       // walk up to the last kv tile in which the mask has a non-zero entry
+    int lo, hi, j_begin;
+    mask_row_range(mask_extents_at(extents, H, seq_q, seq_k), bh % H, seq_q, q0, Br, lo, hi);
+    mask_tile_range(lo, hi, Bc, n_tiles, j_begin, n_tiles);
+  } else if (causal) {
     const int last = q0 + Br - 1 + (seq_k - seq_q);
     const int lim = last < 0 ? 0 : last / Bc + 1;
     n_tiles = lim < n_tiles ? lim : n_tiles;

@@ -2,8 +2,12 @@
 
 Drop-in for reference python/ops/retnet_interface.py:8-57:
 ``S = (q k^T) * mask``, ``r = clamp(sum_j |S|, min=1)`` (treated as a constant in the gradient),
-``o = (S / r) v``.  mask is [H, S_q, S_kv] fp16.  ``causal=True`` promises the mask is zero above the
-diagonal, which lets the kernels skip those tiles (the reference accepts and ignores the flag).
+``o = (S / r) v``.  mask is [H, S_q, S_kv] fp16.  Tiles in which the mask is zero contribute exactly
+nothing, and RetNet's own masks are zero above the diagonal, so by default (``causal=None``) the forward
+scans the mask once (one read of it, on the GPU, no host synchronisation) and forward and backward then
+skip the all-zero tiles at the start and end of every band of rows; the result has the same bits as the
+dense walk.  ``causal=True`` promises zeros above the diagonal instead of scanning, ``causal=False`` walks
+every tile as the reference does (it accepts the flag and ignores it).
 backward returns one gradient per forward input (the reference returns one too few).
 
 ``RetNetDecayAttnFunc(q, k, v, gamma, device_type)`` is the same operator for RetNet's own mask,
@@ -24,7 +28,7 @@ from ._resolve import resolve
 class RetNetAttn(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, q, k, v, mask, device_type: Arch, causal=False):
+    def forward(ctx, q, k, v, mask, device_type: Arch, causal=None):
         if not (q.is_cuda and k.is_cuda and v.is_cuda and mask.is_cuda):
             raise RuntimeError("RetNetAttnFunc runs on the GPU only (HIP kernels); move the tensors to a cuda device")
         assert q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16 and mask.dtype == torch.float16
@@ -40,12 +44,20 @@ class RetNetAttn(torch.autograd.Function):
         o = torch.empty(batch_size, nheads, seqlen_q, head_dim, device=q.device, dtype=torch.float16)
         r = torch.empty(batch_size, nheads, seqlen_q, device=q.device, dtype=torch.float32)
         arrays = [q, k, v, maskr, o, r]
-        tuner = RetTunner(arch=device_type, torch_array=arrays, causal=causal)
+        # the scanning walk is tuned as the causal one: masks that have zero tiles to skip are of that kind
+        tuner = RetTunner(arch=device_type, torch_array=arrays, causal=causal is None or bool(causal))
         cc = resolve(tuner, lambda: gfx950_space.default_forward_config("ret", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        Runtime(device_type, cc).apply(arrays, causal=causal)
+        rt = Runtime(device_type, cc)
+        scan = None
+        if causal is None:                     # the scan lands in `scan`; the backward reads it from there
+            scan = torch.empty(rt.workspace_size(batch_size, nheads, seqlen_q, seqlen_k), dtype=torch.uint8, device=q.device)
+            rt.apply(arrays, causal="scan", workspace=scan)
+        else:
+            rt.apply(arrays, causal=bool(causal))
         ctx.save_for_backward(q, k, v, maskr, r)
         ctx.device_type = device_type
         ctx.causal = causal
+        ctx.mask_scan = scan
         return o
 
     @staticmethod
@@ -63,9 +75,12 @@ class RetNetAttn(torch.autograd.Function):
         # touch it (dQ is produced directly), so a token buffer stands in for the [B,H,S_q,d_qk] tensor.
         dq_accum = torch.zeros(1, device=q.device, dtype=torch.float32)
         arrays = [q, k, v, mask, do, r, dq, dk, dv, dq_accum]
-        tuner = RetBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal)
+        tuner = RetBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal is None or bool(ctx.causal))
         cc = resolve(tuner, lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        Runtime(device_type, cc).apply(arrays, causal=ctx.causal)
+        if ctx.mask_scan is not None:
+            Runtime(device_type, cc).apply(arrays, causal="scanned", workspace=ctx.mask_scan)
+        else:
+            Runtime(device_type, cc).apply(arrays, causal=bool(ctx.causal))
         return dq, dk, dv, None, None, None
 
 

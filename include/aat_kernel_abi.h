@@ -25,8 +25,9 @@
  *     a positive hipError_t on a launch failure, AAT_ERR_SHAPE for an indivisible shape;
  *   - the *_ex entry points take (Seq_q, Seq_k) in that order plus a runtime softmax scale, a causal
  *     flag, an optional workspace and the stream to launch on (a hipStream_t passed as void*);
- *   - workspace_size() says how many bytes of workspace a problem needs (0 unless the configuration
- *     splits the kv range); abi_version() and config_string() identify the library.
+ *   - workspace_size() says how many bytes of workspace a problem needs (attention forward: 0 unless the
+ *     configuration splits the kv range; RetNet: the mask scan of AAT_MASK_SCAN, not needed by the other
+ *     mask modes); abi_version() and config_string() identify the library.
  */
 #ifndef AAT_KERNEL_ABI_H
 #define AAT_KERNEL_ABI_H
@@ -37,6 +38,16 @@
 #define AAT_ERR_SHAPE (-2)      /* Seq_q / Seq_k not divisible by the tile, or a non-positive size */
 #define AAT_ERR_WORKSPACE (-3)  /* workspace missing or smaller than workspace_size() */
 #define AAT_ERR_LIMIT (-4)      /* a valid shape beyond the fixed capacity of an entry point that cannot allocate */
+
+/* Values of the `causal` argument of the RetNet *_ex entry points, whose mask is a tensor: how much of it
+ * to walk.  Tiles in which the mask is zero contribute exactly nothing, so every mode gives the same bits. */
+#define AAT_MASK_DENSE 0    /* every tile (what the reference does) */
+#define AAT_MASK_CAUSAL 1   /* the caller promises mask == 0 above the diagonal: those tiles are skipped */
+#define AAT_MASK_SCAN 2     /* the call first scans the mask (one read of it) into the workspace and then skips
+                               the leading and trailing all-zero tiles of every band of rows; needs
+                               workspace_size() bytes */
+#define AAT_MASK_SCANNED 3  /* as AAT_MASK_SCAN, but the workspace already holds the scan of this same mask and
+                               shape, written by an earlier AAT_MASK_SCAN call of any RetNet library */
 
 typedef unsigned short aat_half; /* raw IEEE binary16 bits */
 

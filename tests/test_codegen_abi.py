@@ -77,6 +77,9 @@ def test_shipping_set_is_built_and_exports_the_abi():
             assert lib.retnet_recurrent_workspace_size(8, 4, 256, 64, 2000, 256) == 0     # unsupported shape
         elif cfg.operation == "attn_bwd":
             assert lib.workspace_size(2, 3, 256, 512) == 2 * 2 * 3 * 256 * 4      # lse2 + delta, fp32 per query row
+        elif cfg.operation in ("ret", "ret_bwd"):       # the mask scan: 4 ranges per band of 32 rows / columns + a byte per 32 x 32 tile
+            assert lib.workspace_size(5, 3, 256, 512) == 1024            # 4 * 3 * (2 * 8 + 2 * 16) + 3 * 8 * 16 = 960, in units of 256
+            assert lib.workspace_size(1, 1, 256, 256) == 256                       # rounded up to 256 bytes
         elif getattr(cfg, "kv_splits", 1) == 1:
             assert lib.workspace_size(1, 1, 256, 256) == 0
 

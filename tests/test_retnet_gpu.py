@@ -214,3 +214,99 @@ def test_decay_rate_must_be_one_per_head_and_in_range():
         aat.RetNetDecayAttnFunc(q, q, q, [0.9], ARCH)
     with pytest.raises(AssertionError):
         aat.RetNetDecayAttnFunc(q, q, q, [0.9, 0.2], ARCH)
+
+
+# ---------------------------------------------------------------------------- skipping the mask's zero tiles
+def _scan_extents(ws, h, sq, sk):
+    """The scan's four arrays (row_lo, row_hi [H, sq/32]; col_lo, col_hi [H, sk/32]) from the workspace bytes."""
+    ints = ws.cpu().numpy().view("int32")
+    nq, nk = h * (sq // 32), h * (sk // 32)
+    return (ints[:nq].reshape(h, -1), ints[nq:2 * nq].reshape(h, -1), ints[2 * nq:2 * nq + nk].reshape(h, -1),
+            ints[2 * nq + nk:2 * nq + 2 * nk].reshape(h, -1))
+
+
+def _masks(h, sq, sk, seed):
+    g = torch.Generator().manual_seed(seed)
+    dense = torch.randn(h, sq, sk, generator=g).half()
+    i = torch.arange(sq).view(sq, 1) + (sk - sq)
+    j = torch.arange(sk).view(1, sk)
+    band = dense * ((j <= i) & (j > i - 100))                        # a sliding window: zeros on both sides
+    blocks = dense * ((torch.arange(sq).view(sq, 1) // 128) == (j // 128) % (sq // 128))   # block pattern off the diagonal too
+    holes = ref_op.retnet_decay_mask(h, sq, sk).clone()
+    holes[:, 64:96, :] = 0                                            # a band of rows that sees nothing
+    holes[:, :, 32:64] = 0                                            # a band of kv positions nobody sees
+    holes[0] = 0                                                      # and a head without any entry
+    negzero = ref_op.retnet_decay_mask(h, sq, sk).clone()
+    negzero[negzero == 0] = -0.0
+    return {"decay": ref_op.retnet_decay_mask(h, sq, sk), "dense": dense, "band": band, "blocks": blocks, "holes": holes,
+            "negative zeros": negzero}
+
+
+@pytest.mark.parametrize("dqk,dv,sq,sk", [(64, 64, 256, 256), (128, 128, 256, 384), (256, 512, 256, 256)])
+def test_scanned_mask_walk_has_the_bits_of_the_dense_walk(dqk, dv, sq, sk):
+    """causal=None (the default) scans the mask for all-zero tiles and skips them in forward and backward;
+    whatever the mask looks like, outputs, r and gradients are those of the dense walk, bit for bit."""
+    q, k, v, _, do = _inputs(2, 2, sq, sk, dqk, dv, seed=21)
+    for name, mask in _masks(2, sq, sk, seed=22).items():
+        outs = {}
+        for mode in (False, None):
+            qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+            o = aat.RetNetAttnFunc(qc, kc, vc, mask.cuda(), ARCH, mode)
+            o.backward(do.cuda())
+            torch.cuda.synchronize()
+            outs[mode] = (o.detach(), qc.grad, kc.grad, vc.grad)
+        for what, a, b in zip(("o", "dq", "dk", "dv"), outs[False], outs[None]):
+            assert torch.equal(a, b), (name, what, (a.float() - b.float()).abs().max().item())
+        if name in ("holes", "band"):                                 # and the dense walk is right to begin with
+            tolerance.assert_close(outs[None][0], ref_op.retnet_ref(q, k, v, mask), f"scan {name} o")
+            _grads_close(f"scan {name}", outs[None][1:], q, k, v, mask, do)
+
+
+def test_mask_scan_records_the_non_zero_ranges():
+    h, sq, sk = 3, 256, 384
+    masks = _masks(h, sq, sk, seed=23)
+    cfg = gfx950_space.default_forward_config("ret", 64, 64, ARCH, sq, sk)
+    rt = Runtime(ARCH, cfg)
+    q, k, v, _, _ = _inputs(1, h, sq, sk, 64, 64, seed=24)
+    for name, mask in masks.items():
+        ws = torch.zeros(rt.workspace_size(1, h, sq, sk), dtype=torch.uint8, device="cuda")
+        o = torch.empty(1, h, sq, 64, dtype=torch.float16, device="cuda")
+        r = torch.empty(1, h, sq, dtype=torch.float32, device="cuda")
+        rt.apply([q.cuda(), k.cuda(), v.cuda(), mask.cuda(), o, r], causal="scan", workspace=ws)
+        torch.cuda.synchronize()
+        row_lo, row_hi, col_lo, col_hi = _scan_extents(ws, h, sq, sk)
+        nz = (mask.float().abs() > 0).view(h, sq // 32, 32, sk // 32, 32).any(4).any(2)      # [h, sq/32, sk/32]
+        for hh in range(h):
+            for b in range(sq // 32):
+                cols = torch.nonzero(nz[hh, b]).flatten()
+                if len(cols) == 0:
+                    assert row_lo[hh, b] >= row_hi[hh, b], (name, hh, b)
+                else:
+                    assert (row_lo[hh, b], row_hi[hh, b]) == (32 * int(cols[0]), 32 * int(cols[-1]) + 32), (name, hh, b)
+            for c in range(sk // 32):
+                rows = torch.nonzero(nz[hh, :, c]).flatten()
+                if len(rows) == 0:
+                    assert col_lo[hh, c] >= col_hi[hh, c], (name, hh, c)
+                else:
+                    assert (col_lo[hh, c], col_hi[hh, c]) == (32 * int(rows[0]), 32 * int(rows[-1]) + 32), (name, hh, c)
+
+
+def test_scan_modes_need_their_workspace_and_reject_unknown_modes():
+    q, k, v, mask, do = _inputs(1, 2, 128, 128, 64, 64, seed=25)
+    dev = [t.cuda() for t in (q, k, v, mask)]
+    o = torch.zeros(1, 2, 128, 64, dtype=torch.float16, device="cuda")
+    r = torch.zeros(1, 2, 128, dtype=torch.float32, device="cuda")
+    cfg = gfx950_space.default_forward_config("ret", 64, 64, ARCH, 128, 128)
+    lib = library.load(Runtime(ARCH, cfg)._path(), "ret")
+    ptrs = [ctypes.c_void_p(t.data_ptr()) for t in (*dev, o, r)]
+    need = lib.workspace_size(1, 2, 128, 128)
+    assert need >= 4 * 2 * 4 * 4 + 2 * 4 * 4
+    small = torch.zeros(need - 1, dtype=torch.uint8, device="cuda")
+    null = ctypes.c_void_p(0)
+    for mode in (2, 3):
+        assert lib.kernel_entry_ex(*ptrs, 1, 2, 128, 128, mode, null, 0, null) == -3
+        assert lib.kernel_entry_ex(*ptrs, 1, 2, 128, 128, mode, ctypes.c_void_p(small.data_ptr()), need - 1, null) == -3
+    assert lib.kernel_entry_ex(*ptrs, 1, 2, 128, 128, 4, null, 0, null) == -2
+    assert lib.kernel_entry_ex(*ptrs, 1, 2, 128, 128, -1, null, 0, null) == -2
+    assert lib.kernel_entry_ex(*ptrs, 1, 2, 128, 128, 0, null, 0, null) == 0          # the other modes need none
+    torch.cuda.synchronize()
