@@ -177,6 +177,29 @@ class BaseTunner:
             json.dump(config.to_dict(), f)
         _memo[self._memo_key()] = config
 
+    # ---- what is not worth timing ----------------------------------------------------------------------
+    def _kernel_matters(self, mangled):
+        """Whether a kernel of a candidate library is one this tuner's problem launches (a library holds
+        several variants: causal or not, decay mask or mask tensor)."""
+        return True
+
+    cost_model = None          # a fitted costmodel.CostModel: tune() then times only its best-ranked candidates
+    keep_fraction = 0.35       # ... this share of them (at least keep_min)
+    keep_min = 8
+
+    def prune(self, configs):
+        """The candidates worth compiling and timing: all of them without a cost model, else those the
+        model ranks in the best ``keep_fraction`` (reference python/tests/export_costmodel_config.py:31-56
+        exports (configuration, cycles) pairs for such a model; the model itself is autotuner/costmodel.py)."""
+        self.pruned = []
+        if self.cost_model is None or len(configs) <= self.keep_min:
+            return configs
+        shape = (self.problem_shape["B"], self.problem_shape["H"], self.problem_shape["Sq"], self.problem_shape["Sk"])
+        ranked = sorted(configs, key=lambda c: self.cost_model.predict(c, shape, self.causal))
+        keep = max(self.keep_min, int(len(ranked) * self.keep_fraction + 0.999))
+        self.pruned = ranked[keep:]
+        return ranked[:keep]
+
     # ---- the loop --------------------------------------------------------------------------------------
     def tune(self, log_path="../logs/", timeout=120, use_cache=True):
         started = time.time()
@@ -191,11 +214,18 @@ class BaseTunner:
             print("Configs to be tuned: ")
             for c in configs:
                 pprint.pprint(c)
+        configs = self.prune(configs)
         results = self.compile_parallel(configs, timeout=timeout)
         timings, best, best_ms = {}, None, FAILED
+        self.rejected_spills = {}
         for res in results:
             if res.lib_name is None:
                 continue                                  # compile failed or timed out
+            spills = codegen.spilling_kernels(codegen.resource_usage(res.lib_name), self._kernel_matters)
+            if spills and os.environ.get("AAT_TUNE_SPILLS", "0") == "0":
+                # the compiler says this candidate keeps part of its working set in scratch memory: not worth timing
+                self.rejected_spills[res.config] = max(k.get("scratch_bytes", 0) for k in spills)
+                continue
             ms = self.profile(res.lib_name)
             if ms == FAILED and self.verbose:
                 pprint.pprint(res.config)
@@ -239,3 +269,8 @@ class BaseTunner:
                 f.write(repr(cfg) + "\n" + str(ms) + "\n")
             f.write("\nbest config: \n" + repr(best) + "\n" + str(best_ms) + "\n")
             f.write("\nsearch time: " + str(elapsed) + "s")
+            # after the reference's layout: what was never timed, and why
+            for cfg, nbytes in getattr(self, "rejected_spills", {}).items():
+                f.write("\nnot timed (compiler reports " + str(nbytes) + " bytes/lane of scratch): " + str(cfg))
+            for cfg in getattr(self, "pruned", []):
+                f.write("\nnot timed (ranked out by the cost model): " + str(cfg))

@@ -11,9 +11,12 @@ in-tree directory so a tuned library is never rebuilt, and a failed or timed-out
 import functools
 import hashlib
 import importlib.util
+import json
 import os
+import re
 import shutil
 import subprocess
+import sys
 from concurrent.futures import ThreadPoolExecutor
 
 _PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
@@ -23,8 +26,11 @@ DEFAULT_BUILD_DIR = os.environ.get("AAT_BUILD_DIR", os.path.join(_PKG, "build"))
 
 # -packed-fp32-ops is switched OFF on purpose: hipcc would otherwise fuse scalar fp32 math into
 # v_pk_*_f32 instructions.
+# -Rpass-analysis=kernel-resource-usage makes the compiler report registers, scratch and occupancy of every kernel
+# it emits; the report is kept next to the library (``resource_usage``) and is what the tuners reject spilling
+# candidates by.
 HIPCC_FLAGS = ["-std=c++17", "-O3", "-fno-math-errno", "-ffp-contract=fast", "-fno-honor-nans", "-fPIC", "-shared", "-w",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Rpass-analysis=kernel-resource-usage"]
 
 
 def hipcc_exe():
@@ -145,8 +151,64 @@ def compile_config(config, arch, build_dir=None, timeout=None, force=False):
         if os.path.exists(tmp):
             os.remove(tmp)
         return None
+    with open(usage_path(out), "w") as f:
+        json.dump(parse_resource_usage(ret.stderr), f, indent=1)
     os.replace(tmp, out)
     return out
+
+
+# ---- the compiler's per-kernel resource report ---------------------------------------------------------
+_USAGE_FIELDS = {"TotalSGPRs": "sgprs", "VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes",
+                 "Occupancy [waves/SIMD]": "occupancy", "SGPRs Spill": "sgpr_spills", "VGPRs Spill": "vgpr_spills",
+                 "LDS Size [bytes/block]": "lds_bytes"}
+_USAGE_LINE = re.compile(r"remark:\s+(.+?):\s+(\S+)\s+\[-Rpass-analysis=kernel-resource-usage\]")
+
+
+def parse_resource_usage(text):
+    """[{"kernel": mangled name, "sgprs", "vgprs", "agprs", "scratch_bytes", "occupancy", "sgpr_spills",
+    "vgpr_spills", "lds_bytes"}, ...] from the remarks hipcc prints under -Rpass-analysis=kernel-resource-usage."""
+    kernels = []
+    for line in text.splitlines():
+        m = _USAGE_LINE.search(line)
+        if not m:
+            continue
+        key, value = m.group(1).strip(), m.group(2)
+        if key == "Function Name":
+            kernels.append({"kernel": value})
+        elif kernels and key in _USAGE_FIELDS and value.lstrip("-").isdigit():
+            kernels[-1][_USAGE_FIELDS[key]] = int(value)
+    return kernels
+
+
+def usage_path(lib_path):
+    return lib_path[:-3] + ".usage.json"
+
+
+def resource_usage(lib_path):
+    """The report written when ``lib_path`` was built, or None for a library built without one."""
+    try:
+        with open(usage_path(lib_path)) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return None
+
+
+def template_bools(mangled):
+    """Trailing boolean template arguments of a mangled kernel name, e.g. [False, True] for ...Lb0ELb1EEEv...;
+    the kernels here end their template lists with the flags that select a variant (causal, decay, ...)."""
+    m = re.search(r"((?:Lb[01]E)+)EEv", mangled)
+    return [c == "1" for c in re.findall(r"Lb([01])E", m.group(1))] if m else []
+
+
+# A few dwords of scratch outside the main loop (a saved address, a loop bound) cost nothing measurable and
+# several tuned winners have them; a candidate whose working set does not fit spills hundreds of bytes.
+MAX_SCRATCH_BYTES = 64
+
+
+def spilling_kernels(usage, matters=None, max_bytes=MAX_SCRATCH_BYTES):
+    """Entries of ``usage`` that keep more than ``max_bytes`` per lane in scratch memory (register spills or
+    stack arrays), restricted to the kernels ``matters(mangled name)`` accepts."""
+    return [k for k in usage or [] if k.get("scratch_bytes", 0) > max_bytes and (matters is None or matters(k["kernel"]))]
 
 
 def compile_parallel(configs, arch, build_dir=None, timeout=None, max_workers=None):
@@ -154,5 +216,15 @@ def compile_parallel(configs, arch, build_dir=None, timeout=None, max_workers=No
     ``configs`` and holds None where a compile failed."""
     workers = max_workers or int(os.environ.get("MAX_JOBS", 0)) or os.cpu_count() or 1
     workers = max(1, min(workers, 16, len(configs) or 1))
+    progress = os.environ.get("AAT_PROGRESS", "0") not in ("", "0")      # long builds under a watchdog: say that work goes on
+    done = [0]
+
+    def build(c):
+        lib = compile_config(c, arch, build_dir, timeout)
+        done[0] += 1
+        if progress and (done[0] % 8 == 0 or done[0] == len(configs)):
+            print(f"[build] {done[0]}/{len(configs)} libraries", file=sys.stderr, flush=True)
+        return lib
+
     with ThreadPoolExecutor(max_workers=workers) as pool:
-        return list(pool.map(lambda c: compile_config(c, arch, build_dir, timeout), configs))
+        return list(pool.map(build, configs))

@@ -71,9 +71,20 @@ def forward_reg_estimate(cfg):
         o_regs = (cfg.Br // MFMA_M) * (cfg.D // 32) * 16 // _waves(cfg)
     if getattr(cfg, "sw_pipeline", 0):
         s_regs *= 2                                   # current and next score tile are both live
-    if o_regs > 128 and q_regs + s_regs + o_regs > 320:
-        return 10 ** 6                                # measured: hipcc spills heavily beyond this point
+    # a count of what must be live, not a prediction of what the register allocator achieves: candidates that
+    # pass it and still spill are rejected by the tuning loop from the compiler's own resource report
     return q_regs + s_regs + p_regs + o_regs + 32
+
+
+def forward_likely_spills(cfg):
+    """Register-fused configurations whose accumulator alone takes half of a wave's budget have always come
+    back from hipcc with hundreds of bytes of scratch.  The tuning loop lets the compiler's report decide;
+    the untuned defaults stay clear of them without compiling anything."""
+    if cfg.fuse_type != "register":
+        return False
+    rt = rows_per_wave(cfg) // MFMA_M
+    o_regs = rt * (cfg.D // 32) * 16
+    return o_regs > 128 and rt * (cfg.Kd // 16) * 4 + rt * (cfg.Bc // 32) * 16 + o_regs > 320
 
 
 def shared_grid_ok(cfg):
@@ -142,8 +153,8 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
 def _shared_candidates(op, br, bc, dim_qk, dim_v, st_qk, st_v, nthreads, wpe):
     out = []
     nw = nthreads // WAVE
-    for w1n in (1, 2):
-        for w2n in sorted({nw, max(1, nw // 2)}):
+    for w1n in (1, 2, 4):
+        for w2n in sorted({nw, max(1, nw // 2), max(1, nw // 4)}):
             if op == "attn":
                 cfg = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, w1n, w2n, waves_per_eu=wpe)
             else:
@@ -166,7 +177,7 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
         else:
             cfg = RetConfig(br, bc, dim_qk, dim_v, dim_qk, bc, sq, sq, sv, nt, True, waves_per_eu=wpe)
         cfg.set_fuse_type("register")
-        if forward_valid(cfg, arch):
+        if forward_valid(cfg, arch) and not forward_likely_spills(cfg):
             return cfg
     # wide value heads: the LDS-fused kernel keeps the accumulator at Br*D/(64*waves) registers
     for br, bc, nt, w1n, w2n in ((128, 64, 512, 2, 8), (64, 64, 256, 2, 4)):
@@ -185,7 +196,7 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
 # ---- backward (RetNet) ---------------------------------------------------------------------------------
 # Three passes of one chained-contraction kernel (dV, dK, dQ).  Br = block-resident rows, Bc = streamed rows
 # per step, for every pass; both sequence lengths must divide by both.
-BWD_BR_LIST = (64, 128)
+BWD_BR_LIST = (64, 128, 256)
 BWD_BC_LIST = (32, 64)
 
 
@@ -248,7 +259,7 @@ def backward_valid(cfg, arch):
 
 def backward_candidates(br, bc, dim_qk, dim_v):
     out = []
-    for nthreads in (128, 256):
+    for nthreads in (128, 256, 512):
         for st_y, st_z in ((1, 1), (2, 2), (2, 1), (3, 2)):
             for wpe in (1, 2):
                 n = nthreads // WAVE

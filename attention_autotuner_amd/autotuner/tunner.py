@@ -7,8 +7,9 @@ test suite replays the reference's published NVIDIA tuning logs, but not built: 
 """
 import ctypes
 import math
+import os
 
-from . import gfx950_space
+from . import codegen, gfx950_space
 from .base_tunner import BaseTunner
 
 
@@ -48,6 +49,16 @@ class _ForwardTunner(BaseTunner):
     validate_register_fuse = _validate
     validate_shared_fuse = _validate
 
+    def _kernel_matters(self, mangled):
+        flags = codegen.template_bools(mangled)
+        if self.operation == "ret":                       # <..., DECAY>
+            return not flags or flags[-1] == bool(self.decay)
+        if "flashattn_fwd_regfuse" in mangled and len(flags) == 4:     # <..., PIPE, CAUSAL, SPLIT, PERSIST>
+            return flags[1] == bool(self.causal)
+        if "flashattn_fwd_smemfuse" in mangled and flags:              # <..., CAUSAL>
+            return flags[-1] == bool(self.causal)
+        return True
+
     def tune(self, *a, **kw):
         if not _is_rocm(self.arch):
             raise RuntimeError(f"{self.arch.name} configurations can be enumerated but not built on this platform")
@@ -59,6 +70,15 @@ class AttnTunner(_ForwardTunner):
 
     def __init__(self, arch, torch_array, causal=False, softmax_scale=None):
         super().__init__(arch, torch_array, "attention", causal=causal, softmax_scale=softmax_scale)
+        # the space has a few hundred candidates: with a fitted cost model next to the tuning cache, only the
+        # third it ranks best is built and timed (AAT_TUNE_PRUNE=0: time everything, as the reference does)
+        model = os.path.join(self.cache_path, "costmodel_attn.json")
+        if _is_rocm(arch) and os.environ.get("AAT_TUNE_PRUNE", "1") != "0" and os.path.exists(model):
+            from .costmodel import CostModel
+            try:
+                self.cost_model = CostModel.load(model)
+            except (OSError, ValueError, KeyError):
+                self.cost_model = None
 
     def _ex_args(self):
         scale = self.softmax_scale
@@ -92,6 +112,10 @@ class RetBwdTunner(BaseTunner):
         if _is_rocm(self.arch):
             return gfx950_space.backward_valid(config, self.arch)
         return _foreign_space(self.arch).backward_valid(config, self.arch)
+
+    def _kernel_matters(self, mangled):                   # ret_bwd_chain<..., PASS, WPE, DECAY>
+        flags = codegen.template_bools(mangled)
+        return not flags or flags[-1] == bool(self.decay)
 
     def tune(self, *a, **kw):
         if not _is_rocm(self.arch):

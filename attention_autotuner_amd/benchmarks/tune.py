@@ -76,6 +76,8 @@ def main(argv=None):
     ap.add_argument("--decay", action="store_true", help="RetNet only: decay mask built in registers from one rate per head")
     ap.add_argument("--compile-only", action="store_true")
     ap.add_argument("--log-dir", default=DEFAULT_LOG_DIR)
+    ap.add_argument("--cache-dir", default=None, help="where the best configuration is recorded (default: the package's tuning cache)")
+    ap.add_argument("--cost-model", default=None, help="a fitted cost model (JSON): only the candidates it ranks best are built and timed")
     args = ap.parse_args(argv)
     b, h, sq, sk, dqk, dv = args.dims
     arch = MI355X()
@@ -92,6 +94,11 @@ def main(argv=None):
         tuner = cls(arch, arrays, decay=True)
     else:
         tuner = cls(arch, arrays, causal=args.causal)
+    if args.cache_dir:
+        tuner.cache_path = args.cache_dir
+    if args.cost_model:
+        from ..autotuner.costmodel import CostModel
+        tuner.cost_model = CostModel.load(args.cost_model)
     if args.compile_only:
         cfgs = [c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)]
         t0 = time.time()
@@ -106,6 +113,7 @@ def main(argv=None):
     print(json.dumps({"op": args.op, "problem": args.dims, "causal": args.causal, "best": str(best), "ms": round(ms, 5),
                       "tflops": round(flops(args.op, b, h, sq, sk, dqk, dv, args.causal) / ms / 1e9, 1),
                       "candidates": len(tuner.last_timings), "ran": len(ok), "worst_ms": round(max(ok), 4),
+                      "spilling_not_timed": len(tuner.rejected_spills), "ranked_out": len(tuner.pruned),
                       "cache": tuner._cache_file(), "log": log_dir}))
     return 0
 

@@ -208,3 +208,68 @@ def test_verify_reference_math_matches_the_oracle_and_rejects_a_perturbed_output
     d = verify.decay_mask(lg, 4, 6)
     assert d.shape == (2, 4, 6) and d[0, 0, 2] == 1.0 and d[0, 0, 3] == 0.0 and abs(d[0, 3, 2].item() - 0.9 ** 3) < 1e-6
     assert abs(d[1, 2, 0].item() - 0.5 ** 4) < 1e-7
+
+
+# ---------------------------------------------------------------------- the compiler's resource report
+REMARKS = """
+x.hip:2:1: remark: Function Name: _ZN3aat13ret_bwd_chainILi256ELi512ELi512ELi128ELi32ELi256ELi3ELi2ELNS_7BwdPassE0ELi1ELb1EEEvPKDF16_ [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     TotalSGPRs: 58 [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     AGPRs: 256 [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     ScratchSize [bytes/lane]: 2416 [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     Dynamic Stack: False [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     Occupancy [waves/SIMD]: 1 [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     SGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     VGPRs Spill: 604 [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark:     LDS Size [bytes/block]: 0 [-Rpass-analysis=kernel-resource-usage]
+x.hip:3:1: remark: Function Name: _ZN3aat13ret_bwd_chainILi256ELi512ELi512ELi128ELi32ELi256ELi3ELi2ELNS_7BwdPassE0ELi1ELb0EEEvPKDF16_ [-Rpass-analysis=kernel-resource-usage]
+x.hip:3:1: remark:     VGPRs: 250 [-Rpass-analysis=kernel-resource-usage]
+x.hip:3:1: remark:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=kernel-resource-usage]
+"""
+
+
+def test_resource_report_is_parsed_and_decides_what_the_tuner_times(tmp_path, monkeypatch):
+    usage = codegen.parse_resource_usage(REMARKS)
+    assert [k["scratch_bytes"] for k in usage] == [2416, 16] and usage[0]["vgprs"] == 256 and usage[0]["vgpr_spills"] == 604
+    assert usage[0]["occupancy"] == 1 and usage[0]["agprs"] == 256 and usage[0]["sgprs"] == 58
+    assert codegen.template_bools(usage[0]["kernel"]) == [True] and codegen.template_bools(usage[1]["kernel"]) == [False]
+    assert codegen.template_bools("_ZN3aat21flashattn_fwd_regfuseILi128ELi128ELi256ELi64ELi512ELi2ELi2ELi2ELb0ELb1ELb0ELb0EEEvPKDF16_") == [False, True, False, False]
+    assert codegen.template_bools("_Z6kernelPf") == []
+    assert [k["scratch_bytes"] for k in codegen.spilling_kernels(usage)] == [2416]          # 16 bytes are below the threshold
+    assert codegen.spilling_kernels(usage, lambda name: not codegen.template_bools(name)[-1]) == []
+    assert codegen.spilling_kernels(None) == []
+    # a decay tuner looks at the decay kernels of a library, a mask-tensor tuner at the others
+    from attention_autotuner_amd.autotuner import RetBwdTunner
+    from attention_autotuner_amd.benchmarks.tune import make_tensors
+    arrays = make_tensors("ret_bwd", 1, 2, 256, 256, 256, 512, "meta")
+    assert RetBwdTunner(ARCH, arrays, decay=True)._kernel_matters(usage[0]["kernel"])
+    assert not RetBwdTunner(ARCH, arrays, causal=True)._kernel_matters(usage[0]["kernel"])
+    attn = AttnTunner(ARCH, make_tensors("attn", 1, 2, 256, 256, 128, 128, "meta"), causal=True)
+    name = "_ZN3aat21flashattn_fwd_regfuseILi128ELi128ELi256ELi64ELi512ELi2ELi2ELi2ELb0ELb%dELb0ELb0EEEvPKDF16_"
+    assert attn._kernel_matters(name % 1) and not attn._kernel_matters(name % 0)
+    # every library of the shipping set carries its report, with one entry per kernel it holds
+    cfg = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
+    report = codegen.resource_usage(codegen.library_path(cfg))
+    assert report and all("vgprs" in k and "scratch_bytes" in k for k in report)
+    assert any("flashattn_fwd_regfuse" in k["kernel"] for k in report)
+
+
+def test_tune_skips_a_candidate_the_compiler_reports_as_spilling(tmp_path, monkeypatch):
+    """The loop never times (here: never even loads) a library whose report shows a spilled working set."""
+    from attention_autotuner_amd.benchmarks.tune import make_tensors
+    tuner = AttnTunner(ARCH, make_tensors("attn", 1, 2, 256, 256, 128, 128, "meta"))
+    tuner.cache_path = str(tmp_path / "cache")
+    good = AttnConfig(128, 64, 128, 128, 128, 64, 2, 2, 256, True, waves_per_eu=2).set_fuse_type("register")
+    bad = AttnConfig(128, 32, 128, 128, 128, 32, 2, 2, 256, True, waves_per_eu=2).set_fuse_type("register")
+    monkeypatch.setattr(tuner, "get_tuned_configs", lambda: [good, bad])
+    monkeypatch.setattr(tuner, "compile_parallel", lambda cfgs, timeout=None: [base_tunner.CompileResult(c, str(c)) for c in cfgs])
+    reports = {str(good): [{"kernel": "_Z1aILb0ELb0ELb0ELb0EEvPf", "scratch_bytes": 0}],
+               str(bad): [{"kernel": "_Z1aILb0ELb0ELb0ELb0EEvPf", "scratch_bytes": 900}]}
+    monkeypatch.setattr(codegen, "resource_usage", lambda lib: reports[lib])
+    timed = []
+    monkeypatch.setattr(tuner, "profile", lambda lib: timed.append(lib) or 1.0)
+    monkeypatch.setattr(tuner, "verify", lambda lib: True)
+    best = tuner.tune(log_path=str(tmp_path / "logs"), use_cache=False)
+    assert best == good and timed == [str(good)] and tuner.rejected_spills == {bad: 900}
+    log = (tmp_path / "logs" / "profile_result_attn_128_128.txt").read_text()
+    assert "not timed (compiler reports 900 bytes/lane of scratch): " + str(bad) in log

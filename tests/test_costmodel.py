@@ -1,0 +1,90 @@
+"""The cost model that prunes the tuning search (the reference exports (configuration, cycles) pairs for such
+a model, python/tests/export_costmodel_config.py:31-56, and never reads them back): fitted on one recorded
+tuning run of an MI355X, it must keep the measured winner of runs it has not seen."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from attention_autotuner_amd.arch import MI355X
+from attention_autotuner_amd.autotuner import AttnConfig, AttnTunner, costmodel
+
+LOGS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tuning_logs", "MI355X")
+RUNS = {                                                  # file -> (shape, causal)
+    "attn_b4h32q2048k2048_c0_128_128.txt": ((4, 32, 2048, 2048), False),
+    "attn_b4h32q2048k2048_c1_128_128.txt": ((4, 32, 2048, 2048), True),
+    "attn_b8h16q1024k1024_c0_128_128.txt": ((8, 16, 1024, 1024), False),
+    "attn_b2h32q4096k4096_c1_128_128.txt": ((2, 32, 4096, 4096), True),
+}
+
+
+def _samples(name):
+    shape, causal = RUNS[name]
+    return costmodel.samples_from_tuning_log(os.path.join(LOGS, name), "attn", 128, 128, shape, causal)
+
+
+def test_log_lines_parse_back_into_the_configurations_that_wrote_them():
+    cfg = AttnConfig(128, 32, 128, 128, 128, 32, 2, 1, 256, True, waves_per_eu=3).set_fuse_type("register")
+    back = costmodel.config_from_log_line(repr(cfg), "attn", 128, 128)
+    assert str(back) == str(cfg) and back.waves_per_eu == 3 and back.fuse_type == "register"
+    shared = AttnConfig(64, 64, 128, 128, 128, 64, 2, 2, 256, True, 2, 4, waves_per_eu=2)
+    shared.fuse_type = "shared"
+    back = costmodel.config_from_log_line(repr(shared), "attn", 128, 128)
+    assert str(back) == str(shared) and (back.warps_mma1_n, back.warps_mma_n) == (2, 4)
+    split = AttnConfig(256, 64, 128, 128, 128, 64, 2, 2, 512, True, waves_per_eu=2, kv_splits=8).set_fuse_type("register")
+    assert costmodel.config_from_log_line(repr(split), "attn", 128, 128).kv_splits == 8
+    runs = _samples("attn_b4h32q2048k2048_c0_128_128.txt")
+    assert len(runs) > 150 and all(0.2 < ms < 5 for *_, ms in runs)
+    assert min(runs, key=lambda s: s[3])[0].Br == 256          # the recorded winner of the headline problem
+
+
+def test_fit_recovers_a_known_linear_law():
+    rng = np.random.default_rng(0)
+    truth = np.array([3e-7, 2e-7, 1e-6, 4e-7, 2e-4, 1e-2, 1e-6, 0.05])
+    cfgs = [s[0] for s in _samples("attn_b4h32q2048k2048_c0_128_128.txt")]
+    shape = (4, 32, 2048, 2048)
+    data = [(c, shape, False, float(truth @ costmodel.features(c, shape)) * (1 + 0.002 * rng.standard_normal())) for c in cfgs]
+    model = costmodel.CostModel().fit(data, ridge=1e-9)
+    pred = np.array([model.predict(c, shape) for c in cfgs])
+    want = np.array([d[3] for d in data])
+    assert np.abs(pred - want).max() <= 0.02 * want.max()
+    assert model.rank_of_best(data) <= 2
+    again = costmodel.CostModel.from_dict(model.to_dict())
+    assert again.predict(cfgs[0], shape) == model.predict(cfgs[0], shape)
+    with pytest.raises(ValueError):
+        costmodel.CostModel.from_dict({"features": ["other"], "weights": [1.0]})
+
+
+def test_model_fitted_on_one_run_keeps_the_winner_of_the_others():
+    model = costmodel.CostModel().fit(_samples("attn_b4h32q2048k2048_c0_128_128.txt"))
+    for name in RUNS:
+        runs = _samples(name)
+        times = np.array([s[3] for s in runs])
+        pred = np.array([model.predict(*s[:3]) for s in runs])
+        keep = np.argsort(pred)[:max(AttnTunner.keep_min, int(len(runs) * AttnTunner.keep_fraction + 0.999))]
+        assert model.rank_of_best(runs) < len(keep), name                  # the measured winner survives the cut
+        assert times[keep].min() == times.min(), name
+        assert np.corrcoef(pred, times)[0, 1] > 0.8, name                  # and the model follows the measurements overall
+    # the model shipped next to the tuning cache is this fit
+    shipped = costmodel.CostModel.load(os.path.join(AttnTunner(MI355X(), _meta(4, 32, 2048)).cache_path, "costmodel_attn.json"))
+    np.testing.assert_allclose(shipped.weights, model.weights, rtol=1e-6)
+
+
+def _meta(b, h, s, d=128):
+    return [torch.empty(b, h, s, d, dtype=torch.float16, device="meta") for _ in range(4)]
+
+
+def test_tuner_prunes_with_the_shipped_model_and_not_without(monkeypatch):
+    tuner = AttnTunner(MI355X(), _meta(4, 32, 2048), causal=True)
+    assert tuner.cost_model is not None
+    cfgs = [c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)]
+    kept = tuner.prune(cfgs)
+    assert len(kept) == max(tuner.keep_min, int(len(cfgs) * tuner.keep_fraction + 0.999)) and len(kept) + len(tuner.pruned) == len(cfgs)
+    winner = min(_samples("attn_b4h32q2048k2048_c1_128_128.txt"), key=lambda s: s[3])[0]
+    assert str(winner) in {str(c) for c in kept}
+    few = cfgs[:tuner.keep_min]
+    assert tuner.prune(few) == few                                          # nothing to gain on a handful
+    monkeypatch.setenv("AAT_TUNE_PRUNE", "0")
+    exhaustive = AttnTunner(MI355X(), _meta(4, 32, 2048), causal=True)
+    assert exhaustive.cost_model is None and exhaustive.prune(cfgs) == cfgs

@@ -130,8 +130,11 @@ def test_mi355x_space_is_valid_and_nonempty():
         reg = [c for c in cfgs if c.fuse_type == "register"]
         shared = [c for c in cfgs if c.fuse_type == "shared"]
         assert shared, (dqk, dv)
-        # d_v = 512 puts 256 accumulator registers on every lane of a register-fused wave: LDS-fused only
-        assert bool(reg) == (dv < 512), (dqk, dv)
+        # d_v = 512 puts 256 accumulator registers on every lane of a register-fused wave: such candidates are
+        # enumerated (the tuning loop rejects them from the compiler's resource report) but never a default
+        assert reg, (dqk, dv)
+        assert all(gfx950_space.forward_likely_spills(c) for c in reg) == (dv == 512), (dqk, dv)
+        assert gfx950_space.default_forward_config("attn", dqk, dv, arch).fuse_type == ("shared" if dv == 512 else "register")
         for c in cfgs:
             if c.fuse_type == "register":
                 assert c.Br % (32 * (c.Nthreads // 64)) == 0      # every wave owns whole 32-row groups
