@@ -84,6 +84,26 @@ class RetNetAttn(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
+_LOG2_GAMMA = {}          # (rates, device) -> log2(gamma) on the device: the rates of a model never change between calls
+
+
+def _log2_gamma(gamma, nheads, device):
+    """fp32 [H] tensor of log2(gamma_h) on ``device``.  Checking the rates and copying them to the GPU takes a
+    host round trip, so the result is kept per set of rates."""
+    values = tuple(float(g) for g in (gamma.detach().cpu().reshape(-1).tolist() if torch.is_tensor(gamma) else gamma))
+    key = (values, str(device))
+    lg = _LOG2_GAMMA.get(key)
+    if lg is None:
+        g64 = torch.tensor(values, dtype=torch.float64)
+        assert g64.numel() == nheads and bool(((g64 >= 0.5) & (g64 <= 1.0)).all()), "one decay rate in [0.5, 1] per head"
+        lg = torch.log2(g64).to(device=device, dtype=torch.float32).contiguous()
+        if len(_LOG2_GAMMA) >= 64:
+            _LOG2_GAMMA.clear()
+        _LOG2_GAMMA[key] = lg
+    assert lg.numel() == nheads, "one decay rate in [0.5, 1] per head"
+    return lg
+
+
 class RetNetDecayAttn(torch.autograd.Function):
 
     @staticmethod
@@ -95,11 +115,9 @@ class RetNetDecayAttn(torch.autograd.Function):
         batch_size, nheads, seqlen_q, key_dim = q.shape
         seqlen_k = k.shape[2]
         head_dim = v.shape[-1]
-        gamma = torch.as_tensor(gamma, dtype=torch.float64).reshape(-1)
-        assert gamma.numel() == nheads and bool(((gamma >= 0.5) & (gamma <= 1.0)).all()), "one decay rate in [0.5, 1] per head"
         assert head_dim % 64 == 0 and head_dim <= 512
         assert key_dim % 64 == 0 and key_dim <= 256
-        lg = torch.log2(gamma).to(device=q.device, dtype=torch.float32).contiguous()
+        lg = _log2_gamma(gamma, nheads, q.device)
 
         o = torch.empty(batch_size, nheads, seqlen_q, head_dim, device=q.device, dtype=torch.float16)
         r = torch.empty(batch_size, nheads, seqlen_q, device=q.device, dtype=torch.float32)

@@ -20,7 +20,14 @@ MAX_RECORDS = 3072
 
 
 def _lib():
-    return library.load_recurrent(codegen.compile_config(RetRecurrentConfig(), ARCH))
+    lib = library.load_recurrent(codegen.compile_config(RetRecurrentConfig(), ARCH))
+    # the first call on a device looks the static array up (and makes the runtime load the kernels): done here,
+    # so that the calls under test find everything in place
+    q, k, v, decay = _inputs(99, 1, 1, 64, 64, 32)
+    out = torch.empty(1, 1, 64, 32, device="cuda")
+    assert lib.retnet_recurrent_fwd_noalloc(*_ptrs(q, k, v, decay, out), 1, 1, 64, 64, 32, 64, ctypes.c_void_p(0)) == 0
+    torch.cuda.synchronize()
+    return lib
 
 
 def _inputs(seed, b, h, kdim, vdim, seqlen):
@@ -46,10 +53,11 @@ def _both(lib, q, k, v, decay, block_kdim):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     assert lib.retnet_recurrent_fwd_ex(*_ptrs(q, k, v, decay, want), *dims, ctypes.c_void_p(ws.data_ptr()), need, stream) == 0
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    free_before, _ = torch.cuda.mem_get_info()          # the driver's view: an allocation by the library would show here
     assert lib.retnet_recurrent_fwd_noalloc(*_ptrs(q, k, v, decay, got), *dims, stream) == 0
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after >= free_before, (free_before, free_after)
     return got, want
 
 
