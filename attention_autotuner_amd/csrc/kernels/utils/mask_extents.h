@@ -114,27 +114,57 @@ mask_scan_rows(const half_t* __restrict__ mask, int* __restrict__ row_lo, int* _
   }
 }
 
-// One thread per band of 32 kv positions: the query range over the tile marks of its column.
+// One block per head: the query range of every band of 32 kv positions, from the tile marks.  The marks
+// go through LDS a slab of bands at a time (read along rows, as they lie in memory; scanned along columns).
+constexpr int kMaskColSlab = 16 * 1024;             // bytes of tile marks held in LDS at a time
 __global__ void __launch_bounds__(kMaskScanThreads)
 mask_scan_cols(const unsigned char* __restrict__ occ, int* __restrict__ col_lo, int* __restrict__ col_hi, int seq_q,
                int seq_k) {
+  __shared__ unsigned char slab[kMaskColSlab];
   const int nbq = seq_q / kMaskBand, nbk = seq_k / kMaskBand;
-  const int h = blockIdx.y;
-  const int cb = blockIdx.x * kMaskScanThreads + threadIdx.x;
-  if (cb >= nbk) return;
-  int lo = 0x7fffffff, hi = 0;
-  for (int b = 0; b < nbq; ++b)
-    if (occ[((size_t)h * nbq + b) * nbk + cb]) {
-      lo = lo == 0x7fffffff ? b * kMaskBand : lo;
-      hi = (b + 1) * kMaskBand;
+  const int h = blockIdx.x;
+  const unsigned char* src = occ + (size_t)h * nbq * nbk;
+  const int bands_per_slab = kMaskColSlab / nbk < 1 ? 1 : kMaskColSlab / nbk;
+  // a thread owns the columns cb, cb + 256, ...; at most 4 of them for seq_k <= 32768 (checked by the launcher)
+  int lo[4], hi[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    lo[i] = 0x7fffffff;
+    hi[i] = 0;
+  }
+  for (int b0 = 0; b0 < nbq; b0 += bands_per_slab) {
+    const int nb = nbq - b0 < bands_per_slab ? nbq - b0 : bands_per_slab;
+    __syncthreads();
+    for (int i = threadIdx.x; i < nb * nbk; i += kMaskScanThreads) slab[i] = src[(size_t)b0 * nbk + i];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int cb = threadIdx.x + i * kMaskScanThreads;
+      if (cb < nbk) {
+#pragma unroll 8
+        for (int b = 0; b < nb; ++b) {              // selects, no branches: the LDS reads of a column overlap
+          const bool nz = slab[b * nbk + cb] != 0;
+          lo[i] = (nz && lo[i] == 0x7fffffff) ? (b0 + b) * kMaskBand : lo[i];
+          hi[i] = nz ? (b0 + b + 1) * kMaskBand : hi[i];
+        }
+      }
     }
-  col_lo[(size_t)h * nbk + cb] = lo;
-  col_hi[(size_t)h * nbk + cb] = hi;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int cb = threadIdx.x + i * kMaskScanThreads;
+    if (cb < nbk) {
+      col_lo[(size_t)h * nbk + cb] = lo[i];
+      col_hi[(size_t)h * nbk + cb] = hi[i];
+    }
+  }
 }
 
 // Enqueues the scan of mask [H, Seq_q, Seq_k] into `workspace` (mask_extent_bytes() bytes).
 inline hipError_t scan_mask(const half_t* mask, int H, int Seq_q, int Seq_k, void* workspace, hipStream_t stream) {
-  if (Seq_q % kMaskBand != 0 || Seq_k % kMaskBand != 0) return hipErrorInvalidValue;
+  if (Seq_q % kMaskBand != 0 || Seq_k % kMaskBand != 0 || Seq_k / kMaskBand > 4 * kMaskScanThreads ||
+      Seq_k / kMaskBand > kMaskColSlab)
+    return hipErrorInvalidValue;
   int* p = static_cast<int*>(workspace);
   const size_t nq = (size_t)H * (size_t)(Seq_q / kMaskBand), nk = (size_t)H * (size_t)(Seq_k / kMaskBand);
   unsigned char* occ = reinterpret_cast<unsigned char*>(p + 2 * nq + 2 * nk);
@@ -143,8 +173,7 @@ inline hipError_t scan_mask(const half_t* mask, int H, int Seq_q, int Seq_k, voi
                                                                                                Seq_q, Seq_k);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  mask_scan_cols<<<dim3((nbk + kMaskScanThreads - 1) / kMaskScanThreads, H), dim3(kMaskScanThreads), 0, stream>>>(
-      occ, p + 2 * nq, p + 2 * nq + nk, Seq_q, Seq_k);
+  mask_scan_cols<<<dim3(H), dim3(kMaskScanThreads), 0, stream>>>(occ, p + 2 * nq, p + 2 * nq + nk, Seq_q, Seq_k);
   return hipGetLastError();
 }
 
