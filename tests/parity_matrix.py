@@ -25,6 +25,12 @@ STANDALONE_BENCH_TILES = [(64, 128, 64, 256, 2), (64, 128, 32, 256, 2), (64, 64,
                           (128, 256, 64, 512, 2), (128, 128, 64, 256, 3), (128, 128, 32, 256, 3)]
 
 
+def ret_register_wide():
+    """The register-fused RetNet forward at d_qk 256, d_v 512 (the reference has this variant,
+    csrc/kernels/retnet/regfuse/regfuse.h:267-340): 256 output accumulators per lane."""
+    return RetConfig(128, 64, 256, 512, 256, 64, 1, 1, 1, 256, True, waves_per_eu=1).set_fuse_type("register")
+
+
 def parity_configs(arch=None):
     arch = arch or MI355X()
     out = []
@@ -37,6 +43,7 @@ def parity_configs(arch=None):
             cfg.fuse_type = fuse
             if gfx950_space.forward_valid(cfg, arch):
                 out.append(cfg)
+    out.append(ret_register_wide())
     for br, bc, nt, st in ATTN_BWD_TILES:
         for row_wpe in (1, 2):
             cfg = AttnBwdConfig(br, bc, 128, 128, nt, st, row_waves_per_eu=row_wpe)

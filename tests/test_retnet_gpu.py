@@ -145,6 +145,23 @@ def test_non_square_and_every_prebuilt_variant():
     assert ran >= 4
 
 
+def test_register_fused_forward_at_dqk256_dv512():
+    """The register-fused kernel holds a 32 x 512 fp32 output block per wave (all 256 accumulation registers);
+    the tuner prefers the LDS-fused kernel at this size, but the variant is built and must be right."""
+    import parity_matrix
+    cfg = parity_matrix.ret_register_wide()
+    assert gfx950_space.forward_valid(cfg, ARCH) and os.path.exists(codegen.library_path(cfg))
+    q, k, v, mask, _ = _inputs(2, 3, 256, 384, 256, 512, seed=12)
+    o_ref, r_ref = ref_op.retnet_ref(q, k, v, ref_op.retnet_decay_mask(3, 256, 384), return_r=True)
+    dev = [t.cuda() for t in (q, k, v, ref_op.retnet_decay_mask(3, 256, 384))]
+    for mode in (False, True, "scan"):
+        o = torch.zeros(2, 3, 256, 512, dtype=torch.float16, device="cuda")
+        r = torch.zeros(2, 3, 256, dtype=torch.float32, device="cuda")
+        Runtime(ARCH, cfg).apply(dev + [o, r], causal=mode)
+        tolerance.assert_close(o, o_ref, f"register-fused 256/512 walk={mode}")
+        assert ((r.cpu() - r_ref).abs() / r_ref).max().item() <= 1e-3
+
+
 def test_reference_signature_entry_points_bwd():
     q, k, v, mask, do = _inputs(1, 2, 128, 128, 64, 64, seed=7, dense_mask=True)
     _, r_ref = ref_op.retnet_ref(q, k, v, mask, return_r=True)
