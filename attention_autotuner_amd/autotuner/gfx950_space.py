@@ -304,6 +304,39 @@ def attn_backward_reg_estimate(cfg):
     return vec, acc + scores
 
 
+def attn_backward_split_reg_estimates(cfg):
+    """(dV-only column kernel, dK-only column kernel) registers per lane: resident fragments, the output
+    accumulators, the score tiles, the fp16 operand of the second contraction, addresses."""
+    rt = cfg.Br // _waves(cfg) // MFMA_M
+    nt = cfg.Bc // 32
+    dv = rt * (cfg.Kd // 16) * 4 + rt * (cfg.D // 32) * 16 + rt * nt * 16 + rt * nt * 8 + 48
+    dk = rt * ((cfg.Kd + cfg.D) // 16) * 4 + rt * (cfg.Kd // 32) * 16 + rt * nt * 32 + rt * nt * 8 + 48
+    return dv, dk
+
+
+def _one_wave_fits(rt, frag_cols, out_cols, score_tiles):
+    """One wave per SIMD: 256 vector + 256 accumulation registers.  Resident fragments, the fp16 operand and
+    addresses are vector registers; outputs are accumulation registers and the score tiles join them if there
+    is room, else they are vector registers too."""
+    vec = rt * (frag_cols // 16) * 4 + rt * 8 + 48
+    acc = rt * (out_cols // 32) * 16
+    scores = rt * score_tiles * 16
+    if acc + scores <= 256:
+        return vec <= 256 and acc <= 256
+    return vec + scores <= 256 and acc <= 256
+
+
+def _split_budget_ok(regs, rt, frag_cols, out_cols, score_tiles, wpe, nw, lds_bytes, arch):
+    """One half of a split column kernel at ``wpe`` waves per SIMD."""
+    if wpe not in (1, 2, 3) or nw > 4 * wpe:
+        return False
+    if lds_bytes * (max(1, (wpe * 4) // nw) if wpe > 1 else 1) > arch.smem_cap:
+        return False
+    if wpe == 1:
+        return _one_wave_fits(rt, frag_cols, out_cols, score_tiles)
+    return regs <= arch.register_per_thread // wpe
+
+
 def attn_backward_valid(cfg, arch):
     nw = _waves(cfg)
     if cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * nw) or cfg.Bc % 32 or cfg.Bc > 128:
@@ -315,7 +348,8 @@ def attn_backward_valid(cfg, arch):
             return False
         if (cfg.Bc * cols // 8) % cfg.Nthreads:
             return False
-    if attn_backward_lds_bytes(cfg) * blocks_per_cu(cfg) > arch.smem_cap:
+    # an occupancy target above one wave per SIMD must be reachable; at one wave per SIMD a single block per CU will do
+    if attn_backward_lds_bytes(cfg) * (blocks_per_cu(cfg) if cfg.waves_per_eu > 1 else 1) > arch.smem_cap:
         return False
     row_wpe = getattr(cfg, "row_waves_per_eu", cfg.waves_per_eu)
     row_bc = getattr(cfg, "row_Bc", cfg.Bc)
@@ -332,6 +366,16 @@ def attn_backward_valid(cfg, arch):
         row_lds = max(cfg.num_stages_qk * row_bc * (cfg.Kd + cfg.D) * 2, cfg.Br * (cfg.Kd * 2 + 16))
         if row_lds * max(1, 8 // nw) > arch.smem_cap:
             return False
+    elif cfg.waves_per_eu == 1:                              # the row kernel on the column kernel's budget
+        if not _one_wave_fits(cfg.Br // nw // MFMA_M, cfg.Kd + cfg.D, cfg.Kd, 2 * (row_bc // 32)):
+            return False
+    if getattr(cfg, "col_split", 0):
+        rt = cfg.Br // nw // MFMA_M
+        dv, dk = attn_backward_split_reg_estimates(cfg)
+        lds = attn_backward_lds_bytes(cfg)
+        return (cfg.waves_per_eu == 1 and
+                _split_budget_ok(dv, rt, cfg.Kd, cfg.D, cfg.Bc // 32, cfg.dv_waves_per_eu, nw, lds, arch) and
+                _split_budget_ok(dk, rt, cfg.Kd + cfg.D, cfg.Kd, 2 * (cfg.Bc // 32), cfg.dk_waves_per_eu, nw, lds, arch))
     vec, acc = attn_backward_reg_estimate(cfg)
     if cfg.waves_per_eu == 1:
         return vec <= 256 and acc <= 256
@@ -354,6 +398,11 @@ def attn_backward_candidates(br, bc, dim_qk, dim_v):
                 out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=wpe))
             for row_bc in (32, 64):
                 out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=1, row_waves_per_eu=2, row_Bc=row_bc))
+            # one column kernel per output, each on the largest occupancy it fits
+            for row_wpe in (1, 2):
+                for dv_wpe, dk_wpe in ((3, 2), (2, 2), (2, 1), (1, 1)):
+                    out.append(AttnBwdConfig(br, bc, dim_qk, dim_v, nthreads, stages, waves_per_eu=1, row_waves_per_eu=row_wpe,
+                                             col_split=1, dv_waves_per_eu=dv_wpe, dk_waves_per_eu=dk_wpe))
     return out
 
 
@@ -365,4 +414,11 @@ def default_attn_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
             cfg = AttnBwdConfig(br, bc, dim_qk, dim_v, nt, st, waves_per_eu=wpe, row_waves_per_eu=row_wpe)
             if attn_backward_valid(cfg, arch):
                 return cfg
+    # head sizes whose dV and dK accumulators cannot share a wave: one column kernel per output
+    for br, bc, nt, st in ((128, 32, 256, 3), (128, 32, 256, 2), (64, 32, 128, 2)):
+        if any(s and (s % br or s % bc) for s in (seq_q, seq_k)):
+            continue
+        cfg = AttnBwdConfig(br, bc, dim_qk, dim_v, nt, st, waves_per_eu=1, col_split=1)
+        if attn_backward_valid(cfg, arch):
+            return cfg
     raise NoValidConfigError(f"no default attn_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")

@@ -19,6 +19,12 @@
 // dK^T += Q^T dS, dQ^T += K^T dS) -- so each tile is fetched once and laid out with the dual swizzle.
 // Cost: S and dP are evaluated by both kernels (7 instead of 5 contractions per score).
 //
+// The column kernel can also be built for one of its two outputs (OUTS): dV alone needs neither V nor dP
+// (two contractions), dK alone needs everything but the dV accumulators (three).  Run as a pair they cost
+// one more evaluation of S, and each fits a register budget the two-output kernel does not: two waves per
+// SIMD at d = 128, and one wave per SIMD at d_qk = 256 / d_v = 512, where dV (256 accumulators per lane)
+// and dK (128) cannot share a wave at all.
+//
 // lse2 = lse * log2(e) and delta come from attn_bwd_prepare (one pass over O and dO); the COL kernel
 // copies the 2 * BY values of a streamed tile into LDS next to the tile.
 #pragma once
@@ -95,7 +101,8 @@ __global__ void __launch_bounds__(256) attn_bwd_prepare(const half_t* __restrict
 // x1, x2: resident-side matrices (COL: k, v; ROW: q, dO); y1, y2: streamed-side matrices (COL: q, dO;
 // ROW: k, v); all [B*H, S, width] fp16.  lse2, delta: [B*H, seq_q] fp32.  COL writes out1 = dV and
 // out2 = dK; ROW writes out2 = dQ.  c2 = softmax_scale * log2(e); out_scale = softmax_scale.
-template <int Kd, int D, int BX, int BY, int Nthreads, int NS, AttnBwdPass PASS, int WPE = 1>
+// OUTS (COL only): 3 = both outputs, 1 = dV only (x2, delta and out2 are not touched), 2 = dK only.
+template <int Kd, int D, int BX, int BY, int Nthreads, int NS, AttnBwdPass PASS, int WPE = 1, int OUTS = 3>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, const half_t* __restrict__ y1,
                const half_t* __restrict__ y2, const float* __restrict__ lse2, const float* __restrict__ delta,
@@ -106,6 +113,9 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
                 WM = T::WM;
   constexpr int PF = AAT_PF;
   constexpr bool COL = T::COL;
+  static_assert(COL ? (OUTS >= 1 && OUTS <= 3) : OUTS == 3, "output selection is a column-kernel option");
+  constexpr bool kOut1 = COL && (OUTS & 1);       // dV
+  constexpr bool kOut2 = !COL || (OUTS & 2);      // dK or dQ: needs dP and with it X2, delta
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x;
@@ -148,9 +158,9 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
   const int wave_base = wave * 64;
 
   // resident operands: this lane's row of X1 (width Kd) and of X2 (width D) as MFMA B fragments
-  h8 x1f[RT][KS], x2f[RT][DS];
+  h8 x1f[RT][KS], x2f[RT][kOut2 ? DS : 1];
   load_q_frags<RT, KS, Kd>(x1f, x1 + ((size_t)bh * seq_x + x0 + wave * WM + n) * Kd + 8 * h);
-  load_q_frags<RT, DS, D>(x2f, x2 + ((size_t)bh * seq_x + x0 + wave * WM + n) * D + 8 * h);
+  if constexpr (kOut2) load_q_frags<RT, DS, D>(x2f, x2 + ((size_t)bh * seq_x + x0 + wave * WM + n) * D + 8 * h);
 
   // LDS addresses inside stage 0: first-contraction fragments (rows n, chunk 2ks+h) and transposing reads
   uint32_t y1addr[KS], y2addr[DS], z1lo[KT], z1hi[KT], z2lo[DT], z2hi[DT];
@@ -191,13 +201,13 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
   }
 
   // accumulators: acc1 = dV^T (COL only, D wide), acc2 = dK^T (COL) or dQ^T (ROW), Kd wide
-  f16v acc1[RT][COL ? DT : 1], acc2[RT][KT];
+  f16v acc1[RT][kOut1 ? DT : 1], acc2[RT][kOut2 ? KT : 1];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-    for (int i = 0; i < (COL ? DT : 1); ++i) acc1[rt][i] = zero16();
+    for (int i = 0; i < (kOut1 ? DT : 1); ++i) acc1[rt][i] = zero16();
 #pragma unroll
-    for (int i = 0; i < KT; ++i) acc2[rt][i] = zero16();
+    for (int i = 0; i < (kOut2 ? KT : 1); ++i) acc2[rt][i] = zero16();
   }
 
   auto issue = [&](int j, int st) {
@@ -231,16 +241,18 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
       // one wave per SIMD: outputs in the accumulation registers, resident fragments in vector registers
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
-        if constexpr (COL) {
+        if constexpr (kOut1) {
 #pragma unroll
           for (int i = 0; i < DT; ++i) asm volatile("" : "+a"(acc1[rt][i]));
         }
+        if constexpr (kOut2) {
 #pragma unroll
-        for (int i = 0; i < KT; ++i) asm volatile("" : "+a"(acc2[rt][i]));
+          for (int i = 0; i < KT; ++i) asm volatile("" : "+a"(acc2[rt][i]));
+#pragma unroll
+          for (int i = 0; i < DS; ++i) asm volatile("" : "+v"(x2f[rt][i]));
+        }
 #pragma unroll
         for (int i = 0; i < KS; ++i) asm volatile("" : "+v"(x1f[rt][i]));
-#pragma unroll
-        for (int i = 0; i < DS; ++i) asm volatile("" : "+v"(x2f[rt][i]));
       }
     }
     // tile j has landed (with three buffers tile j+1 may still be in flight); every wave is past tile j-1
@@ -259,10 +271,10 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
 
     // first contractions: s = Y1 X1^T (scores), p = Y2 X2^T (dP), both transposed (lane owns resident row)
     // the score tiles accumulate in vector registers when the outputs alone fill the accumulation registers
-    constexpr bool kVacc = WPE == 1 && RT * ((COL ? DT : 0) + KT + 2 * NT) * 16 > 256;
-    f16v s[RT][NT], dp[RT][NT];
+    constexpr bool kVacc = WPE == 1 && RT * ((kOut1 ? DT : 0) + (kOut2 ? KT + NT : 0) + NT) * 16 > 256;
+    f16v s[RT][NT], dp[RT][kOut2 ? NT : 1];
     qk_gemm_steps<RT, NT, KS, NCK, PF, kVacc>(s, x1f, y1addr, off, [](int) {});
-    qk_gemm_steps<RT, NT, DS, NCD, PF, kVacc>(dp, x2f, y2addr, off, [](int) {});
+    if constexpr (kOut2) qk_gemm_steps<RT, NT, DS, NCD, PF, kVacc>(dp, x2f, y2addr, off, [](int) {});
 
     // P = exp2(s*c2 - lse2[q]),  dS = P * (dP - delta[q]);  register v of tile t is streamed row 32t + 8(v/4) + 4h + v%4.
     // Only a tile the diagonal crosses runs the masking code.  COL: the statistics of the streamed rows come
@@ -276,18 +288,21 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
       auto read_stats = [&](auto it) {
         constexpr int i = decltype(it)::value, tg = i % (NT * 4);    // the statistics do not depend on rt
         l2r[i % 2] = lds_read_f4_async(stat_addr, off + (32 * (tg / 4) + 8 * (tg % 4)) * 4);
-        dlr[i % 2] = lds_read_f4_async(stat_addr, off + (BY + 32 * (tg / 4) + 8 * (tg % 4)) * 4);
+        if constexpr (kOut2) dlr[i % 2] = lds_read_f4_async(stat_addr, off + (BY + 32 * (tg / 4) + 8 * (tg % 4)) * 4);
       };
       if constexpr (COL) read_stats(std::integral_constant<int, 0>{});
       static_for<G>([&](auto it) {
         constexpr int i = decltype(it)::value, rt = i / (NT * 4), t = (i / 4) % NT, g = i % 4;
-        f4v l2 = l2r[i % 2], dl = dlr[i % 2];
+        f4v l2 = l2r[i % 2], dl = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (kOut2) dl = dlr[i % 2];
         if constexpr (COL) {
           if constexpr (i + 1 < G) {
             read_stats(std::integral_constant<int, i + 1>{});
-            lds_wait_younger<2>(l2, dl);
+            if constexpr (kOut2) lds_wait_younger<2>(l2, dl);
+            else lds_wait_younger<1>(l2);
           } else {
-            lds_wait_younger<0>(l2, dl);
+            if constexpr (kOut2) lds_wait_younger<0>(l2, dl);
+            else lds_wait_younger<0>(l2);
           }
         }
         // The score of resident row x and streamed row y = j*BY + c + 4h (c = 32t + 8g + e, a constant) is masked
@@ -299,13 +314,15 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
           constexpr int vbase = 4 * g, cbase = 32 * t + 8 * g;
           const int v = vbase + e;
           const float lrow = COL ? l2[e] : lse_row[rt];
-          const float drow = COL ? dl[e] : delta_row[rt];
           float p = fast_exp2(s[rt][t][v] * c2 - lrow);
           if constexpr (MASKED) {
             if (COL ? lim > cbase + e : cbase + e > lim) p = 0.f;
           }
           s[rt][t][v] = p;
-          dp[rt][t][v] = p * (dp[rt][t][v] - drow);
+          if constexpr (kOut2) {
+            const float drow = COL ? dl[e] : delta_row[rt];
+            dp[rt][t][v] = p * (dp[rt][t][v] - drow);
+          }
         }
       });
     };
@@ -314,16 +331,18 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
 
     // second contractions: COL  dV^T += dO^T P  and  dK^T += Q^T dS;   ROW  dQ^T += K^T dS
     h8 ef[RT][NT][2];
-    if constexpr (COL) {
+    if constexpr (kOut1) {
       pv_gemm_steps_hl<RT, NT, DT, NCD, PF>(acc1, ef, z2lo, z2hi, off, [&](int g) {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) ef[rt][g >> 1][g & 1] = pack8_rne(s[rt][g >> 1], 8 * (g & 1));
       });
     }
-    pv_gemm_steps_hl<RT, NT, KT, NCK, PF>(acc2, ef, z1lo, z1hi, off, [&](int g) {
+    if constexpr (kOut2) {
+      pv_gemm_steps_hl<RT, NT, KT, NCK, PF>(acc2, ef, z1lo, z1hi, off, [&](int g) {
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) ef[rt][g >> 1][g & 1] = pack8_rne(dp[rt][g >> 1], 8 * (g & 1));
-    });
+        for (int rt = 0; rt < RT; ++rt) ef[rt][g >> 1][g & 1] = pack8_rne(dp[rt][g >> 1], 8 * (g & 1));
+      });
+    }
   };
   for (int j = j_begin; j < j_end; j += NS) {
     static_for<NS>([&](auto k_tag) {
@@ -363,8 +382,8 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
     }
     wait_lgkm0();                                           // the staging rows are reused by the next output
   };
-  if constexpr (COL) store(acc1, std::integral_constant<int, D>{}, out1, 1.0f);
-  store(acc2, std::integral_constant<int, Kd>{}, out2, out_scale);
+  if constexpr (kOut1) store(acc1, std::integral_constant<int, D>{}, out1, 1.0f);
+  if constexpr (kOut2) store(acc2, std::integral_constant<int, Kd>{}, out2, out_scale);
 }
 
 }  // namespace aat

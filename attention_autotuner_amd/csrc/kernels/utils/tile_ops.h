@@ -102,6 +102,10 @@ AAT_DEV f4v lds_read_f4_async(uint32_t base, int imm) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(base + hi), "i"(imm & 0xffff));
   return v;
 }
+template <int N> AAT_DEV void lds_wait_younger(f4v& a) {
+  static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(a) : "n"(N));
+}
 template <int N> AAT_DEV void lds_wait_younger(f4v& a, f4v& b) {
   static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));

@@ -11,7 +11,9 @@ reference uses as its own correctness check:
 * ``attention_bwd_ref`` is the closed form of the attention gradients (the reference declares the
   operator, python/ops/attention_interface.py:37-58, and leaves it empty): with ``P = softmax(S)``,
   ``delta = rowsum(dO * O)``: ``dV = P^T dO``, ``dS = P * (dO V^T - delta)``, ``dK = scale dS^T Q``,
-  ``dQ = scale dS K``; pinned by autograd through ``attention_ref`` and fp64 gradcheck.
+  ``dQ = scale dS K``; pinned by autograd through ``attention_ref`` and fp64 gradcheck.  With
+  ``operand_dtype=torch.float16`` P and dS are rounded before the contraction that consumes them, as the kernels
+  do; ``attention_bwd_rounding_bound`` is the worst case that rounding can move each gradient entry by.
 * ``retnet_ref``      follows reference python/utils/ref_op.py:8-13 (``S = q k^T * mask``,
   ``r = clamp(sum|S|, min=1)`` detached, ``o = (S / r) v``) and also returns ``r``.
 * ``retnet_bwd_ref``  is the closed form the backward kernel evaluates, reference
@@ -66,9 +68,7 @@ def attention_ref(q, k, v, softmax_scale=None, causal=False, return_lse=False):
     return (o, lse) if return_lse else o
 
 
-def attention_bwd_ref(q, k, v, do, softmax_scale=None, causal=False, o=None, lse=None):
-    """Gradients of ``attention_ref`` w.r.t. q, k, v.  ``o`` / ``lse`` (as a forward kernel stored them) are
-    used for delta and P when given, otherwise recomputed."""
+def _attention_bwd_parts(q, k, v, do, softmax_scale, causal, o, lse, operand_dtype=None):
     q, k, v, do = _f32(q), _f32(k), _f32(v), _f32(do)
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(q.shape[-1])
@@ -78,12 +78,42 @@ def attention_bwd_ref(q, k, v, do, softmax_scale=None, causal=False, o=None, lse
     lse = torch.logsumexp(s, dim=-1) if lse is None else _f32(lse)
     p = torch.nan_to_num(torch.exp(s - lse.unsqueeze(-1)), nan=0.0, posinf=0.0)
     o = p @ v if o is None else _f32(o)
+    if operand_dtype is not None:
+        o = o.to(operand_dtype).float()                     # delta is taken from the output as the forward stored it
     delta = (do * o).sum(dim=-1, keepdim=True)
-    dv = p.transpose(-1, -2) @ do
     ds = p * (do @ v.transpose(-1, -2) - delta)
+    return q, k, v, do, softmax_scale, p, ds, o
+
+
+def attention_bwd_ref(q, k, v, do, softmax_scale=None, causal=False, o=None, lse=None, operand_dtype=None):
+    """Gradients of ``attention_ref`` w.r.t. q, k, v.  ``o`` / ``lse`` (as a forward kernel stored them) are
+    used for delta and P when given, otherwise recomputed.  ``operand_dtype=torch.float16`` restates the
+    kernels' arithmetic: delta from the fp16 output, P and dS rounded before the contraction that consumes
+    them (the roundings of the reference's RetNet backward, csrc/kernels/retnet/bwd/bwd_colblock.h:509,551;
+    the reference has no attention backward)."""
+    q, k, v, do, softmax_scale, p, ds, _ = _attention_bwd_parts(q, k, v, do, softmax_scale, causal, o, lse, operand_dtype)
+    if operand_dtype is not None:
+        p, ds = p.to(operand_dtype).float(), ds.to(operand_dtype).float()
+    dv = p.transpose(-1, -2) @ do
     dk = (ds.transpose(-1, -2) @ q) * softmax_scale
     dq = (ds @ k) * softmax_scale
     return dq, dk, dv
+
+
+def attention_bwd_rounding_bound(q, k, v, do, softmax_scale=None, causal=False, o_stored=None):
+    """Per-entry sums of term magnitudes for dq, dk, dv: the fp16 roundings of the kernels' arithmetic (P, dS,
+    and the output that delta is taken from) move a gradient entry by at most 2^-11 times its sum.  An error e_i
+    in delta_i moves every dS_ij of the row by P_ij e_i; with the exact output rounded to fp16 e_i is at most
+    2^-11 sum_d |dO_id O_id|, with ``o_stored`` (the output a forward kernel actually wrote) it is the actual
+    difference |sum_d dO_id (o_stored - O)_id|, entered here divided by 2^-11."""
+    q, k, v, do, softmax_scale, p, ds, o = _attention_bwd_parts(q, k, v, do, softmax_scale, causal, None, None)
+    p = p.abs()
+    if o_stored is None:
+        delta_dev = (do * o).abs().sum(dim=-1, keepdim=True)
+    else:
+        delta_dev = (do * (_f32(o_stored) - o)).sum(dim=-1, keepdim=True).abs() * 2.0 ** 11
+    ds = ds.abs() + p * delta_dev
+    return (ds @ k.abs()) * softmax_scale, (ds.transpose(-1, -2) @ q.abs()) * softmax_scale, p.transpose(-1, -2) @ do.abs()
 
 
 def retnet_ref(q, k, v, mask, return_r=False):

@@ -10,13 +10,13 @@ in the last place of the reference above (``check`` with its defaults):
     |ref| <  4 :  |err| <= 2e-3
     |ref| >= 4 :  |err| <= ulp_fp16(ref) = 2^(floor(log2 |ref|) - 10)
 
-Every forward output and every attention gradient is held to this rule against the exact fp32 form, and every
-RetNet gradient against the oracle's restatement of the reference kernel's arithmetic (P and dS rounded to
-fp16 before the contraction that consumes them, ``retnet_bwd_ref(..., operand_dtype=torch.float16)``).
+Every forward output is held to this rule against the exact fp32 form, and every gradient against the oracle's
+restatement of the reference kernel's arithmetic (P and dS rounded to fp16 before the contraction that
+consumes them, ``retnet_bwd_ref`` / ``attention_bwd_ref`` with ``operand_dtype=torch.float16``).
 
-Against the *exact* fp32 form a RetNet gradient carries that operand rounding as well: each P or dS entry moves
+Against the *exact* fp32 form a gradient carries that operand rounding as well: each P or dS entry moves
 by up to 2^-11 of its magnitude, so a gradient entry moves by up to 2^-11 * T with T the sum of the magnitudes
-of its terms (``ref_op.retnet_bwd_rounding_bound``).  Where a row of the mask lets one or two kv positions
+of its terms (``ref_op.retnet_bwd_rounding_bound``, ``ref_op.attention_bwd_rounding_bound``).  Where a row of the mask lets one or two kv positions
 through (the first rows of a causal or decay mask) nothing averages that out and the entries are O(1): an entry
 near 4 moves by 2e-3 before its own rounding to fp16 adds another 1e-3.  The reference's kernel rounds at the
 same two points, so this is the accuracy of the operator as published, not of this implementation.

@@ -16,8 +16,16 @@ PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
 SHARED_TILES = [(128, 64, 256, 2, 2, 1, 4, 2), (64, 64, 256, 1, 1, 2, 4, 2), (64, 64, 256, 2, 1, 2, 2, 2), (64, 64, 256, 1, 1, 2, 4, 1)]
 SHARED_DIMS = [(64, 64), (128, 128), (256, 512)]
 # attention backward: head-size pairs run at their defaults, and (Br, Bc, Nthreads, buffers) variants at 128/128
-ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (256, 128), (256, 256)]
+ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (256, 128), (256, 256), (256, 512)]
 ATTN_BWD_TILES = [(64, 32, 128, 2), (64, 64, 128, 2), (128, 64, 256, 3), (128, 32, 256, 2)]
+# ... and with one column kernel per output: (Br, Bc, Nthreads, buffers, row waves/SIMD, row Bc, dV waves/SIMD, dK waves/SIMD)
+ATTN_BWD_SPLIT_TILES = [(128, 32, 256, 2, 2, 32, 2, 2), (128, 64, 256, 2, 2, 32, 2, 1), (128, 32, 256, 3, 2, 32, 3, 2),
+                        (64, 32, 128, 2, 1, 32, 1, 1)]
+
+
+def attn_bwd_split_config(br, bc, nt, st, row_wpe, row_bc, dv_wpe, dk_wpe, dqk=128, dv=128):
+    return AttnBwdConfig(br, bc, dqk, dv, nt, st, waves_per_eu=1, row_waves_per_eu=row_wpe, row_Bc=row_bc, col_split=1,
+                         dv_waves_per_eu=dv_wpe, dk_waves_per_eu=dk_wpe)
 # kv-splitting variants: (d_qk, d_v, splits)
 SPLIT_VARIANTS = [(128, 128, 4), (128, 128, 8), (64, 64, 2)]
 # register-fused configurations the stand-alone attention benchmark times (csrc/benchmarks/attention.hip): (d, Br, Bc, threads, waves/SIMD)
@@ -44,6 +52,8 @@ def parity_configs(arch=None):
             if gfx950_space.forward_valid(cfg, arch):
                 out.append(cfg)
     out.append(ret_register_wide())
+    out += [attn_bwd_split_config(*t) for t in ATTN_BWD_SPLIT_TILES]
+    out.append(AttnBwdConfig(64, 64, 128, 128, 128, 2, row_waves_per_eu=2, row_Bc=32))      # row kernel with a tile height of its own
     for br, bc, nt, st in ATTN_BWD_TILES:
         for row_wpe in (1, 2):
             cfg = AttnBwdConfig(br, bc, 128, 128, nt, st, row_waves_per_eu=row_wpe)

@@ -1,11 +1,12 @@
 """GPU parity of the attention backward (dq, dk, dv) against the CPU oracle, through the operator and
 through the C ABI.
 
-Tolerance (oracle/tolerance.py): max |err| <= 2e-3 on fp16 gradients versus the fp32 oracle on the same
+Tolerance (oracle/tolerance.py; gradients are checked twice, see _grads_close): max |err| <= 2e-3 on fp16 gradients versus the fp32 oracle on the same
 seeded inputs wherever |ref| < 4, one fp16 unit in the last place of the reference above; the forward's
 log-sum-exp is compared at 1e-3 absolute.
 """
 import ctypes
+import os
 import math
 
 import pytest
@@ -37,6 +38,18 @@ def _close(got, ref):
     return ok, (worst_small, worst_large)
 
 
+def _grads_close(what, grads, q, k, v, do, scale, causal, o=None):
+    """dq, dk, dv held to the literal rule against the kernels' arithmetic (delta from the fp16 output the
+    forward stored -- ``o`` when the operator's own forward wrote it -- and P, dS rounded to fp16 before the
+    dependent contraction) and, against the exact fp32 form, to what those roundings can do in the worst case."""
+    as_kernel = ref_op.attention_bwd_ref(q, k, v, do, scale, causal, o=o, operand_dtype=torch.float16)
+    exact = ref_op.attention_bwd_ref(q, k, v, do, scale, causal)
+    terms = ref_op.attention_bwd_rounding_bound(q, k, v, do, scale, causal, o_stored=o)
+    for name, g, wk, we, t in zip(("dq", "dk", "dv"), grads, as_kernel, exact, terms):
+        tolerance.assert_close(g, wk, f"{what} {name} vs fp16-operand form")
+        tolerance.assert_close_rounded_operand(g, we, t, f"{what} {name} vs exact fp32 form")
+
+
 def _op_grads(q, k, v, do, causal, scale=None):
     qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
     o = aat.flash_attn_func(qc, kc, vc, ARCH, causal, scale)
@@ -50,10 +63,7 @@ def _op_grads(q, k, v, do, causal, scale=None):
 def test_operator_backward_matches_oracle(dqk, dv, sq, sk, causal):
     q, k, v, do = _inputs(2, 3, sq, sk, dqk, dv, seed=sq + dqk)
     o, dq, dk, dv_ = _op_grads(q, k, v, do, causal)
-    ref = ref_op.attention_bwd_ref(q, k, v, do, None, causal)
-    for name, g, r in zip(("dq", "dk", "dv"), (dq, dk, dv_), ref):
-        ok, worst = _close(g, r)
-        assert ok, (name, worst)
+    _grads_close(f"{dqk}/{dv} {sq}x{sk} causal={causal}", (dq, dk, dv_), q, k, v, do, None, causal, o=o.detach())
 
 
 def test_forward_lse_entry_matches_oracle():
@@ -74,10 +84,7 @@ def test_config2_backward_b4_h32_s2048_d128(causal):
     o, dq, dk, dv_ = _op_grads(q, k, v, do, causal)
     for b, h in ((0, 0), (2, 17), (3, 31)):          # (batch, head) slices are independent
         sl = (slice(b, b + 1), slice(h, h + 1))
-        ref = ref_op.attention_bwd_ref(q[sl], k[sl], v[sl], do[sl], None, causal)
-        for name, g, r in zip(("dq", "dk", "dv"), (dq[sl], dk[sl], dv_[sl]), ref):
-            ok, worst = _close(g, r)
-            assert ok, (name, b, h, worst)
+        _grads_close(f"config 2 ({b},{h}) causal={causal}", (dq[sl], dk[sl], dv_[sl]), q[sl], k[sl], v[sl], do[sl], None, causal, o=o[sl].detach())
     # size-independent properties on the whole problem: rows of dS sum to zero, so with K := 1 dQ vanishes;
     # and the gradients are linear in dO
     ones = torch.ones_like(k)
@@ -103,10 +110,7 @@ def test_tile_variants_agree(br, bc, nt, st, row_wpe):
     arrays = [t.cuda() for t in (q, k, v, o_ref.half(), do, lse_ref)]
     grads = [torch.empty_like(arrays[0]), torch.empty_like(arrays[1]), torch.empty_like(arrays[2])]
     Runtime(ARCH, cfg).apply(arrays + grads, softmax_scale=0.11, causal=True)
-    ref = ref_op.attention_bwd_ref(q, k, v, do, 0.11, True)
-    for name, g, r in zip(("dq", "dk", "dv"), grads, ref):
-        ok, worst = _close(g, r)
-        assert ok, (cfg, name, worst)
+    _grads_close(str(cfg), grads, q, k, v, do, 0.11, True)
 
 
 def test_row_kernel_with_its_own_tile_height():
@@ -118,10 +122,7 @@ def test_row_kernel_with_its_own_tile_height():
     arrays = [t.cuda() for t in (q, k, v, o_ref.half(), do, lse_ref)]
     grads = [torch.empty_like(arrays[0]), torch.empty_like(arrays[1]), torch.empty_like(arrays[2])]
     Runtime(ARCH, cfg).apply(arrays + grads, softmax_scale=0.11, causal=True)
-    ref = ref_op.attention_bwd_ref(q, k, v, do, 0.11, True)
-    for name, g, r in zip(("dq", "dk", "dv"), grads, ref):
-        ok, worst = _close(g, r)
-        assert ok, (cfg, name, worst)
+    _grads_close(str(cfg), grads, q, k, v, do, 0.11, True)
 
 
 def test_abi_error_paths_and_stream():
@@ -148,8 +149,29 @@ def test_abi_error_paths_and_stream():
 
 
 def test_unsupported_head_sizes_say_so():
-    q, k, v, do = _inputs(1, 1, 128, 128, 256, 512, seed=9)
+    """192-wide rows have no dual swizzle (64 or multiples of 128): the forward runs, the backward says so."""
+    q, k, v, do = _inputs(1, 1, 128, 128, 192, 192, seed=9)
     qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
     o = aat.flash_attn_func(qc, kc, vc, ARCH)
     with pytest.raises(NotImplementedError):
         o.backward(do.cuda())
+
+
+@pytest.mark.parametrize("tile", parity_matrix.ATTN_BWD_SPLIT_TILES)
+def test_one_column_kernel_per_output_agrees(tile):
+    """dV and dK from separate column kernels (each on its own register budget), against the oracle and, bit for
+    bit, against the two-output kernel of the same tile shape (same arithmetic in the same order)."""
+    q, k, v, do = _inputs(1, 2, 256, 384, 128, 128, seed=15)
+    cfg = parity_matrix.attn_bwd_split_config(*tile)
+    assert gfx950_space.attn_backward_valid(cfg, ARCH), cfg
+    for causal in (False, True):
+        o_ref, lse_ref = ref_op.attention_ref(q, k, v, 0.09, causal, return_lse=True)
+        arrays = [t.cuda() for t in (q, k, v, o_ref.half(), do, lse_ref)]
+        grads = [torch.empty_like(arrays[0]), torch.empty_like(arrays[1]), torch.empty_like(arrays[2])]
+        Runtime(ARCH, cfg).apply(arrays + grads, softmax_scale=0.09, causal=causal)
+        _grads_close(f"{cfg} causal={causal}", grads, q, k, v, do, 0.09, causal)
+        whole = AttnBwdConfig(cfg.Br, cfg.Bc, 128, 128, cfg.Nthreads, cfg.num_stages_qk)
+        if gfx950_space.attn_backward_valid(whole, ARCH) and os.path.exists(codegen.library_path(whole)):
+            both = [torch.empty_like(g) for g in grads]
+            Runtime(ARCH, whole).apply(arrays + both, softmax_scale=0.09, causal=causal)
+            assert torch.equal(both[1], grads[1]) and torch.equal(both[2], grads[2]), (cfg, causal)

@@ -218,6 +218,28 @@ def test_retnet_bwd_rounded_operands_stay_within_the_rounding_bound():
     assert dq[0, 0, 3, 0] == 4.0 and dk[0, 0, 3, 0] == 2.0 and dv[0, 0, 3, 1] == 16.0
 
 
+def test_attention_bwd_rounded_operands_stay_within_the_rounding_bound():
+    q, k, v, do = _rand(1, 2, 24, 64, seed=61), _rand(1, 2, 40, 64, seed=62), _rand(1, 2, 40, 128, seed=63), _rand(1, 2, 24, 128, seed=64)
+    for causal in (False, True):
+        exact = ref_op.attention_bwd_ref(q, k, v, do, 0.2, causal)
+        rounded = ref_op.attention_bwd_ref(q, k, v, do, 0.2, causal, operand_dtype=torch.float16)
+        bounds = ref_op.attention_bwd_rounding_bound(q, k, v, do, 0.2, causal)
+        stored = ref_op.attention_ref(q, k, v, 0.2, causal).half()           # the same bound from the actual difference in delta
+        tight = ref_op.attention_bwd_rounding_bound(q, k, v, do, 0.2, causal, o_stored=stored)
+        assert all((t <= b * 1.001 + 1e-6).all() for t, b in zip(tight, bounds))
+        differs = False
+        for e, g, b in zip(exact, rounded, bounds):
+            assert ((e - g).abs() <= 2.0 ** -11 * b * 1.001 + 1e-7).all()
+            differs |= bool((e != g).any())
+        assert differs
+    # one visible key per query: P = 1 exactly, so dV = dO; dS = dO.v - dO.o vanishes up to the rounding of o
+    one = [t[..., :1, :] for t in (q, k, v, do)]
+    dq, dk, dv = ref_op.attention_bwd_ref(*one, 0.2, True)
+    assert torch.equal(dv, one[3].float()) and dq.abs().max() <= 1e-5 and dk.abs().max() <= 1e-5
+    dq16, _, dv16 = ref_op.attention_bwd_ref(*one, 0.2, True, operand_dtype=torch.float16)
+    assert torch.equal(dv16, one[3].float()) and dq16.abs().max() <= 2.0 ** -11 * (one[3].float().abs() * one[2].float().abs()).sum() * 0.2 * one[1].abs().max() * 1.01
+
+
 # ------------------------------------------------------------------------------------ the parity bound
 def test_tolerance_rule_accepts_and_rejects_what_it_says():
     from oracle import tolerance
