@@ -34,7 +34,7 @@
 #include "../../utils/tile_ops.h"
 
 #ifndef AAT_PF
-#define AAT_PF 2
+#define AAT_PF 4
 #endif
 
 namespace aat {
@@ -247,20 +247,38 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
       wait_vmcnt<0>();
     }
     block_sync();
-    if constexpr (NSZ == 1) issue_z(j, 0);
-    if (more) {
-      if constexpr (NSZ == 2) issue_z(j + 1, zs1);
-      if constexpr (NSY == 2) issue_ym(j + 1, ys1);
-    }
-    if constexpr (NSY == 3) {
-      if (j + 2 < j_end) issue_ym(j + 2, ys2);
-    }
+    // The copies this tile starts -- Z_j (one Z buffer) or Z_{j+1} (two), then Y/mask_{j+1} (two Y buffers) or
+    // Y/mask_{j+2} (three) -- go out one LDS-DMA instruction per step of the first contraction: issued in a
+    // burst each of them holds the only wave of the SIMD for 100 cycles and more, between matrix
+    // instructions for about half of that.  The order (Z before Y/mask) is the one the waits above count on.
+    constexpr int kZi = T::ZDma::kIters, kYi = T::YDma::kIters, kMi = DECAY ? 0 : T::MDma::kIters;
+    const bool z_now = NSZ == 1 || more;
+    const bool ym_now = NSY == 3 ? (j + 2 < j_end) : (NSY == 2 && more);
+    const int zj = NSZ == 1 ? j : j + 1, yj = NSY == 3 ? j + 2 : j + 1;
+    constexpr int zslot = NSZ == 1 ? 0 : zs1, yslot = NSY == 3 ? ys2 : ys1;
+    const char* const zsrc = zg + (size_t)zj * BY * DZ * 2;
+    const char* const ysrc = yg + (size_t)yj * T::kYBytes;
+    const char* const msrc = DECAY ? nullptr : (COL ? mg + (size_t)yj * BY * seq_k * 2 : mg + (size_t)yj * BY * 2);
+    auto issue_nth = [&](int i) {
+      if (i < kZi) {
+        if (z_now) zdma.issue_one(i, zsrc, zbuf + zslot * T::kZBytes, wave_base);
+      } else if (i < kZi + kYi) {
+        if (NSY > 1 && ym_now) ydma.issue_one(i - kZi, ysrc, ybuf + yslot * T::kYBytes, wave_base);
+      } else if (i < kZi + kYi + kMi) {
+        if constexpr (!DECAY) {
+          if (NSY > 1 && ym_now) mdma.issue_one(i - kZi - kYi, msrc, mbuf + yslot * T::kMBytes, wave_base);
+        }
+      }
+    };
     constexpr int yoff = ys * T::kYBytes, moff = ys * T::kMBytes, zoff = zs * T::kZBytes;
 
     f16v tacc[RT][NT];
     // the score tile accumulates in vector registers when the outputs fill the accumulation registers
     constexpr bool kVacc = WPE == 1 && RT * (DT + NT) * 16 > 256;
-    qk_gemm_steps<RT, NT, KS, NCY, PF, kVacc>(tacc, xf, yaddr, yoff, [](int) {});
+    qk_gemm_steps<RT, NT, KS, NCY, PF, kVacc>(tacc, xf, yaddr, yoff, [&](int step) { issue_nth(step); });
+    static_for<(kZi + kYi + kMi > NT * KS ? kZi + kYi + kMi - NT * KS : 0)>([&](auto t) {
+      issue_nth(NT * KS + decltype(t)::value);      // more copies than steps: the rest in one go
+    });
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       if constexpr (DECAY) {

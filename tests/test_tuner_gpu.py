@@ -80,3 +80,29 @@ def test_backward_libraries_pass_the_guard(op, cls, dims):
     idx = next(iter(tuner._reference))
     tuner._reference[idx] = tuner._reference[idx] + 1.0
     assert not tuner.verify(codegen.compile_config(cfg, ARCH))
+
+
+def test_a_library_that_is_not_built_is_compiled_on_this_machine_and_runs(tmp_path, monkeypatch):
+    """The path a first call takes without prebuilt libraries: hipcc on the GPU box itself (one small
+    configuration, into a scratch build directory), then the launch, checked against the oracle; and with
+    compiling switched off the same miss is an error that names the library."""
+    from attention_autotuner_amd.autotuner import Runtime
+    from attention_autotuner_amd.autotuner.runtime import KernelLaunchError
+    from oracle import ref_op
+    cfg = AttnConfig(64, 32, 64, 64, 64, 32, 1, 1, 128, True, waves_per_eu=1).set_fuse_type("register")
+    assert gfx950_space.forward_valid(cfg, ARCH)
+    build = str(tmp_path / "build")
+    monkeypatch.setenv("AAT_NO_JIT", "1")
+    with pytest.raises(codegen.MissingLibraryError, match="AAT_NO_JIT"):
+        Runtime(ARCH, cfg, tmp_dir=build)
+    monkeypatch.setenv("AAT_NO_JIT", "0")
+    rt = Runtime(ARCH, cfg, tmp_dir=build)                     # compiles here
+    assert rt._path().startswith(build) and os.path.exists(rt._path())
+    usage = codegen.resource_usage(rt._path())
+    assert usage and not codegen.spilling_kernels(usage)
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(1, 2, 128, 64, generator=g).half() for _ in range(3))
+    o = torch.zeros(1, 2, 128, 64, dtype=torch.float16, device="cuda")
+    for causal in (False, True):
+        rt.apply([q.cuda(), k.cuda(), v.cuda(), o], causal=causal)
+        assert (o.float().cpu() - ref_op.attention_ref(q, k, v, None, causal)).abs().max().item() <= 2e-3
