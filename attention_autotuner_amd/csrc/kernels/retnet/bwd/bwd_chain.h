@@ -275,7 +275,22 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
     f16v tacc[RT][NT];
     // the score tile accumulates in vector registers when the outputs fill the accumulation registers
     constexpr bool kVacc = WPE == 1 && RT * (DT + NT) * 16 > 256;
-    qk_gemm_steps<RT, NT, KS, NCY, PF, kVacc>(tacc, xf, yaddr, yoff, [&](int step) { issue_nth(step); });
+    // COL: r of this tile's query rows turns into 1/r here, a reciprocal per step, in the shadow of the matrix
+    // instructions (16 of them in a row cost 140 cycles in front of the element-wise step)
+    qk_gemm_steps<RT, NT, KS, NCY, PF, kVacc>(tacc, xf, yaddr, yoff, [&](int step) {
+      issue_nth(step);
+      if constexpr (COL) {
+        constexpr int kFirst = NT * KS > 2 * NT * 16 ? NT * KS - NT * 16 : 0;      // late: the loads have landed long ago
+        if (step >= kFirst && step - kFirst < NT * 16) {
+          const int i = step - kFirst;
+          rv[i >> 2][i & 3] = fast_rcp(rv[i >> 2][i & 3]);
+        }
+      }
+    });
+    if constexpr (COL && NT * KS < NT * 16) {       // fewer steps than values: the rest here
+#pragma unroll
+      for (int i = NT * KS; i < NT * 16; ++i) rv[i >> 2][i & 3] = fast_rcp(rv[i >> 2][i & 3]);
+    }
     static_for<(kZi + kYi + kMi > NT * KS ? kZi + kYi + kMi - NT * KS : 0)>([&](auto t) {
       issue_nth(NT * KS + decltype(t)::value);      // more copies than steps: the rest in one go
     });
@@ -286,7 +301,7 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
         const int xrow0 = x0 + wave * WM + rt * 32;
         if constexpr (COL) {                       // lane owns kv = xrow0 + n; registers run over q rows j*BY + off
           const int base = j * BY - (xrow0 + n - diag);
-          const auto inv_r = [&](int t, int v) { return fast_rcp(rv[4 * t + (v >> 2)][v & 3]); };
+          const auto inv_r = [&](int t, int v) { return rv[4 * t + (v >> 2)][v & 3]; };
           if (j * BY < xrow0 + 31 - diag) decay.template apply<true>(tacc[rt], base, inv_r);
           else decay.template apply<false>(tacc[rt], base, inv_r);
         } else {                                   // lane owns q = xrow0 + n; registers run over kv columns j*BY + off
@@ -302,7 +317,7 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
           const h4 m = lds_read_tr_h4_at(maddr[rt][i] + moff);
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            tacc[rt][i >> 2][4 * (i & 3) + e] *= (float)m[e] * fast_rcp(rv[i][e]);
+            tacc[rt][i >> 2][4 * (i & 3) + e] *= (float)m[e] * rv[i][e];
         }
       } else {
         apply_mask<NT>(tacc[rt], maddr[rt], moff);
