@@ -210,7 +210,13 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
     for (int i = 0; i < (kOut2 ? KT : 1); ++i) acc2[rt][i] = zero16();
   }
 
-  auto issue = [&](int j, int st) {
+  // Step j of the walk works on streamed tile tile_of(j): the row kernel walks its kv tiles upwards, the column
+  // kernel its query tiles downwards from the end of the sequence.  Either way the blocks of a head that run at the
+  // same time start on the same tile of a causal walk and share it in L2 (a column block needs the tiles from its
+  // own diagonal to the end: walked upwards every block would stream its range alone).
+  const auto tile_of = [&](int j) { return COL ? j_begin + j_end - 1 - j : j; };
+  auto issue = [&](int step, int st) {
+    const int j = tile_of(step);
     char* base = smem + st * T::kStageBytes;
     y1dma.issue(y1g + (size_t)j * T::kY1Bytes, base, wave_base);
     y2dma.issue(y2g + (size_t)j * T::kY2Bytes, base + T::kY1Bytes, wave_base);
@@ -280,7 +286,8 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
     // Only a tile the diagonal crosses runs the masking code.  COL: the statistics of the streamed rows come
     // from LDS four rows at a time, read by hand one group ahead (a tracked read here is answered with a
     // full lgkmcnt(0) per group: eight exposed LDS round trips per tile for the only wave of the SIMD).
-    const bool diag_tile = causal && (COL ? (x0 + BX - 1 > j * BY + diag) : ((j + 1) * BY - 1 > x0 + diag));
+    const int jt = tile_of(j);                      // the tile of this step
+    const bool diag_tile = causal && (COL ? (x0 + BX - 1 > jt * BY + diag) : ((jt + 1) * BY - 1 > x0 + diag));
     auto softmax_part = [&](auto masked_tag) {
       constexpr bool MASKED = decltype(masked_tag)::value;
       constexpr int G = RT * NT * 4;                                 // groups of four streamed rows
@@ -305,10 +312,10 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
             else lds_wait_younger<0>(l2);
           }
         }
-        // The score of resident row x and streamed row y = j*BY + c + 4h (c = 32t + 8g + e, a constant) is masked
-        // when kv > q + diag: COL (x is kv) x - diag - j*BY - 4h > c, ROW (x is q) c > x + diag - j*BY - 4h.
+        // The score of resident row x and streamed row y = jt*BY + c + 4h (c = 32t + 8g + e, a constant) is masked
+        // when kv > q + diag: COL (x is kv) x - diag - jt*BY - 4h > c, ROW (x is q) c > x + diag - jt*BY - 4h.
         const int xrow = x0 + wave * WM + rt * 32 + n;               // resident row of this lane
-        const int lim = (COL ? xrow - diag : xrow + diag) - j * BY - 4 * h;
+        const int lim = (COL ? xrow - diag : xrow + diag) - jt * BY - 4 * h;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           constexpr int vbase = 4 * g, cbase = 32 * t + 8 * g;
