@@ -160,11 +160,14 @@ mask_scan_cols(const unsigned char* __restrict__ occ, int* __restrict__ col_lo, 
   }
 }
 
+// The column scan keeps one running range per thread for up to four bands of 32 kv positions.
+inline bool mask_scan_supported(int Seq_q, int Seq_k) {
+  return Seq_q % kMaskBand == 0 && Seq_k % kMaskBand == 0 && Seq_k / kMaskBand <= 4 * kMaskScanThreads &&
+         Seq_k / kMaskBand <= kMaskColSlab;
+}
 // Enqueues the scan of mask [H, Seq_q, Seq_k] into `workspace` (mask_extent_bytes() bytes).
 inline hipError_t scan_mask(const half_t* mask, int H, int Seq_q, int Seq_k, void* workspace, hipStream_t stream) {
-  if (Seq_q % kMaskBand != 0 || Seq_k % kMaskBand != 0 || Seq_k / kMaskBand > 4 * kMaskScanThreads ||
-      Seq_k / kMaskBand > kMaskColSlab)
-    return hipErrorInvalidValue;
+  if (!mask_scan_supported(Seq_q, Seq_k)) return hipErrorInvalidValue;
   int* p = static_cast<int*>(workspace);
   const size_t nq = (size_t)H * (size_t)(Seq_q / kMaskBand), nk = (size_t)H * (size_t)(Seq_k / kMaskBand);
   unsigned char* occ = reinterpret_cast<unsigned char*>(p + 2 * nq + 2 * nk);
@@ -196,6 +199,7 @@ inline hipError_t prepare_mask_walk(int mode, const half_t* mask, int H, int Seq
                                     hipStream_t stream, MaskWalk* walk) {
   walk->causal = mode == kMaskCausal ? 1 : 0;
   walk->extents = nullptr;
+  if (!mask_scan_supported(Seq_q, Seq_k)) return hipSuccess;      // beyond the scan's reach (S_kv > 32768): every tile, same bits
   if (mode == kMaskScan) {
     const hipError_t e = scan_mask(mask, H, Seq_q, Seq_k, workspace, stream);
     if (e != hipSuccess) return e;

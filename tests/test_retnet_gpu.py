@@ -327,3 +327,16 @@ def test_scan_modes_need_their_workspace_and_reject_unknown_modes():
     assert lib.kernel_entry_ex(*ptrs, 1, 2, 128, 128, -1, null, 0, null) == -2
     assert lib.kernel_entry_ex(*ptrs, 1, 2, 128, 128, 0, null, 0, null) == 0          # the other modes need none
     torch.cuda.synchronize()
+
+
+def test_scan_mode_beyond_the_scan_s_reach_walks_every_tile():
+    """More than 32768 kv positions: the scan is skipped and every tile walked; results unchanged."""
+    sq, sk = 128, 33280
+    q, k, v, _, _ = _inputs(1, 1, sq, sk, 64, 64, seed=31)
+    mask = ref_op.retnet_decay_mask(1, sq, sk)
+    outs = []
+    for mode in (False, None):
+        with torch.no_grad():
+            outs.append(aat.RetNetAttnFunc(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), ARCH, mode))
+    assert torch.equal(outs[0], outs[1])
+    tolerance.assert_close(outs[1], ref_op.retnet_ref(q, k, v, mask), "S_kv 33280")
