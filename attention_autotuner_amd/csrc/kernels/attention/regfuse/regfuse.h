@@ -270,8 +270,13 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
         if constexpr (MASKED) wave_sees = j * Bc <= q0 + wave * WM + WM - 1 + diag;
 
         f16v sacc[RT][NT];
+        // The matrix phases run at a raised wave priority: with two or three waves on the SIMD the one that has
+        // MFMAs to issue goes first and the others' softmax arithmetic fills the gaps, not the other way round
+        // (causal forward at three waves per SIMD: -1.4 %; nothing at two).
         if (wave_sees) {
+          __builtin_amdgcn_s_setprio(2);
           qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
+          __builtin_amdgcn_s_setprio(0);
         }
         if constexpr (PERSIST) {
           if (!more && has_next) load_q_frags_async<RT, KS, Kd>(qf, q_next);   // the last scores of this row block are done; waited for at (A)
@@ -296,10 +301,12 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
         }
         if (wave_sees) {
           h8 pf[RT][NT][2];
+          __builtin_amdgcn_s_setprio(2);
           pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) pack_p_group<NT>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
           });
+          __builtin_amdgcn_s_setprio(0);
         }
       };
       run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
