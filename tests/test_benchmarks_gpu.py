@@ -1,5 +1,5 @@
-"""The stand-alone benchmark programs (counterparts of reference benchmarks/attention.cu and the recurrent part of
-benchmarks/retnet/retnet.cu) run on the GPU and agree with the Python-side timing of the same kernels."""
+"""The stand-alone benchmark programs (counterparts of reference benchmarks/attention.cu, benchmarks/retnet/retnet.cu
+and benchmarks/retnet/retnet_bwd.cu) run on the GPU and agree with the Python-side timing of the same kernels."""
 import os
 import re
 import subprocess
@@ -60,3 +60,63 @@ def test_retnet_recurrent_bench_checks_one_slice_and_reports():
     print(out)
     assert "-> ok" in out and "MISMATCH" not in out
     assert re.search(r"median [\d.]+ .* TFLOP/s", out)
+
+
+RET_LINE = re.compile(r"^(smemfuse|regfuse|bwd chain)\s+Br=(\d+) Bc=(\d+) thr=(\d+) bufs=(\S+) (?:grid=(\S+) )?waves/SIMD=(\d+)\s+mask (\w+)\s+"
+                      r"mean ([\d.]+) ms\s+median ([\d.]+).*-> (ok|MISMATCH)")
+
+
+def _retnet_rows(out):
+    rows = [m for m in (RET_LINE.match(l) for l in out.splitlines()) if m]
+    assert rows and all(m[11] == "ok" for m in rows), out                  # the programs check a slice of every result on the host
+    return {(m[1], int(m[2]), int(m[3]), int(m[4]), m[5], m[6], int(m[7]), m[8]): float(m[10]) for m in rows}
+
+
+def _retnet_tensors(b, h, s, dqk=256, dv=512):
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k = (torch.randn(b, h, s, dqk, device="cuda", generator=g).half() for _ in range(2))
+    v, do = (torch.randn(b, h, s, dv, device="cuda", generator=g).half() for _ in range(2))
+    mask = torch.randn(h, s, s, device="cuda", generator=g).half()
+    return q, k, v, do, mask
+
+
+def test_retnet_bench_checks_every_mask_mode_and_agrees_with_the_library_timing():
+    """Small shape first (every configuration x every way of handing over the mask, each verified on the host), then the
+    reference's shape (benchmarks/retnet/retnet.cu:218) for the dense walk against the library launcher of the same kernel."""
+    small = _retnet_rows(_run("retnet_bench", "1", "2", "256", "256", "--no-flush"))
+    assert {key[7] for key in small} == {"dense", "causal", "scan", "decay"} and len(small) == 16
+    out = _run("retnet_bench", "4", "8", "2048", "2048", "--mask", "dense", "--no-flush")
+    print(out)
+    times = _retnet_rows(out)
+    key = ("smemfuse", 128, 64, 512, "1/1/1", "2x8", 2, "dense")
+    from attention_autotuner_amd.autotuner import prebuilt
+    cfg = next(c for c in prebuilt.cached_configs() if c.operation == "ret" and (c.Kd, c.D) == (256, 512)
+               and (c.Br, c.Bc, c.Nthreads, c.warps_mma1_n, c.warps_mma_n, c.waves_per_eu) == (128, 64, 512, 2, 8, 2))
+    q, k, v, _, mask = _retnet_tensors(4, 8, 2048)
+    o = torch.empty_like(v)
+    r = torch.empty(4, 8, 2048, device="cuda", dtype=torch.float32)
+    launch = Runtime(ARCH, cfg).bind([q, k, v, mask, o, r], causal=False)
+    lib_ms = LaunchTimer(min_warmup_ms=50).measure(launch, calls=200).median
+    print(f"retnet_bench {key}: {times[key]:.4f} ms; library launcher: {lib_ms:.4f} ms")
+    assert abs(times[key] - lib_ms) <= 0.10 * lib_ms
+    assert times[key] == min(times.values())                              # the tuned configuration leads the list
+
+
+def test_retnet_bwd_bench_checks_every_mask_mode_and_agrees_with_the_library_timing():
+    small = _retnet_rows(_run("retnet_bwd_bench", "1", "2", "256", "256", "--no-flush"))
+    assert {key[7] for key in small} == {"dense", "causal", "scan", "decay"} and len(small) == 12
+    out = _run("retnet_bwd_bench", "4", "8", "2048", "2048", "--mask", "dense", "--no-flush")
+    print(out)
+    times = _retnet_rows(out)
+    key = ("bwd chain", 128, 64, 256, "1/1", None, 1, "dense")
+    from attention_autotuner_amd.autotuner import prebuilt
+    # the configuration the tuner recorded for this problem's dense walk; its library is part of the shipped set
+    cfg = next(c for c in prebuilt.cached_configs() if c.operation == "ret_bwd" and (c.Kd, c.D) == (256, 512)
+               and (c.Br, c.Bc, c.Nthreads, c.num_stages_qk, c.num_stages_dv, c.waves_per_eu) == (128, 64, 256, 1, 1, 1))
+    q, k, v, do, mask = _retnet_tensors(4, 8, 2048)
+    r = torch.full((4, 8, 2048), 1000.0, device="cuda", dtype=torch.float32)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    launch = Runtime(ARCH, cfg).bind([q, k, v, mask, do, r, dq, dk, dv, torch.zeros(1, device="cuda")], causal=False)
+    lib_ms = LaunchTimer(min_warmup_ms=50).measure(launch, calls=100).median
+    print(f"retnet_bwd_bench {key}: {times[key]:.4f} ms; library launcher: {lib_ms:.4f} ms")
+    assert abs(times[key] - lib_ms) <= 0.10 * lib_ms
