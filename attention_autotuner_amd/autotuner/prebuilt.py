@@ -98,7 +98,7 @@ def prune_stale(build_dir=None):
         keep = "-" + codegen.source_digest(op) + "."
         for dirpath, _, files in os.walk(os.path.join(root, op)):
             for fn in files:
-                if fn.endswith((".so", ".hip", ".log")) and keep not in fn:
+                if fn.endswith((".so", ".hip", ".log", ".usage.json")) and keep not in fn:
                     os.remove(os.path.join(dirpath, fn))
                     removed += 1
     return removed

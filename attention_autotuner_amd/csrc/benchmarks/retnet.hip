@@ -160,6 +160,7 @@ int main(int argc, char** argv) {
   test_smemfuse_retnet<128, 64, 512, 1, 1, 1, 2, 8, 2>(ps, t);
   test_smemfuse_retnet<128, 64, 512, 1, 1, 1, 2, 4, 2>(ps, t);
   test_smemfuse_retnet<64, 64, 256, 1, 1, 1, 2, 4, 1>(ps, t);
+  test_regfuse_retnet<128, 32, 256, 1, 1, 1, 1>(ps, t);
   test_regfuse_retnet<128, 64, 256, 1, 1, 1, 1>(ps, t);
 
   for (auto* x : {&t.q, &t.k, &t.v, &t.mask_dense, &t.mask_decay, &t.o}) x->release();

@@ -103,7 +103,9 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
 
   h8 qf[RT][KS];
   load_q_frags<RT, KS, Kd>(qf, q + ((size_t)bh * seq_q + q0 + wave * WM + n) * Kd + 8 * h);
-  uint32_t kaddr[KS], vaddr[DT], maddr[RT][NT * 4];
+  // one mask address per 32-row group where the tile's rows are a power of two of chunks (see apply_mask_folded)
+  constexpr bool kFoldMask = (NCM & (NCM - 1)) == 0 && NCM <= 16;
+  uint32_t kaddr[KS], vaddr[DT], maddr[RT][kFoldMask ? 1 : NT * 4];
   {
     int koff[KS], voff[DT];
     k_frag_offsets<KS, NCK>(koff, n, h);
@@ -115,7 +117,7 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int i = 0; i < NT * 4; ++i)
+      for (int i = 0; i < (kFoldMask ? 1 : NT * 4); ++i)
         maddr[rt][i] = lds_addr(mbuf + lds_chunk_off<NCM, Swz::Rows16>(wave * WM + rt * 32 + n, i) + 8 * h);
   }
 
@@ -126,7 +128,13 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
     row[rt].big_r = 0.f;
     row[rt].r_ref = 1.f;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] = zero16();
+    for (int dt = 0; dt < DT; ++dt) {
+      oacc[rt][dt] = zero16();
+      // One wave per SIMD: the zeros go into accumulation registers here.  As literals they also reach the epilogue
+      // on the path of a block without kv tiles, and the compiler then keeps that copy of the whole tile in vector
+      // registers across the main loop.
+      if constexpr (WPE == 1) asm volatile("" : "+a"(oacc[rt][dt]));
+    }
   }
 
   auto issue_km = [&](int j, int par) {          // K tile j and mask tile j travel together
@@ -175,7 +183,8 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
         if ((j + 1) * Bc - 1 > own0) decay.template apply<true>(sacc[rt], own0 + n - j * Bc, one);
         else decay.template apply<false>(sacc[rt], own0 + n - j * Bc, one);
       } else {
-        apply_mask<NT>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
+        if constexpr (kFoldMask) apply_mask_folded<NT>(sacc[rt], maddr[rt][0], NSM == 2 ? PAR * T::kMBytes : 0);
+        else apply_mask<NT>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
       }
       retention_step<NT, DT, WPE == 1>(sacc[rt], row[rt], oacc[rt]);
     }
@@ -202,6 +211,12 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
   }
 
   // ---- epilogue -------------------------------------------------------------------------------------
+  if constexpr (WPE == 1) {        // the accumulators leave the loop where the MFMAs left them (see kv_tile)
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
+  }
   wait_vmcnt<0>();
   block_sync();
   float scale[RT];

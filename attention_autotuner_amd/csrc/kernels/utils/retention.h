@@ -35,6 +35,23 @@ AAT_DEV void apply_mask(f16v (&s)[NT], const uint32_t (&maddr)[NT * 4], int buf_
   }
 }
 
+// The same from one address register.  In a Rows16-swizzled tile whose rows are a power of two of chunks, chunk i
+// of a row sits at (row start + 16 (i ^ x)) with x fixed per row; a row starts at a multiple of its own size (the
+// buffer does too), so that is (address of the row's chunk 0) ^ 16 i.  chunk0 = that address + 8h.
+template <int NT>
+AAT_DEV void apply_mask_folded(f16v (&s)[NT], uint32_t chunk0, int buf_off) {
+  asm volatile("" : "+v"(chunk0));      // or the 4 NT addresses are computed once, ahead of the loop, and kept in registers
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const h4 m = *reinterpret_cast<AAT_AS3 const h4*>((uintptr_t)((chunk0 ^ (uint32_t)((4 * t + g) << 4)) + buf_off));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[t][4 * g + e] *= (float)m[e];
+    }
+  }
+}
+
 // Decay mask evaluated in registers instead of read from a [H, S_q, S_kv] tensor.  The reference always
 // streams the tensor (reference: python/ops/retnet_interface.py:26-31) and lists "causal config" and the
 // mask stream's cost ("retnet performance issue ... mask stage 2?") as open items (README.md:102-114):
@@ -74,7 +91,8 @@ struct DecayMask {
   // this tile, entries above it are zeroed.
   template <bool DIAG, class Extra>
   AAT_DEV void apply(f16v (&s)[NT], int base, Extra&& extra) const {
-    const float tf = fast_exp2(lg * (float)(OWN_Q ? base - h4 : base + h4));
+    const int own = OWN_Q ? base - h4 : base + h4;        // this lane's distance to the diagonal at register 0
+    const float tf = fast_exp2(lg * (float)own);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -84,9 +102,9 @@ struct DecayMask {
         for (int e = 0; e < 4; ++e) {
           const int v = 4 * g + e;
           float m = tg * fa[e] * extra(t, v);
-          if constexpr (DIAG) {
-            const int off = 32 * t + 8 * g + h4 + e;
-            if ((OWN_Q ? base - off : base + off) < 0) m = 0.f;
+          if constexpr (DIAG) {          // against a literal: base -/+ (offset + 4h) per register would be 16 NT values kept per lane
+            const int off = 32 * t + 8 * g + e;
+            if ((OWN_Q ? own - off : own + off) < 0) m = 0.f;
           }
           s[t][v] *= m;
         }
@@ -96,8 +114,7 @@ struct DecayMask {
 
 // Fold one masked score tile into the row statistics and turn it into P = S / r_ref (in place).
 // Rescales the O accumulators when the reference scale moves.
-// ACC_PIN: the O accumulators live in accumulation registers (kernels above 256 registers); rescale
-// them one 16-register block at a time so the copies through vector registers stay short-lived.
+// ACC_PIN: the O accumulators live in accumulation registers (kernels above 256 registers) and are rescaled there.
 template <int NT, int DT, bool ACC_PIN = false>
 AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) {
   float part = 0.f;
@@ -111,11 +128,23 @@ AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) 
     const float r_new = fmaxf(row.big_r, 1.0f);
     const float alpha = row.r_ref * fast_rcp(r_new);
     row.r_ref = r_new;
+    if constexpr (ACC_PIN) {
+      // In place, one register at a time, by hand: given the loop the compiler reads dozens of accumulation
+      // registers ahead of the multiplications and spills vector registers to make room for them.
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
+      for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
-      if constexpr (ACC_PIN) asm volatile("" : "+a"(oacc[dt]));
+        for (int v = 0; v < 16; ++v) {
+          float x = oacc[dt][v], t;
+          asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %2, %1\n\tv_accvgpr_write_b32 %0, %1"
+                       : "+a"(x), "=&v"(t) : "v"(alpha));
+          oacc[dt][v] = x;
+        }
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
     }
   }
   const float inv = fast_rcp(row.r_ref);

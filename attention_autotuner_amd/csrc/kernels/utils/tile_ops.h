@@ -217,11 +217,16 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
   constexpr int G = NT * 2;              // groups of 16 kv rows
   constexpr int S = G * DT;
   constexpr int kRow16 = 16 * NCV * 16, kRow8 = 8 * NCV * 16;
+  // The Rows4 swizzle of rows of whole 16-chunk groups exchanges chunks inside a group of 16 only, and a d-tile
+  // is four chunks wide: d-tile dt sits 256 bytes per group behind d-tile dt % 4, so four address registers
+  // serve any output width (the others are never read and cost nothing).
+  constexpr bool kFold = NCV % 16 == 0 && DT > 4;
+  auto addr = [&](int i) { return (kFold ? vaddr[(i % DT) % 4] + ((i % DT) / 4) * 256 : vaddr[i % DT]) + buf_off + (i / DT) * kRow16; };
   h4 lo[PF], hi[PF];
 #pragma unroll
   for (int i = 0; i < PF && i < S; ++i) {
-    lo[i] = lds_read_tr_h4_at(vaddr[i % DT] + buf_off + (i / DT) * kRow16);
-    hi[i] = lds_read_tr_h4_at(vaddr[i % DT] + buf_off + (i / DT) * kRow16 + kRow8);
+    lo[i] = lds_read_tr_h4_at(addr(i));
+    hi[i] = lds_read_tr_h4_at(addr(i) + kRow8);
   }
   pack(0);
   sched_fence();
@@ -231,8 +236,8 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
     const h8 vf = cat_h4(lo[step % PF], hi[step % PF]);
     if (step + PF < S) {
       const int nx = step + PF;
-      lo[step % PF] = lds_read_tr_h4_at(vaddr[nx % DT] + buf_off + (nx / DT) * kRow16);
-      hi[step % PF] = lds_read_tr_h4_at(vaddr[nx % DT] + buf_off + (nx / DT) * kRow16 + kRow8);
+      lo[step % PF] = lds_read_tr_h4_at(addr(nx));
+      hi[step % PF] = lds_read_tr_h4_at(addr(nx) + kRow8);
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
@@ -255,23 +260,29 @@ AAT_DEV void store_o_tile(const f16v (&oacc)[RT][DT], const float (&row_scale)[R
     const float sc = row_scale[rt];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+      // Accumulators that fill the accumulation registers come back one 16-register block at a time: left to
+      // itself the compiler copies all of them into vector registers at the end of the main loop, and the kernel
+      // spills for it.  The empty statements keep their order, so block dt is still where the MFMAs left it here.
+      f16v blk = oacc[rt][dt];
+      if constexpr (RT * DT * 16 >= 256) asm volatile("" : "+a"(blk));
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int d0 = 32 * dt + 8 * g + 4 * h;
         char* dst = ostage + (rt * 32 + n) * O_STRIDE + d0 * kElem;
         if constexpr (kElem == 2) {
-          const h2 a = pack_rne(oacc[rt][dt][4 * g] * sc, oacc[rt][dt][4 * g + 1] * sc);
-          const h2 b = pack_rne(oacc[rt][dt][4 * g + 2] * sc, oacc[rt][dt][4 * g + 3] * sc);
+          const h2 a = pack_rne(blk[4 * g] * sc, blk[4 * g + 1] * sc);
+          const h2 b = pack_rne(blk[4 * g + 2] * sc, blk[4 * g + 3] * sc);
           h4 w;
           w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
           *reinterpret_cast<h4*>(dst) = w;
         } else {
           f4v w;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) w[e] = oacc[rt][dt][4 * g + e] * sc;
+          for (int e = 0; e < 4; ++e) w[e] = blk[4 * g + e] * sc;
           *reinterpret_cast<f4v*>(dst) = w;
         }
       }
+      if constexpr (RT * DT * 16 >= 256) sched_fence();
     }
   }
   wait_lgkm0();                                   // the staging region is private to this wave

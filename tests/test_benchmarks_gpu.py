@@ -84,7 +84,7 @@ def test_retnet_bench_checks_every_mask_mode_and_agrees_with_the_library_timing(
     """Small shape first (every configuration x every way of handing over the mask, each verified on the host), then the
     reference's shape (benchmarks/retnet/retnet.cu:218) for the dense walk against the library launcher of the same kernel."""
     small = _retnet_rows(_run("retnet_bench", "1", "2", "256", "256", "--no-flush"))
-    assert {key[7] for key in small} == {"dense", "causal", "scan", "decay"} and len(small) == 16
+    assert {key[7] for key in small} == {"dense", "causal", "scan", "decay"} and len(small) == 20
     out = _run("retnet_bench", "4", "8", "2048", "2048", "--mask", "dense", "--no-flush")
     print(out)
     times = _retnet_rows(out)
