@@ -130,7 +130,12 @@ ret_fwd_smemfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, con
 #pragma unroll
   for (int rt = 0; rt < RT2; ++rt)
 #pragma unroll
-    for (int dt = 0; dt < DT2; ++dt) oacc[rt][dt] = zero16();
+    for (int dt = 0; dt < DT2; ++dt) {
+      oacc[rt][dt] = zero16();
+      // one wave per SIMD: zero into accumulation registers, or the literal zeros that also reach the epilogue on
+      // the path of a block without kv tiles are kept in vector registers across the main loop
+      if constexpr (WPE == 1) asm volatile("" : "+a"(oacc[rt][dt]));
+    }
   RetentionRow row[RT1];
 #pragma unroll
   for (int rt = 0; rt < RT1; ++rt) {
@@ -225,11 +230,7 @@ ret_fwd_smemfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, con
     if (__builtin_amdgcn_readfirstlane(any) != 0) {
 #pragma unroll
       for (int rt = 0; rt < RT2; ++rt) {
-        const float a = alpha_s[row2 + rt * 32 + n];
-#pragma unroll
-        for (int dt = 0; dt < DT2; ++dt)
-#pragma unroll
-          for (int vv = 0; vv < 16; ++vv) oacc[rt][dt][vv] *= a;
+        rescale_acc<DT2, WPE == 1>(oacc[rt], alpha_s[row2 + rt * 32 + n]);
       }
     }
     pv_gemm_from_lds<RT2, DT2, Bc / 16, NCV>(oacc, paddr, vaddr, NSV == 2 ? PAR * T::kVBytes : 0);

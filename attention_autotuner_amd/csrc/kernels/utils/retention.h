@@ -112,6 +112,26 @@ struct DecayMask {
   }
 };
 
+// O <- O * alpha for one 32-row group.  IN_PLACE: the accumulators live in accumulation registers (kernels above 256
+// registers) and are multiplied there, one register at a time, by hand: given the loop the compiler reads dozens of
+// accumulation registers ahead of the multiplications and spills vector registers to make room for them.
+template <int DT, bool IN_PLACE>
+AAT_DEV void rescale_acc(f16v (&oacc)[DT], float alpha) {
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      if constexpr (IN_PLACE) {
+        float x = oacc[dt][v], t;
+        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %2, %1\n\tv_accvgpr_write_b32 %0, %1"
+                     : "+a"(x), "=&v"(t) : "v"(alpha));
+        oacc[dt][v] = x;
+      } else {
+        oacc[dt][v] *= alpha;
+      }
+    }
+}
+
 // Fold one masked score tile into the row statistics and turn it into P = S / r_ref (in place).
 // Rescales the O accumulators when the reference scale moves.
 // ACC_PIN: the O accumulators live in accumulation registers (kernels above 256 registers) and are rescaled there.
@@ -128,24 +148,7 @@ AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) 
     const float r_new = fmaxf(row.big_r, 1.0f);
     const float alpha = row.r_ref * fast_rcp(r_new);
     row.r_ref = r_new;
-    if constexpr (ACC_PIN) {
-      // In place, one register at a time, by hand: given the loop the compiler reads dozens of accumulation
-      // registers ahead of the multiplications and spills vector registers to make room for them.
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float x = oacc[dt][v], t;
-          asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %2, %1\n\tv_accvgpr_write_b32 %0, %1"
-                       : "+a"(x), "=&v"(t) : "v"(alpha));
-          oacc[dt][v] = x;
-        }
-    } else {
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
-    }
+    rescale_acc<DT, ACC_PIN>(oacc, alpha);
   }
   const float inv = fast_rcp(row.r_ref);
 #pragma unroll
