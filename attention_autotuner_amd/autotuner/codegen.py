@@ -17,6 +17,7 @@ import re
 import shutil
 import subprocess
 import sys
+import threading
 from concurrent.futures import ThreadPoolExecutor
 
 _PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
@@ -138,7 +139,7 @@ def compile_config(config, arch, build_dir=None, timeout=None, force=False):
         return None
     with open(src, "w") as f:
         f.write(text)
-    tmp = out + f".tmp{os.getpid()}"
+    tmp = out + f".tmp{os.getpid()}_{threading.get_ident()}"     # two threads of one process may build the same library
     try:
         ret = subprocess.run(hipcc_command(src, tmp, arch), timeout=timeout, capture_output=True, text=True)
     except subprocess.TimeoutExpired:
@@ -219,12 +220,17 @@ def compile_parallel(configs, arch, build_dir=None, timeout=None, max_workers=No
     progress = os.environ.get("AAT_PROGRESS", "0") not in ("", "0")      # long builds under a watchdog: say that work goes on
     done = [0]
 
+    first = {}                                     # a configuration listed twice is built once
+    for c in configs:
+        first.setdefault(library_path(c, build_dir), c)
+
     def build(c):
         lib = compile_config(c, arch, build_dir, timeout)
         done[0] += 1
-        if progress and (done[0] % 8 == 0 or done[0] == len(configs)):
-            print(f"[build] {done[0]}/{len(configs)} libraries", file=sys.stderr, flush=True)
+        if progress and (done[0] % 8 == 0 or done[0] == len(first)):
+            print(f"[build] {done[0]}/{len(first)} libraries", file=sys.stderr, flush=True)
         return lib
 
     with ThreadPoolExecutor(max_workers=workers) as pool:
-        return list(pool.map(build, configs))
+        built = dict(zip(first, pool.map(build, first.values())))
+    return [built[library_path(c, build_dir)] for c in configs]
