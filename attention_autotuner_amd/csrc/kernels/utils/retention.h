@@ -114,7 +114,8 @@ struct DecayMask {
 
 // O <- O * alpha for one 32-row group.  IN_PLACE: the accumulators live in accumulation registers (kernels above 256
 // registers) and are multiplied there, one register at a time, by hand: given the loop the compiler reads dozens of
-// accumulation registers ahead of the multiplications and spills vector registers to make room for them.
+// accumulation registers ahead of the multiplications and spills vector registers to make room for them.  The matrix
+// instructions that last wrote these registers are a whole score contraction back, so no read here needs a wait.
 template <int DT, bool IN_PLACE>
 AAT_DEV void rescale_acc(f16v (&oacc)[DT], float alpha) {
 #pragma unroll
@@ -130,6 +131,9 @@ AAT_DEV void rescale_acc(f16v (&oacc)[DT], float alpha) {
         oacc[dt][v] *= alpha;
       }
     }
+  // The compiler does not see the writes above and inserts no wait states between the last of them and a matrix
+  // instruction that takes the register as its addend; this runs once in hundreds of tiles.
+  if constexpr (IN_PLACE) asm volatile("s_nop 3" : "+a"(oacc[DT - 1]));
 }
 
 // Fold one masked score tile into the row statistics and turn it into P = S / r_ref (in place).

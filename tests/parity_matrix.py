@@ -39,6 +39,14 @@ def ret_register_wide():
     return RetConfig(128, 64, 256, 512, 256, 64, 1, 1, 1, 256, True, waves_per_eu=1).set_fuse_type("register")
 
 
+def ret_shared_wide_one_wave():
+    """The LDS-fused RetNet forward with four waves at d_v 512: a wave of the second grid holds 32 rows x 512 columns, the
+    same 256 accumulation registers per lane, and rescales them in place like the register-fused kernel."""
+    cfg = RetConfig(128, 64, 256, 512, 256, 64, 1, 1, 1, 256, True, 1, 4, waves_per_eu=1)
+    cfg.fuse_type = "shared"
+    return cfg
+
+
 def parity_configs(arch=None):
     arch = arch or MI355X()
     out = []
@@ -52,6 +60,7 @@ def parity_configs(arch=None):
             if gfx950_space.forward_valid(cfg, arch):
                 out.append(cfg)
     out.append(ret_register_wide())
+    out.append(ret_shared_wide_one_wave())
     out += [attn_bwd_split_config(*t) for t in ATTN_BWD_SPLIT_TILES]
     out.append(AttnBwdConfig(64, 64, 128, 128, 128, 2, row_waves_per_eu=2, row_Bc=32))      # row kernel with a tile height of its own
     for br, bc, nt, st in ATTN_BWD_TILES:

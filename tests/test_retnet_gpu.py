@@ -145,14 +145,16 @@ def test_non_square_and_every_prebuilt_variant():
     assert ran >= 4
 
 
-def test_register_fused_forward_at_dqk256_dv512():
-    """The register-fused kernel holds a 32 x 512 fp32 output block per wave: all 256 accumulation registers of a wave that
-    has its SIMD to itself, rescaled in place when the lazy normaliser moves (the sums of |S| pass 256 within the first
-    tiles here).  It is built without a byte of scratch and must be right for every way of handing over the mask."""
+@pytest.mark.parametrize("which", ["register", "shared"])
+def test_one_wave_forward_with_256_accumulators_at_dqk256_dv512(which):
+    """The register-fused kernel (and the LDS-fused one with four waves) holds a 32 x 512 fp32 output block per wave: all
+    256 accumulation registers of a wave that has its SIMD to itself, rescaled in place when the lazy normaliser moves
+    (the sums of |S| pass 256 within the first tiles here).  It is built without a byte of scratch and must be right
+    for every way of handing over the mask."""
     import parity_matrix
-    cfg = parity_matrix.ret_register_wide()
+    cfg = parity_matrix.ret_register_wide() if which == "register" else parity_matrix.ret_shared_wide_one_wave()
     assert gfx950_space.forward_valid(cfg, ARCH) and os.path.exists(codegen.library_path(cfg))
-    report = [k for k in codegen.resource_usage(codegen.library_path(cfg)) if "ret_fwd_regfuse" in k["kernel"]]
+    report = [k for k in codegen.resource_usage(codegen.library_path(cfg)) if "ret_fwd_" in k["kernel"]]
     assert len(report) == 2 and all(k["scratch_bytes"] == 0 and k["agprs"] == 256 for k in report), report
     q, k, v, mask, _ = _inputs(2, 3, 256, 384, 256, 512, seed=12)
     o_ref, r_ref = ref_op.retnet_ref(q, k, v, ref_op.retnet_decay_mask(3, 256, 384), return_r=True)
@@ -162,7 +164,7 @@ def test_register_fused_forward_at_dqk256_dv512():
         o = torch.zeros(2, 3, 256, 512, dtype=torch.float16, device="cuda")
         r = torch.zeros(2, 3, 256, dtype=torch.float32, device="cuda")
         Runtime(ARCH, cfg).apply(dev + [o, r], causal=mode)
-        tolerance.assert_close(o, o_ref, f"register-fused 256/512 walk={mode}")
+        tolerance.assert_close(o, o_ref, f"{which}-fused 256/512 walk={mode}")
         assert ((r.cpu() - r_ref).abs() / r_ref).max().item() <= 1e-3
     # the decay rates in registers instead of the tensor (the mask is then exact, not rounded to fp16)
     _, _, _, _, gamma, exact = _decay_problem(2, 3, 256, 384, 256, 512, seed=0)
@@ -171,7 +173,7 @@ def test_register_fused_forward_at_dqk256_dv512():
     o = torch.zeros(2, 3, 256, 512, dtype=torch.float16, device="cuda")
     r = torch.zeros(2, 3, 256, dtype=torch.float32, device="cuda")
     Runtime(ARCH, cfg).apply(dev[:3] + [lg, o, r], decay=True)
-    tolerance.assert_close(o, o_ref, "register-fused 256/512 decay rates")
+    tolerance.assert_close(o, o_ref, f"{which}-fused 256/512 decay rates")
     assert ((r.cpu() - r_ref).abs() / r_ref).max().item() <= 1e-3
 
 
