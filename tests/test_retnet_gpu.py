@@ -355,3 +355,44 @@ def test_scan_mode_beyond_the_scan_s_reach_walks_every_tile():
             outs.append(aat.RetNetAttnFunc(q.cuda(), k.cuda(), v.cuda(), mask.cuda(), ARCH, mode))
     assert torch.equal(outs[0], outs[1])
     tolerance.assert_close(outs[1], ref_op.retnet_ref(q, k, v, mask), "S_kv 33280")
+
+
+def test_scanned_forward_and_backward_replay_from_a_captured_graph():
+    """The mask scan is two kernels on the caller's stream and the walk reads its ranges on the GPU: forward (scan
+    included) and backward (scan reused) can be captured as one graph; replays with new inputs and a new mask match
+    eager launches bit for bit."""
+    b, h, sq, sk, dqk, dv = 1, 2, 256, 384, 64, 128
+    q, k, v, mask, do = (t.cuda() for t in _inputs(b, h, sq, sk, dqk, dv, seed=41))
+    fcfg = gfx950_space.default_forward_config("ret", dqk, dv, ARCH, sq, sk)
+    bcfg = gfx950_space.default_backward_config(dqk, dv, ARCH, sq, sk)
+    fwd, bwd = Runtime(ARCH, fcfg), Runtime(ARCH, bcfg)
+    o = torch.empty(b, h, sq, dv, dtype=torch.float16, device="cuda")
+    r = torch.empty(b, h, sq, dtype=torch.float32, device="cuda")
+    dq, dk, dvv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    acc = torch.zeros(1, dtype=torch.float32, device="cuda")
+    ws = torch.empty(fwd.workspace_size(b, h, sq, sk), dtype=torch.uint8, device="cuda")
+
+    def run(o_, r_, dq_, dk_, dv_, ws_):
+        fwd.apply([q, k, v, mask, o_, r_], causal="scan", workspace=ws_)
+        bwd.apply([q, k, v, mask, do, r_, dq_, dk_, dv_, acc], causal="scanned", workspace=ws_)
+
+    run(o, r, dq, dk, dvv, ws)                             # first call outside capture: one-time LDS opt-in
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(o, r, dq, dk, dvv, ws)
+    for seed in (42, 43, 44):
+        q2, k2, v2, m2, do2 = _inputs(b, h, sq, sk, dqk, dv, seed=seed)
+        if seed == 43:                                     # another pattern of zero tiles: a band instead of a triangle
+            m2 = m2 * (torch.arange(sq).view(1, sq, 1) - torch.arange(sk).view(1, 1, sk) < 96).half()
+        for dst, src in ((q, q2), (k, k2), (v, v2), (mask, m2), (do, do2)):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = [torch.empty_like(t) for t in (o, r, dq, dk, dvv)]
+        run(*eager, torch.empty_like(ws))
+        torch.cuda.synchronize()
+        for got, want in zip((o, r, dq, dk, dvv), eager):
+            assert torch.equal(got, want)
+        o_ref, r_ref = ref_op.retnet_ref(q2, k2, v2, m2, return_r=True)
+        tolerance.assert_close(o, o_ref, f"captured scanned forward seed={seed}")
