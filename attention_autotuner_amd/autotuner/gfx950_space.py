@@ -233,8 +233,22 @@ def backward_reg_estimate(cfg):
     return vec, acc
 
 
+DS_ROWS = (128, 256)          # kv rows per block of the dK kernel that reads a stored dS (64-row query tiles, two stages)
+DS_TILE = 64
+
+
 def backward_valid(cfg, arch):
     nw = _waves(cfg)
+    ds_rows = getattr(cfg, "ds_rows", 0)
+    if ds_rows:
+        if ds_rows not in DS_ROWS or cfg.Br % DS_TILE or cfg.waves_per_eu != 1:
+            return False
+        # the row pass stages a dS tile behind its stream buffers; the dK kernel holds two (Q tile, dS tile) pairs
+        row_lds = cfg.num_stages_qk * (cfg.Bc * cfg.D * 2 + cfg.Br * cfg.Bc * 2) + cfg.num_stages_dv * cfg.Bc * cfg.Kd * 2
+        if row_lds + cfg.Br * (cfg.Bc * 2 + 16) > arch.smem_cap:
+            return False
+        if 2 * DS_TILE * (cfg.Kd + ds_rows) * 2 > arch.smem_cap:
+            return False
     if cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * nw) or cfg.Bc % 32:
         return False
     if nw > 4 * cfg.waves_per_eu:
@@ -265,6 +279,11 @@ def backward_candidates(br, bc, dim_qk, dim_v):
                 n = nthreads // WAVE
                 out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, BlockKSmem=dim_qk,
                                         num_stages_qk=st_y, num_stages_mask=st_y, num_stages_dv=st_z, waves_per_eu=wpe))
+                if wpe == 1:          # ... and with dS stored by the dQ pass for a dK kernel of its own (needs the workspace)
+                    for ds_rows in DS_ROWS:
+                        out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, BlockKSmem=dim_qk,
+                                                num_stages_qk=st_y, num_stages_mask=st_y, num_stages_dv=st_z,
+                                                waves_per_eu=wpe, ds_rows=ds_rows))
     return out
 
 

@@ -22,6 +22,19 @@ _ERRORS = {-2: "sequence lengths are not multiples of the configuration's tile (
            -3: "workspace missing or too small"}
 
 
+def _grown(workspace, need, device, keep):
+    """A workspace of ``need`` bytes.  ``keep``: the one handed in holds a mask scan an earlier launch left (mode
+    "scanned") and is smaller than this library wants (a backward that also stores dS): its bytes move to the head of
+    the new one, where the library looks for them."""
+    new = torch.empty(need, dtype=torch.uint8, device=device)
+    if keep:
+        if workspace is None:
+            raise KernelLaunchError('mask mode "scanned" needs the workspace an earlier "scan" launch filled')
+        old = workspace.reshape(-1).view(torch.uint8)
+        new[:old.numel()].copy_(old)
+    return new
+
+
 class Runtime:
     def __init__(self, arch, config, tmp_dir=None, libname=None):
         self.arch = arch
@@ -57,7 +70,7 @@ class Runtime:
         lib = library.load(self._path(), op)
         need = int(lib.workspace_size(B, H, Sq, Sk))
         if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
-            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            workspace = _grown(workspace, need, q.device, keep=causal == "scanned")
         ws_ptr = ctypes.c_void_p(workspace.data_ptr() if workspace is not None else 0)
         ws_bytes = ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0)
         if op in library.SCALED_OPS:
@@ -96,7 +109,7 @@ class Runtime:
         lib = library.load(self._path(), op)
         need = int(lib.workspace_size(B, H, Sq, Sk))
         if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
-            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            workspace = _grown(workspace, need, q.device, keep=causal == "scanned")
         args = [ctypes.c_void_p(t.data_ptr()) for t in torch_array] + [B, H, Sq, Sk]
         if op in library.SCALED_OPS:
             args.append(ctypes.c_float(softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])))

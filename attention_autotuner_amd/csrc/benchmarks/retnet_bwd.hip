@@ -12,6 +12,7 @@
 // operator).  TFLOP/s counts the five contractions, 2*B*H*Sq*Sk*(3 d_qk + 2 d_v), halved for the walks that
 // skip the tiles above the diagonal.
 #include "../kernels/retnet/bwd/bwd_chain.h"
+#include "../kernels/retnet/bwd/dk_from_ds.h"
 #include "../kernels/retnet/smemfuse/smemfuse.h"
 #include "retnet_common.h"
 
@@ -24,6 +25,7 @@ struct Tensors {
   HostDevice<half_t> q, k, v, dout, mask_dense, mask_decay, o, dq, dk, dv;
   HostDevice<float> r, log2_gamma;
   void* scan = nullptr;
+  half_t* ds = nullptr;          // [B*H, Sq, Sk]: dS as the row pass forms it, for the dK kernel that reads it back
 };
 
 // r (and the scan of the decay mask) as the forward leaves them.
@@ -140,17 +142,17 @@ static void test_retnet_bwd(const ProblemShape& ps, Tensors& t) {
     auto launch = [&] {
       if (m == MaskKind::Decay) {
         const float* lg = t.log2_gamma.dev;
-        dv_decay<<<grid_v, block, TV::kSmemBytes, 0>>>(t.k.dev, t.q.dev, t.dout.dev, nullptr, t.r.dev, t.dv.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr);
-        dk_decay<<<grid_k, block, TK::kSmemBytes, 0>>>(t.v.dev, t.dout.dev, t.q.dev, nullptr, t.r.dev, t.dk.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr);
-        dq_decay<<<grid_q, block, TQ::kSmemBytes, 0>>>(t.dout.dev, t.v.dev, t.k.dev, nullptr, t.r.dev, t.dq.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr);
+        dv_decay<<<grid_v, block, TV::kSmemBytes, 0>>>(t.k.dev, t.q.dev, t.dout.dev, nullptr, t.r.dev, t.dv.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr, nullptr);
+        dk_decay<<<grid_k, block, TK::kSmemBytes, 0>>>(t.v.dev, t.dout.dev, t.q.dev, nullptr, t.r.dev, t.dk.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr, nullptr);
+        dq_decay<<<grid_q, block, TQ::kSmemBytes, 0>>>(t.dout.dev, t.v.dev, t.k.dev, nullptr, t.r.dev, t.dq.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr, nullptr);
         return;
       }
       const int mode = m == MaskKind::Dense ? aat::kMaskDense : m == MaskKind::Causal ? aat::kMaskCausal : aat::kMaskScanned;
       aat::MaskWalk walk;
       HIP_OK(aat::prepare_mask_walk(mode, mask, ps.H, ps.Sq, ps.Sk, t.scan, 0, &walk));
-      dv_plain<<<grid_v, block, TV::kSmemBytes, 0>>>(t.k.dev, t.q.dev, t.dout.dev, mask, t.r.dev, t.dv.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents);
-      dk_plain<<<grid_k, block, TK::kSmemBytes, 0>>>(t.v.dev, t.dout.dev, t.q.dev, mask, t.r.dev, t.dk.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents);
-      dq_plain<<<grid_q, block, TQ::kSmemBytes, 0>>>(t.dout.dev, t.v.dev, t.k.dev, mask, t.r.dev, t.dq.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents);
+      dv_plain<<<grid_v, block, TV::kSmemBytes, 0>>>(t.k.dev, t.q.dev, t.dout.dev, mask, t.r.dev, t.dv.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents, nullptr);
+      dk_plain<<<grid_k, block, TK::kSmemBytes, 0>>>(t.v.dev, t.dout.dev, t.q.dev, mask, t.r.dev, t.dk.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents, nullptr);
+      dq_plain<<<grid_q, block, TQ::kSmemBytes, 0>>>(t.dout.dev, t.v.dev, t.k.dev, mask, t.r.dev, t.dq.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents, nullptr);
     };
     for (auto* x : {&t.dq, &t.dk, &t.dv}) HIP_OK(hipMemset(x->dev, 0xff, x->host.size() * sizeof(half_t)));
     launch();
@@ -161,6 +163,69 @@ static void test_retnet_bwd(const ProblemShape& ps, Tensors& t) {
     const aat_bench::Timing tm = aat_bench::do_bench(launch, ps.flush);
     const double fl = 2.0 * ps.B * ps.H * (double)ps.Sq * ps.Sk * (3 * Kd + 2 * D) * share_of_dense(m);
     std::printf("%-52s mask %-6s mean %.4f ms  median %.4f  p20 %.4f  p80 %.4f  (%d launches)  %.1f TFLOP/s = %.1f%% of 2.5 PFLOP/s"
+                "  check: max |err| %.2e of %.2f -> %s\n", name, name_of(m), tm.mean_ms, tm.median_ms, tm.p20_ms, tm.p80_ms, tm.launches,
+                fl / tm.median_ms * 1e-9, fl / tm.median_ms * 1e-9 / 25.0, agree.max_err, agree.max_ref, agree.ok() ? "ok" : "MISMATCH");
+  }
+}
+
+// The same with dS stored by the row pass and read back by a dK kernel of its own
+// <resident rows, streamed rows, threads, Y/Z buffers of the chained passes; kv rows, query rows, threads, stages, waves per SIMD of the dK kernel>
+template <int Br, int Bc, int NT, int NSY, int NSZ, int KBX, int KBY, int KNT, int KNS, int KWPE>
+static void test_retnet_bwd_stored_ds(const ProblemShape& ps, Tensors& t) {
+  constexpr int WPE = 1;
+  constexpr int RTv = Br / (NT / 64) / 32;
+  constexpr int DVB = (WPE == 1 && RTv * D <= 512) ? D : 256;
+  using TV = aat::RetBwdChain<Kd, D, DVB, Br, Bc, NT, NSY, NSZ, BwdPass::Col>;
+  using TQ = aat::RetBwdChain<D, Kd, Kd, Br, Bc, NT, NSY, NSZ, BwdPass::Row>;
+  using TK = aat::RetBwdDk<Kd, KBX, KBY, KNT, KNS>;
+  static_assert(Br % KBY == 0, "a query tile of the dK kernel lies inside one block of the row pass");
+  char name[160];
+  std::snprintf(name, sizeof name, "bwd chain Br=%d Bc=%d thr=%d bufs=%d/%d waves/SIMD=%d dK from dS %dx%d", Br, Bc, NT, NSY, NSZ, WPE, KBX, KBY);
+  if (ps.Sq % Br || ps.Sk % Br || ps.Sq % Bc || ps.Sk % Bc || ps.Sk % KBX || ps.Sq % KBY) {
+    std::printf("%-70s skipped: sequence lengths\n", name);
+    return;
+  }
+  auto dv_plain = &aat::ret_bwd_chain<Kd, D, DVB, Br, Bc, NT, NSY, NSZ, BwdPass::Col, WPE, false>;
+  auto dq_plain = &aat::ret_bwd_chain<D, Kd, Kd, Br, Bc, NT, NSY, NSZ, BwdPass::Row, WPE, false, true>;
+  auto dv_decay = &aat::ret_bwd_chain<Kd, D, DVB, Br, Bc, NT, NSY, NSZ, BwdPass::Col, WPE, true>;
+  auto dq_decay = &aat::ret_bwd_chain<D, Kd, Kd, Br, Bc, NT, NSY, NSZ, BwdPass::Row, WPE, true, true>;
+  auto dk_ds = &aat::ret_bwd_dk_from_ds<Kd, KBX, KBY, KNT, KNS, KWPE>;
+  HIP_OK(hipFuncSetAttribute((const void*)dv_plain, hipFuncAttributeMaxDynamicSharedMemorySize, TV::kSmemBytes));
+  HIP_OK(hipFuncSetAttribute((const void*)dv_decay, hipFuncAttributeMaxDynamicSharedMemorySize, TV::kSmemBytes));
+  HIP_OK(hipFuncSetAttribute((const void*)dq_plain, hipFuncAttributeMaxDynamicSharedMemorySize, TQ::kSmemBytesDsOut));
+  HIP_OK(hipFuncSetAttribute((const void*)dq_decay, hipFuncAttributeMaxDynamicSharedMemorySize, TQ::kSmemBytesDsOut));
+  HIP_OK(hipFuncSetAttribute((const void*)dk_ds, hipFuncAttributeMaxDynamicSharedMemorySize, TK::kSmemBytes));
+  const dim3 block(NT), grid_v(ps.B * ps.H * (ps.Sk / Br), D / DVB), grid_q(ps.B * ps.H * (ps.Sq / Br));
+  const dim3 kblock(KNT), grid_k(ps.B * ps.H * (ps.Sk / KBX));
+  for (MaskKind m : kAllMasks) {
+    if (ps.only && std::strcmp(ps.only, name_of(m))) continue;
+    forward_for(ps, t, m);
+    const half_t* mask = m == MaskKind::Dense ? t.mask_dense.dev : t.mask_decay.dev;
+    auto launch = [&] {
+      if (m == MaskKind::Decay) {
+        const float* lg = t.log2_gamma.dev;
+        dv_decay<<<grid_v, block, TV::kSmemBytes, 0>>>(t.k.dev, t.q.dev, t.dout.dev, nullptr, t.r.dev, t.dv.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr, nullptr);
+        dq_decay<<<grid_q, block, TQ::kSmemBytesDsOut, 0>>>(t.dout.dev, t.v.dev, t.k.dev, nullptr, t.r.dev, t.dq.dev, ps.H, ps.Sk, ps.Sq, 1, lg, nullptr, t.ds);
+        dk_ds<<<grid_k, kblock, TK::kSmemBytes, 0>>>(t.q.dev, t.ds, t.dk.dev, ps.H, ps.Sk, ps.Sq, 1, nullptr, Br, Bc);
+        return;
+      }
+      const int mode = m == MaskKind::Dense ? aat::kMaskDense : m == MaskKind::Causal ? aat::kMaskCausal : aat::kMaskScanned;
+      aat::MaskWalk walk;
+      HIP_OK(aat::prepare_mask_walk(mode, mask, ps.H, ps.Sq, ps.Sk, t.scan, 0, &walk));
+      dv_plain<<<grid_v, block, TV::kSmemBytes, 0>>>(t.k.dev, t.q.dev, t.dout.dev, mask, t.r.dev, t.dv.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents, nullptr);
+      dq_plain<<<grid_q, block, TQ::kSmemBytesDsOut, 0>>>(t.dout.dev, t.v.dev, t.k.dev, mask, t.r.dev, t.dq.dev, ps.H, ps.Sk, ps.Sq, walk.causal, nullptr, walk.extents, t.ds);
+      dk_ds<<<grid_k, kblock, TK::kSmemBytes, 0>>>(t.q.dev, t.ds, t.dk.dev, ps.H, ps.Sk, ps.Sq, walk.causal, walk.extents, Br, Bc);
+    };
+    for (auto* x : {&t.dq, &t.dk, &t.dv}) HIP_OK(hipMemset(x->dev, 0xff, x->host.size() * sizeof(half_t)));
+    HIP_OK(hipMemset(t.ds, 0x7f, (size_t)ps.B * ps.H * ps.Sq * ps.Sk * sizeof(half_t)));     // NaN patterns where nothing is written
+    launch();
+    HIP_OK(hipGetLastError());
+    HIP_OK(hipDeviceSynchronize());
+    const Agreement agree = check_slice(ps, t, m);
+    g_failures += !agree.ok();
+    const aat_bench::Timing tm = aat_bench::do_bench(launch, ps.flush);
+    const double fl = 2.0 * ps.B * ps.H * (double)ps.Sq * ps.Sk * (3 * Kd + 2 * D) * share_of_dense(m);
+    std::printf("%-70s mask %-6s mean %.4f ms  median %.4f  p20 %.4f  p80 %.4f  (%d launches)  %.1f TFLOP/s = %.1f%% of 2.5 PFLOP/s"
                 "  check: max |err| %.2e of %.2f -> %s\n", name, name_of(m), tm.mean_ms, tm.median_ms, tm.p20_ms, tm.p80_ms, tm.launches,
                 fl / tm.median_ms * 1e-9, fl / tm.median_ms * 1e-9 / 25.0, agree.max_err, agree.max_ref, agree.ok() ? "ok" : "MISMATCH");
   }
@@ -197,7 +262,11 @@ int main(int argc, char** argv) {
   t.dk = empty<half_t>(nk);
   t.dv = empty<half_t>(nv);
   HIP_OK(hipMalloc(&t.scan, aat::mask_extent_bytes(ps.H, ps.Sq, ps.Sk)));
+  HIP_OK(hipMalloc(&t.ds, (size_t)ps.B * ps.H * ps.Sq * ps.Sk * sizeof(half_t)));
 
+  test_retnet_bwd_stored_ds<128, 64, 256, 1, 1, 128, 64, 256, 2, 2>(ps, t);
+  test_retnet_bwd_stored_ds<128, 32, 256, 1, 1, 256, 64, 512, 2, 2>(ps, t);
+  test_retnet_bwd_stored_ds<128, 64, 256, 1, 1, 256, 64, 512, 2, 2>(ps, t);
   test_retnet_bwd<128, 32, 256, 3, 2, 1>(ps, t);
   test_retnet_bwd<128, 64, 256, 1, 1, 1>(ps, t);
   test_retnet_bwd<128, 32, 256, 2, 2, 1>(ps, t);
@@ -206,6 +275,7 @@ int main(int argc, char** argv) {
   t.r.release();
   t.log2_gamma.release();
   HIP_OK(hipFree(t.scan));
+  HIP_OK(hipFree(t.ds));
   if (g_failures) std::printf("%d result(s) disagree with the host formulas\n", g_failures);
   return g_failures ? 1 : 0;
 }

@@ -32,6 +32,7 @@
 #include "../../utils/mask_extents.h"
 #include "../../utils/retention.h"
 #include "../../utils/tile_ops.h"
+#include "ds_layout.h"
 
 #ifndef AAT_PF
 #define AAT_PF 4
@@ -68,6 +69,11 @@ struct RetBwdChain {
   static constexpr int kMainBytes = NSY * (kYBytes + kMBytes) + NSZ * kZBytes;
   static constexpr int kEpiBytes = BX * kOStride;
   static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
+  // DS_OUT variant of the row pass: a wave-private staging area behind the stream buffers, in which a dS tile
+  // turns from 8-byte pieces per lane into whole rows
+  static constexpr int kDsStride = BY * 2 + 16;
+  static constexpr int kDsStageBytes = BX * kDsStride;
+  static constexpr int kSmemBytesDsOut = (kMainBytes + kDsStageBytes > kEpiBytes) ? kMainBytes + kDsStageBytes : kEpiBytes;
 };
 
 // x, y, z, out: [B*H, S, width] fp16 with S = seq_x for x/out and seq_y for y/z; mask [H, seq_q, seq_k];
@@ -75,13 +81,16 @@ struct RetBwdChain {
 // `causal` promises mask == 0 above the diagonal and only shortens the walk over streamed tiles.
 // DECAY: the mask is gamma_h^(q + diag - kv) below the diagonal and zero above it, built in registers
 // from lg2gamma[h] = log2(gamma_h); `mask` is not read and tiles above the diagonal are skipped.
+// DS_OUT (row pass only): the fp16 E tiles (= dS) this pass forms are also written to ds_out (64 x 64 blocks, ds_layout.h), for
+// a dK kernel that reads them instead of evaluating them again (dk_from_ds.h).  Only the tiles of the walk are written.
 template <int KX, int DZ, int DZB, int BX, int BY, int Nthreads, int NSY, int NSZ, BwdPass PASS, int WPE = 1,
-          bool DECAY = false>
+          bool DECAY = false, bool DS_OUT = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const half_t* __restrict__ z,
               const half_t* __restrict__ mask, const float* __restrict__ r, half_t* __restrict__ out, int H,
               int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr,
-              const int* __restrict__ extents = nullptr) {
+              const int* __restrict__ extents = nullptr, half_t* __restrict__ ds_out = nullptr) {
+  static_assert(!DS_OUT || PASS == BwdPass::Row, "dS is written by the row pass");
   if constexpr (DECAY) causal = 1;
   using T = RetBwdChain<KX, DZ, DZB, BX, BY, Nthreads, NSY, NSZ, PASS>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCY = T::NCY, NCZ = T::NCZ, NCM = T::NCM, WM = T::WM;
@@ -213,6 +222,7 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   };
   constexpr int kYmInstr = T::YDma::kIters + (DECAY ? 0 : T::MDma::kIters);   // LDS-DMA instructions per thread for one Y (+ mask) tile
   constexpr int kRInstr = COL ? NT * 4 : 0;                     // register loads of r per tile
+  constexpr int kDsInstr = DS_OUT ? RT * BY / 16 : 0;           // 16-byte stores of the dS tile per lane, the youngest memory operations of a tile
   // Issue order (three Y/mask buffers):  prologue  YM(j0) Z(j0) YM(j0+1);  tile j  Z(j+1) YM(j+2).
   // Loads retire in order, so "at most kYmInstr (+ the r loads of the next tile) outstanding" at the top
   // of tile j means YM(j) and Z(j) have landed while YM(j+1) may still be in flight: a Y/mask tile gets
@@ -251,7 +261,7 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
     sched_fence();
     // (A) Y_j and mask_j (and with two Z buffers Z_j) have landed; every wave is past the previous tile.
     if constexpr (NSY == 3) {
-      if (more) wait_vmcnt<kYmInstr + kRInstr>();
+      if (more) wait_vmcnt<kYmInstr + kRInstr + kDsInstr>();
       else wait_vmcnt<0>();
     } else {
       wait_vmcnt<0>();
@@ -343,12 +353,61 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
     if constexpr (NSZ == 1 || NSY == 1) {
       if constexpr (NSZ == 1) wait_vmcnt<0>();
       block_sync();
+    }
+    // What this tile sends to memory from here -- with one Y buffer the copy of the next Y and mask tile, with DS_OUT
+    // the dS tile -- goes out behind the first operand reads of the second contraction.  Where those reads are left
+    // to the compiler (more than one wave per SIMD) it waits in front of the first of them for the Z copy with
+    // vmcnt(0), since it cannot see the wait above, and that would take in everything issued before the read too.
+    const auto send_late = [&]() {
+      sched_fence();
       if constexpr (NSY == 1) {
         if (more) issue_ym(j + 1, 0);
       }
-    }
+      if constexpr (DS_OUT) {
+        // The tile as the second contraction will see it (the same roundings).  A lane holds 8-byte pieces of its row
+        // (kv 8g + 4h .. + 3): stored as they are, every instruction touches 32 rows 16 bytes at a time and the pass
+        // runs a third longer.  Through the wave's staging area they leave as whole rows, 16 bytes per lane.
+        // The LDS accesses are written as instructions: in front of an LDS access it can see, the compiler waits for
+        // every LDS-DMA copy in flight, here the next tile's, which were issued a moment ago.
+        char* const stage = smem + T::kMainBytes + wave * WM * T::kDsStride;
+        const uint32_t st_w = lds_addr(stage + n * T::kDsStride + 8 * h);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const h2 a = pack_rne(tacc[rt][t][4 * g], tacc[rt][t][4 * g + 1]);
+              const h2 b = pack_rne(tacc[rt][t][4 * g + 2], tacc[rt][t][4 * g + 3]);
+              h4 w;
+              w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
+              asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(st_w), "v"(w), "i"(rt * 32 * T::kDsStride + (32 * t + 8 * g) * 2));
+            }
+        wait_lgkm0();                                 // the staging area is private to this wave
+        constexpr int kChunksPerRow = BY / 8, kRowsPerInstr = 64 / kChunksPerRow, kStores = WM * kChunksPerRow / 64;
+        constexpr int kBatch = kStores < 4 ? kStores : 4;                 // reads in flight before their stores
+        static_assert(64 % kChunksPerRow == 0 && kStores % kBatch == 0, "whole rows per store instruction");
+        static_assert(WM <= 64, "a wave's rows lie in one row of dS blocks");
+        const int srow = lane / kChunksPerRow, sc = lane % kChunksPerRow;
+        const uint32_t st_r = lds_addr(stage + srow * T::kDsStride + sc * 16);
+        half_t* const dst = ds_out + ds_block_offset(bh, x0 + wave * WM + srow, jt * BY + sc * 8, seq_q, seq_k);
+#pragma unroll
+        for (int i0 = 0; i0 < kStores; i0 += kBatch) {
+          f4v val[kBatch];
+#pragma unroll
+          for (int i = 0; i < kBatch; ++i) val[i] = lds_read_f4_async(st_r, (i0 + i) * kRowsPerInstr * T::kDsStride);
+          static_for<kBatch>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            lds_wait_younger<kBatch - 1 - i>(val[i]);
+            // rows of one store instruction lie in one 64-row block (kRowsPerInstr divides 64): 64 elements apart
+            __builtin_nontemporal_store(val[i], reinterpret_cast<f4v*>(dst + (size_t)(i0 + i) * kRowsPerInstr * 64));
+          });
+        }
+      }
+    };
     h8 ef[RT][NT][2];
-    pv_gemm_steps<RT, NT, DT, NCZ, PF>(acc, ef, zaddr, zoff, [&](int g) {
+    pv_gemm_steps<RT, NT, DT, NCZ, PF, WPE == 1>(acc, ef, zaddr, zoff, [&](int g) {
+      if (g == 0) send_late();
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) pack_group<NT>(ef[rt], tacc[rt], g);
     });

@@ -198,7 +198,7 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
       }
     }
     h8 pf[RT][NT][2];
-    pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
+    pv_gemm_steps<RT, NT, DT, NCV, PF, WPE == 1>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) pack_group<NT>(pf[rt], sacc[rt], g);
     });

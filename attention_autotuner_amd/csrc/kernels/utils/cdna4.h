@@ -169,7 +169,8 @@ template <int N, int I = 0, class F> AAT_DEV void static_for(F&& f) {
 // or two VGPRs of addressing instead of a 64-bit pointer per instruction.  That works when the block's
 // threads cover whole rows per instruction (NT % NC == 0): then a thread keeps its chunk column and
 // only the swizzle term can change from one instruction to the next, with a short period.
-template <int ROWS, int NC, int NT, Swz MODE>
+// AUX: cache-policy bits of the load (2 = non-temporal: data read once).
+template <int ROWS, int NC, int NT, Swz MODE, int AUX = 0>
 struct TileDma {
   static constexpr int kChunks = ROWS * NC;
   static_assert(kChunks % NT == 0, "tile chunks must divide evenly over the block's threads");
@@ -214,7 +215,7 @@ struct TileDma {
     asm volatile("" : "+s"(base));                     // keep the uniform part in SGPRs (saddr form)
     const uint32_t lane_off = loff[kRegular ? i % kDistinct : i];
     __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)(base + lane_off),
-                                     (AAT_AS3 void*)(lds + (i * NT + wave_base) * 16), 16, 0, 0);
+                                     (AAT_AS3 void*)(lds + (i * NT + wave_base) * 16), 16, 0, AUX);
   }
 };
 

@@ -111,6 +111,27 @@ template <int N> AAT_DEV void lds_wait_younger(f4v& a, f4v& b) {
   asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
 
+// The transposing 8-byte read (lds_read_tr_h4_at) issued the same way, and the wait for a pair of them.
+AAT_DEV h4 lds_read_tr_h4_async(uint32_t base, int imm) {
+  h4 v;
+  const uint32_t hi = (uint32_t)imm & ~0xffffu;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(base + hi), "i"(imm & 0xffff));
+  return v;
+}
+template <int N> AAT_DEV void lds_wait_younger(h4& a, h4& b) {
+  static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
+  asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+
+// One operand read of the second contraction and its wait, either way: BLIND as above, otherwise left to the compiler.
+template <bool BLIND> AAT_DEV h4 lds_read_tr_h4_either(uint32_t base, int imm) {
+  if constexpr (BLIND) return lds_read_tr_h4_async(base, imm);
+  else return lds_read_tr_h4_at(base + imm);
+}
+template <bool BLIND, int N> AAT_DEV void lds_wait_younger_either(h4& a, h4& b) {
+  if constexpr (BLIND) lds_wait_younger<N>(a, b);
+}
+
 // MFMA with its accumulator forced into vector registers.  A kernel that owns more than 256 registers
 // gets every compiler-issued MFMA in the form that accumulates in the 256 accumulation registers; when
 // the output accumulators fill those, the short-lived score tile has to live in vector registers, which
@@ -178,40 +199,50 @@ AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const u
 // transposing reads of d-tile dt (kv rows 4h..4h+3 and 8+4h..8+4h+3 of the first 16-row step; later steps
 // add 16 rows, which no swizzle here sees).  pack(g) must fill pf[*][g/2][g%2] (the P operand of kv rows
 // 16g .. 16g+15); it is called one group ahead of use, between MFMAs.
-template <int RT, int NT, int DT, int NCV, int PF, class Pack>
+// BLIND: the V reads are issued behind the compiler's back like the K reads above.  In front of an LDS read it
+// can see the compiler waits, with vmcnt(0), for every LDS-DMA copy in flight -- the next tile's, issued at the
+// top of this one, which then has only the first contraction to arrive in instead of the whole tile.  With one
+// wave on the SIMD nothing covers that wait (RetNet forward at d_qk 256 / d_v 512: -6 % with BLIND); with two or
+// three another wave does, and the counted waits cost a little instead (attention forward, causal: +1.5 %).
+// buf_off must fold to a constant.
+template <int RT, int NT, int DT, int NCV, int PF, bool BLIND = false, class Pack>
 AAT_DEV void pv_gemm_steps_hl(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint32_t (&vlo)[DT],
                               const uint32_t (&vhi)[DT], int buf_off, Pack&& pack) {
   constexpr int G = NT * 2;              // groups of 16 kv rows
   constexpr int S = G * DT;
   constexpr int kRow16 = 16 * NCV * 16;
+  static_assert(!BLIND || 2 * PF < 16, "two reads per step in flight, counted by a 4-bit counter");
   h4 lo[PF], hi[PF];
 #pragma unroll
   for (int i = 0; i < PF && i < S; ++i) {
-    lo[i] = lds_read_tr_h4_at(vlo[i % DT] + buf_off + (i / DT) * kRow16);
-    hi[i] = lds_read_tr_h4_at(vhi[i % DT] + buf_off + (i / DT) * kRow16);
+    lo[i] = lds_read_tr_h4_either<BLIND>(vlo[i % DT], buf_off + (i / DT) * kRow16);
+    hi[i] = lds_read_tr_h4_either<BLIND>(vhi[i % DT], buf_off + (i / DT) * kRow16);
   }
   pack(0);
   sched_fence();
-#pragma unroll
-  for (int step = 0; step < S; ++step) {
-    const int g = step / DT, dt = step % DT;
-    const h8 vf = cat_h4(lo[step % PF], hi[step % PF]);
-    if (step + PF < S) {
-      const int nx = step + PF;
-      lo[step % PF] = lds_read_tr_h4_at(vlo[nx % DT] + buf_off + (nx / DT) * kRow16);
-      hi[step % PF] = lds_read_tr_h4_at(vhi[nx % DT] + buf_off + (nx / DT) * kRow16);
+  static_for<S>([&](auto step_tag) {
+    constexpr int step = decltype(step_tag)::value;
+    constexpr int g = step / DT, dt = step % DT;
+    h4 clo = lo[step % PF], chi = hi[step % PF];
+    if constexpr (step + PF < S) {
+      constexpr int nx = step + PF;
+      lo[step % PF] = lds_read_tr_h4_either<BLIND>(vlo[nx % DT], buf_off + (nx / DT) * kRow16);
+      hi[step % PF] = lds_read_tr_h4_either<BLIND>(vhi[nx % DT], buf_off + (nx / DT) * kRow16);
     }
+    lds_wait_younger_either<BLIND, 2 * ((step + PF < S) ? PF : S - 1 - step)>(clo, chi);
+    const h8 vf = cat_h4(clo, chi);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
-    if (dt == 0 && g + 1 < G) pack(g + 1);
+    if constexpr (dt == 0 && g + 1 < G) pack(g + 1);
     sched_fence();
-  }
+  });
 }
 
 // O^T += V^T P^T over one kv tile.  vaddr[dt] = LDS address this lane presents to the transposing read
 // for d-tile dt, kv rows 0..3 (+4h) of the V buffer.  pack(g) must fill pf[*][g/2][g%2] (the P operand of
 // kv rows 16g .. 16g+15); it is called one group ahead of use, between MFMAs.
-template <int RT, int NT, int DT, int NCV, int PF, class Pack>
+// BLIND: as in pv_gemm_steps_hl.
+template <int RT, int NT, int DT, int NCV, int PF, bool BLIND = false, class Pack>
 AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint32_t (&vaddr)[DT], int buf_off,
                            Pack&& pack) {
   constexpr int G = NT * 2;              // groups of 16 kv rows
@@ -221,29 +252,34 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
   // is four chunks wide: d-tile dt sits 256 bytes per group behind d-tile dt % 4, so four address registers
   // serve any output width (the others are never read and cost nothing).
   constexpr bool kFold = NCV % 16 == 0 && DT > 4;
-  auto addr = [&](int i) { return (kFold ? vaddr[(i % DT) % 4] + ((i % DT) / 4) * 256 : vaddr[i % DT]) + buf_off + (i / DT) * kRow16; };
+  static_assert(!BLIND || 2 * PF < 16, "two reads per step in flight, counted by a 4-bit counter");
+  auto read = [&](int i, int half) {
+    return lds_read_tr_h4_either<BLIND>(kFold ? vaddr[(i % DT) % 4] : vaddr[i % DT],
+                                (kFold ? ((i % DT) / 4) * 256 : 0) + buf_off + (i / DT) * kRow16 + half * kRow8);
+  };
   h4 lo[PF], hi[PF];
 #pragma unroll
   for (int i = 0; i < PF && i < S; ++i) {
-    lo[i] = lds_read_tr_h4_at(addr(i));
-    hi[i] = lds_read_tr_h4_at(addr(i) + kRow8);
+    lo[i] = read(i, 0);
+    hi[i] = read(i, 1);
   }
   pack(0);
   sched_fence();
-#pragma unroll
-  for (int step = 0; step < S; ++step) {
-    const int g = step / DT, dt = step % DT;
-    const h8 vf = cat_h4(lo[step % PF], hi[step % PF]);
-    if (step + PF < S) {
-      const int nx = step + PF;
-      lo[step % PF] = lds_read_tr_h4_at(addr(nx));
-      hi[step % PF] = lds_read_tr_h4_at(addr(nx) + kRow8);
+  static_for<S>([&](auto step_tag) {
+    constexpr int step = decltype(step_tag)::value;
+    constexpr int g = step / DT, dt = step % DT;
+    h4 clo = lo[step % PF], chi = hi[step % PF];
+    if constexpr (step + PF < S) {
+      lo[step % PF] = read(step + PF, 0);
+      hi[step % PF] = read(step + PF, 1);
     }
+    lds_wait_younger_either<BLIND, 2 * ((step + PF < S) ? PF : S - 1 - step)>(clo, chi);
+    const h8 vf = cat_h4(clo, chi);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
-    if (dt == 0 && g + 1 < G) pack(g + 1);
+    if constexpr (dt == 0 && g + 1 < G) pack(g + 1);
     sched_fence();
-  }
+  });
 }
 
 // Epilogue: scale the wave's O^T accumulators per row, convert (fp16 with RNE, or fp32 as is),

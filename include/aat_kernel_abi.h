@@ -27,7 +27,8 @@
  *     flag, an optional workspace and the stream to launch on (a hipStream_t passed as void*);
  *   - workspace_size() says how many bytes of workspace a problem needs (attention forward: 0 unless the
  *     configuration splits the kv range; RetNet: the mask scan of AAT_MASK_SCAN, not needed by the other
- *     mask modes); abi_version() and config_string() identify the library.
+ *     mask modes, and for a backward built with a stored dS the optional room for it); abi_version() and
+ *     config_string() identify the library.
  */
 #ifndef AAT_KERNEL_ABI_H
 #define AAT_KERNEL_ABI_H
@@ -110,7 +111,11 @@ int kernel_entry_decay(aat_half* q, aat_half* k, aat_half* v, const float* log2_
 
 #elif defined(AAT_OP_RET_BWD)
 /* RetNet parallel backward.  Replaces: reference csrc/kernels/retnet/bwd/profile_code.py:53 and :98.
- * dqaccum is fp32 scratch the caller has zeroed; dq, dk, dv are fully overwritten. */
+ * dqaccum is fp32 scratch the caller has zeroed; dq, dk, dv are fully overwritten.
+ * A library built with a stored dS (configuration field ds_rows != 0) reports B*H*Seq_q*Seq_k fp16 more in
+ * workspace_size(): given that room, the dQ pass writes the dS tiles it forms and dK comes from a kernel that
+ * reads them back; given less (or none, as through the reference-signature entry points) dK comes from the
+ * chained pass that evaluates dS a second time, with the results of a library built without it. */
 float profile(aat_half* q, aat_half* k, aat_half* v, aat_half* mask, aat_half* dO, float* r,
               aat_half* dq, aat_half* dk, aat_half* dv, float* dqaccum, int B, int H, int Seq_q,
               int Seq_k);

@@ -3,7 +3,7 @@ same thing.  ``parity_configs()`` lists them so the build step can compile them 
 compiled inside a GPU test)."""
 from attention_autotuner_amd.arch import MI355X
 from attention_autotuner_amd.autotuner import gfx950_space
-from attention_autotuner_amd.autotuner.configs import AttnBwdConfig, AttnConfig, RetConfig
+from attention_autotuner_amd.autotuner.configs import AttnBwdConfig, AttnConfig, RetBwdConfig, RetConfig
 
 # attention forward, register-fused: (Br, Bc, Nthreads, K buffers, V buffers, waves per SIMD) for every head-size pair below
 PARITY_TILES = [
@@ -47,6 +47,16 @@ def ret_shared_wide_one_wave():
     return cfg
 
 
+# RetNet backward with dS stored by the dQ pass and read back by a dK kernel of its own: (d_qk, d_v, Br, Bc, threads, kv rows of the dK kernel)
+RET_BWD_STORED_DS = [(256, 512, 128, 64, 256, 128), (256, 512, 128, 64, 256, 256), (256, 512, 128, 32, 256, 256), (64, 128, 64, 32, 128, 128)]
+
+
+def ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, ds_rows, stages=(1, 1)):
+    n = nt // 64
+    return RetBwdConfig(br, bc, dqk, dv, n, n, n, n, nt, True, BlockKSmem=dqk, num_stages_qk=stages[0], num_stages_mask=stages[0],
+                        num_stages_dv=stages[1], waves_per_eu=1, ds_rows=ds_rows)
+
+
 def parity_configs(arch=None):
     arch = arch or MI355X()
     out = []
@@ -61,6 +71,8 @@ def parity_configs(arch=None):
                 out.append(cfg)
     out.append(ret_register_wide())
     out.append(ret_shared_wide_one_wave())
+    for t in RET_BWD_STORED_DS:
+        out += [ret_bwd_stored_ds_config(*t), ret_bwd_stored_ds_config(*t[:5], 0)]      # and the same passes without it
     out += [attn_bwd_split_config(*t) for t in ATTN_BWD_SPLIT_TILES]
     out.append(AttnBwdConfig(64, 64, 128, 128, 128, 2, row_waves_per_eu=2, row_Bc=32))      # row kernel with a tile height of its own
     for br, bc, nt, st in ATTN_BWD_TILES:

@@ -62,14 +62,17 @@ def test_retnet_recurrent_bench_checks_one_slice_and_reports():
     assert re.search(r"median [\d.]+ .* TFLOP/s", out)
 
 
-RET_LINE = re.compile(r"^(smemfuse|regfuse|bwd chain)\s+Br=(\d+) Bc=(\d+) thr=(\d+) bufs=(\S+) (?:grid=(\S+) )?waves/SIMD=(\d+)\s+mask (\w+)\s+"
-                      r"mean ([\d.]+) ms\s+median ([\d.]+).*-> (ok|MISMATCH)")
+RET_LINE = re.compile(r"^(?P<kind>smemfuse|regfuse|bwd chain)\s+Br=(?P<br>\d+) Bc=(?P<bc>\d+) thr=(?P<thr>\d+) bufs=(?P<bufs>\S+) (?:grid=(?P<grid>\S+) )?"
+                      r"waves/SIMD=(?P<waves>\d+)(?: dK from dS (?P<ds>\d+)x\d+)?\s+mask (?P<mask>\w+)\s+"
+                      r"mean [\d.]+ ms\s+median (?P<median>[\d.]+).*-> (?P<verdict>ok|MISMATCH)")
 
 
 def _retnet_rows(out):
+    """(kind, Br, Bc, threads, buffers, grid, waves per SIMD, mask mode, kv rows of the dK-from-dS kernel or None) -> median ms"""
     rows = [m for m in (RET_LINE.match(l) for l in out.splitlines()) if m]
-    assert rows and all(m[11] == "ok" for m in rows), out                  # the programs check a slice of every result on the host
-    return {(m[1], int(m[2]), int(m[3]), int(m[4]), m[5], m[6], int(m[7]), m[8]): float(m[10]) for m in rows}
+    assert rows and all(m["verdict"] == "ok" for m in rows), out           # the programs check a slice of every result on the host
+    return {(m["kind"], int(m["br"]), int(m["bc"]), int(m["thr"]), m["bufs"], m["grid"], int(m["waves"]), m["mask"],
+             int(m["ds"]) if m["ds"] else None): float(m["median"]) for m in rows}
 
 
 def _retnet_tensors(b, h, s, dqk=256, dv=512):
@@ -88,10 +91,11 @@ def test_retnet_bench_checks_every_mask_mode_and_agrees_with_the_library_timing(
     out = _run("retnet_bench", "4", "8", "2048", "2048", "--mask", "dense", "--no-flush")
     print(out)
     times = _retnet_rows(out)
-    key = ("smemfuse", 128, 64, 512, "1/1/1", "2x8", 2, "dense")
     from attention_autotuner_amd.autotuner import prebuilt
+    # the configuration the tuner recorded for this problem's dense walk; its library is part of the shipped set
     cfg = next(c for c in prebuilt.cached_configs() if c.operation == "ret" and (c.Kd, c.D) == (256, 512)
-               and (c.Br, c.Bc, c.Nthreads, c.warps_mma1_n, c.warps_mma_n, c.waves_per_eu) == (128, 64, 512, 2, 8, 2))
+               and (c.fuse_type, c.Br, c.Bc, c.Nthreads, c.waves_per_eu) == ("register", 128, 64, 256, 1))
+    key = ("regfuse", 128, 64, 256, "1/1/1", None, 1, "dense", None)
     q, k, v, _, mask = _retnet_tensors(4, 8, 2048)
     o = torch.empty_like(v)
     r = torch.empty(4, 8, 2048, device="cuda", dtype=torch.float32)
@@ -104,15 +108,16 @@ def test_retnet_bench_checks_every_mask_mode_and_agrees_with_the_library_timing(
 
 def test_retnet_bwd_bench_checks_every_mask_mode_and_agrees_with_the_library_timing():
     small = _retnet_rows(_run("retnet_bwd_bench", "1", "2", "256", "256", "--no-flush"))
-    assert {key[7] for key in small} == {"dense", "causal", "scan", "decay"} and len(small) == 12
+    assert {key[7] for key in small} == {"dense", "causal", "scan", "decay"} and len(small) == 24
+    assert {key[8] for key in small} == {None, 128, 256}
     out = _run("retnet_bwd_bench", "4", "8", "2048", "2048", "--mask", "dense", "--no-flush")
     print(out)
     times = _retnet_rows(out)
-    key = ("bwd chain", 128, 64, 256, "1/1", None, 1, "dense")
+    key = ("bwd chain", 128, 64, 256, "1/1", None, 1, "dense", 256)
     from attention_autotuner_amd.autotuner import prebuilt
     # the configuration the tuner recorded for this problem's dense walk; its library is part of the shipped set
     cfg = next(c for c in prebuilt.cached_configs() if c.operation == "ret_bwd" and (c.Kd, c.D) == (256, 512)
-               and (c.Br, c.Bc, c.Nthreads, c.num_stages_qk, c.num_stages_dv, c.waves_per_eu) == (128, 64, 256, 1, 1, 1))
+               and (c.Br, c.Bc, c.Nthreads, c.num_stages_qk, c.num_stages_dv, c.waves_per_eu, c.ds_rows) == (128, 64, 256, 1, 1, 1, 256))
     q, k, v, do, mask = _retnet_tensors(4, 8, 2048)
     r = torch.full((4, 8, 2048), 1000.0, device="cuda", dtype=torch.float32)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)

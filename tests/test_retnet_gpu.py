@@ -396,3 +396,98 @@ def test_scanned_forward_and_backward_replay_from_a_captured_graph():
             assert torch.equal(got, want)
         o_ref, r_ref = ref_op.retnet_ref(q2, k2, v2, m2, return_r=True)
         tolerance.assert_close(o, o_ref, f"captured scanned forward seed={seed}")
+
+
+# ------------------------------------------------------------------------ dS stored by the dQ pass, read by the dK kernel
+def _poisoned(nbytes):
+    return torch.full((nbytes,), 0x7f, dtype=torch.uint8, device="cuda")       # fp16 NaN wherever nothing gets written
+
+
+def _bwd_through(cfg, arrays, mode, scan_of=None, decay=False):
+    """dq, dk, dv of one backward launch of ``cfg`` with a NaN-filled workspace; ``scan_of``: the forward runtime whose
+    scan the "scanned" mode reuses."""
+    q, k, v, mask, do, r = arrays
+    rt = Runtime(ARCH, cfg)
+    b, h, sq, sk = q.shape[0], q.shape[1], q.shape[2], k.shape[2]
+    outs = [torch.full_like(t, float("nan")) for t in (q, k, v)]
+    tail = [] if decay else [torch.zeros(1, device="cuda")]
+    need = rt.workspace_size(b, h, sq, sk)
+    ws = _poisoned(max(need, scan_of.workspace_size(b, h, sq, sk) if scan_of is not None else 0))
+    if mode == "scanned":                       # the forward's scan lands at the head of the backward's own buffer ...
+        o = torch.empty(b, h, sq, v.shape[-1], dtype=torch.float16, device="cuda")
+        scan_of.apply([q, k, v, mask, o, torch.empty_like(r)], causal="scan", workspace=ws)
+    rt.apply([q, k, v, mask, do, r, *outs, *tail], causal=mode, workspace=ws, decay=decay)
+    if mode == "scanned" and scan_of.workspace_size(b, h, sq, sk) < need:
+        # ... or in the forward's smaller one, which the runtime then moves into one of the backward's size
+        small = ws[:scan_of.workspace_size(b, h, sq, sk)].clone()
+        again = [torch.full_like(t, float("nan")) for t in (q, k, v)]
+        rt.apply([q, k, v, mask, do, r, *again, *tail], causal=mode, workspace=small)
+        for a, c in zip(outs, again):
+            assert torch.equal(a, c)
+    torch.cuda.synchronize()
+    return outs
+
+
+@pytest.mark.parametrize("dqk,dv,br,bc,nt,ds_rows", __import__("parity_matrix").RET_BWD_STORED_DS)
+@pytest.mark.parametrize("sq,sk", [(256, 256), (256, 512), (512, 256)])
+def test_backward_with_a_stored_ds_agrees_with_the_one_that_evaluates_it_twice(dqk, dv, br, bc, nt, ds_rows, sq, sk):
+    """The dQ pass writes only the dS tiles it walks, so the workspace is full of NaN elsewhere and the dK kernel must
+    take exactly the written part: dense, causal-promise and scanned walks of a decay mask, a banded mask, S_q != S_kv."""
+    import parity_matrix
+    with_ds = parity_matrix.ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, ds_rows)
+    plain = parity_matrix.ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, 0)
+    assert gfx950_space.backward_valid(with_ds, ARCH) and os.path.exists(codegen.library_path(with_ds))
+    b, h = 2, 3
+    q, k, v, do, gamma, exact = _decay_problem(b, h, sq, sk, dqk, dv, seed=sq + sk + ds_rows)
+    mask = exact.half()                              # zero above the diagonal that ends in the last row and column
+    band = mask * ((torch.arange(sq).view(1, sq, 1) + (sk - sq) - torch.arange(sk).view(1, 1, sk)) < 160).half()
+    fwd = Runtime(ARCH, gfx950_space.default_forward_config("ret", dqk, dv, ARCH, sq, sk))
+    rt = Runtime(ARCH, with_ds)
+    assert rt.workspace_size(b, h, sq, sk) >= b * h * sq * sk * 2 + fwd.workspace_size(b, h, sq, sk)
+    for name, m, modes in (("decay", mask, (False, True, "scanned")), ("band", band, (False, "scanned"))):
+        _, r_ref = ref_op.retnet_ref(q, k, v, m, return_r=True)
+        dev = [t.cuda() for t in (q, k, v, m, do)] + [r_ref.cuda().contiguous()]
+        for mode in modes:
+            got = _bwd_through(with_ds, dev, mode, scan_of=fwd)
+            want = _bwd_through(plain, dev, mode, scan_of=fwd)
+            assert torch.equal(got[0], want[0]) and torch.equal(got[2], want[2]), (name, mode)      # dQ and dV: the same kernels
+            assert bool(torch.isfinite(got[1].float()).all()), (name, mode)
+            _grads_close(f"stored dS {name} walk={mode}", got, q, k, v, m, do, r_ref)
+    # the decay rates in registers
+    _, r_ref = ref_op.retnet_ref(q, k, v, exact, return_r=True)
+    dev = [t.cuda() for t in (q, k, v)] + [torch.log2(gamma).float().cuda(), do.cuda(), r_ref.cuda().contiguous()]
+    got = _bwd_through(with_ds, dev, True, decay=True)
+    _grads_close("stored dS decay rates", got, q, k, v, exact, do, r_ref)
+
+
+def test_without_room_for_ds_the_library_evaluates_it_twice():
+    """The reference-signature entry points have no workspace to give, and a caller of the others may give a small one or
+    none: dK then comes from the chained pass, and the results are those of the library built without the stored dS."""
+    import parity_matrix
+    t = parity_matrix.RET_BWD_STORED_DS[0]
+    libs = [library.load(Runtime(ARCH, parity_matrix.ret_bwd_stored_ds_config(*t[:5], rows))._path(), "ret_bwd") for rows in (t[5], 0)]
+    q, k, v, mask, do = (x.cuda() for x in _inputs(1, 2, 256, 256, 256, 512, seed=5))
+    r = torch.full((1, 2, 256), 30.0, device="cuda")
+    need = libs[0].workspace_size(1, 2, 256, 256)
+    assert need >= 2 * 256 * 256 * 2 > libs[1].workspace_size(1, 2, 256, 256)
+    assert libs[0].workspace_size(1, 2, 256, 192) == libs[1].workspace_size(1, 2, 256, 192)      # lengths the dK kernel's tiles do not fit
+    small = torch.empty(need - 256, dtype=torch.uint8, device="cuda")
+    got = {}
+    for name, lib in zip(("stored", "plain"), libs):
+        for how in ("reference signature", "no workspace", "small workspace"):
+            outs = [torch.full_like(x, float("nan")) for x in (q, k, v)]
+            ptrs = [ctypes.c_void_p(x.data_ptr()) for x in (q, k, v, mask, do, r, *outs, torch.zeros(1, device="cuda"))]
+            if how == "reference signature":
+                assert lib.kernel_entry(*ptrs, 1, 2, 256, 256) == 0
+            elif how == "no workspace":
+                assert lib.kernel_entry_ex(*ptrs, 1, 2, 256, 256, 1, None, 0, None) == 0
+            else:
+                assert lib.kernel_entry_ex(*ptrs, 1, 2, 256, 256, 1, ctypes.c_void_p(small.data_ptr()), small.numel(), None) == 0
+            torch.cuda.synchronize()
+            got[name, how] = outs
+    for how in ("reference signature", "no workspace", "small workspace"):
+        for a, b in zip(got["stored", how], got["plain", how]):
+            assert torch.equal(a, b), how
+    # the scanning modes still need their ranges
+    ptrs = [ctypes.c_void_p(x.data_ptr()) for x in (q, k, v, mask, do, r, *got["plain", "no workspace"], torch.zeros(1, device="cuda"))]
+    assert libs[0].kernel_entry_ex(*ptrs, 1, 2, 256, 256, 3, None, 0, None) == -3
