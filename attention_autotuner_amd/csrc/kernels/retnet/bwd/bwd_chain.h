@@ -264,7 +264,9 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
       if (more) wait_vmcnt<kYmInstr + kRInstr + kDsInstr>();
       else wait_vmcnt<0>();
     } else {
-      wait_vmcnt<0>();
+      // the previous tile's dS stores are the youngest memory operations in flight and nobody waits for them
+      if (DS_OUT && j > j_begin) wait_vmcnt<kDsInstr>();
+      else wait_vmcnt<0>();
     }
     block_sync();
     // The copies this tile starts -- Z_j (one Z buffer) or Z_{j+1} (two), then Y/mask_{j+1} (two Y buffers) or
@@ -354,60 +356,68 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
       if constexpr (NSZ == 1) wait_vmcnt<0>();
       block_sync();
     }
+    // DS_OUT: the tile as the second contraction will see it (the same roundings).  A lane holds 8-byte pieces of its
+    // row (kv 8g + 4h .. + 3): stored as they are, every instruction touches 32 rows 16 bytes at a time and the pass
+    // runs a third longer.  Through a wave-private staging area they leave as whole rows, 16 bytes per lane.  The three
+    // steps -- into the staging area, back out of it, to memory -- ride along with successive groups of the second
+    // contraction, so the latency of each passes under matrix instructions; LDS executes a wave's instructions in
+    // order, so the reads need no wait for the writes.  The LDS accesses are written as instructions: in front of an
+    // LDS access it can see, the compiler waits for every LDS-DMA copy in flight, here the next tile's.
+    constexpr int kChunksPerRow = BY / 8, kRowsPerInstr = 64 / kChunksPerRow, kStores = DS_OUT ? WM * kChunksPerRow / 64 : 1;
+    static_assert(!DS_OUT || (64 % kChunksPerRow == 0 && WM <= 64), "whole rows per store instruction, in one row of dS blocks");
+    static_assert(!DS_OUT || kStores <= 8, "reads of the staging area in flight");
+    char* const stage = smem + T::kMainBytes + wave * WM * T::kDsStride;
+    f4v staged[kStores];
+    const auto ds_stage = [&]() {
+      const uint32_t st_w = lds_addr(stage + n * T::kDsStride + 8 * h);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const h2 a = pack_rne(tacc[rt][t][4 * g], tacc[rt][t][4 * g + 1]);
+            const h2 b = pack_rne(tacc[rt][t][4 * g + 2], tacc[rt][t][4 * g + 3]);
+            h4 w;
+            w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
+            asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(st_w), "v"(w), "i"(rt * 32 * T::kDsStride + (32 * t + 8 * g) * 2));
+          }
+    };
+    const auto ds_fetch = [&]() {
+      const uint32_t st_r = lds_addr(stage + (lane / kChunksPerRow) * T::kDsStride + (lane % kChunksPerRow) * 16);
+#pragma unroll
+      for (int i = 0; i < kStores; ++i) staged[i] = lds_read_f4_async(st_r, i * kRowsPerInstr * T::kDsStride);
+    };
+    const auto ds_store = [&]() {
+      half_t* const dst = ds_out + ds_block_offset(bh, x0 + wave * WM + lane / kChunksPerRow, jt * BY + (lane % kChunksPerRow) * 8, seq_q, seq_k);
+      static_for<kStores>([&](auto i_tag) {
+        constexpr int i = decltype(i_tag)::value;
+        lds_wait_younger<kStores - 1 - i>(staged[i]);
+        // rows of one store instruction lie in one 64-row block (kRowsPerInstr divides 64): 64 elements apart
+        __builtin_nontemporal_store(staged[i], reinterpret_cast<f4v*>(dst + (size_t)i * kRowsPerInstr * 64));
+      });
+    };
     // What this tile sends to memory from here -- with one Y buffer the copy of the next Y and mask tile, with DS_OUT
     // the dS tile -- goes out behind the first operand reads of the second contraction.  Where those reads are left
     // to the compiler (more than one wave per SIMD) it waits in front of the first of them for the Z copy with
     // vmcnt(0), since it cannot see the wait above, and that would take in everything issued before the read too.
-    const auto send_late = [&]() {
-      sched_fence();
-      if constexpr (NSY == 1) {
-        if (more) issue_ym(j + 1, 0);
+    constexpr int G = NT * 2;                       // groups of the second contraction
+    const auto ride_along = [&](int g) {
+      if (g == 0) {
+        sched_fence();
+        if constexpr (NSY == 1) {
+          if (more) issue_ym(j + 1, 0);
+        }
+        if constexpr (DS_OUT) ds_stage();
       }
       if constexpr (DS_OUT) {
-        // The tile as the second contraction will see it (the same roundings).  A lane holds 8-byte pieces of its row
-        // (kv 8g + 4h .. + 3): stored as they are, every instruction touches 32 rows 16 bytes at a time and the pass
-        // runs a third longer.  Through the wave's staging area they leave as whole rows, 16 bytes per lane.
-        // The LDS accesses are written as instructions: in front of an LDS access it can see, the compiler waits for
-        // every LDS-DMA copy in flight, here the next tile's, which were issued a moment ago.
-        char* const stage = smem + T::kMainBytes + wave * WM * T::kDsStride;
-        const uint32_t st_w = lds_addr(stage + n * T::kDsStride + 8 * h);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const h2 a = pack_rne(tacc[rt][t][4 * g], tacc[rt][t][4 * g + 1]);
-              const h2 b = pack_rne(tacc[rt][t][4 * g + 2], tacc[rt][t][4 * g + 3]);
-              h4 w;
-              w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
-              asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(st_w), "v"(w), "i"(rt * 32 * T::kDsStride + (32 * t + 8 * g) * 2));
-            }
-        wait_lgkm0();                                 // the staging area is private to this wave
-        constexpr int kChunksPerRow = BY / 8, kRowsPerInstr = 64 / kChunksPerRow, kStores = WM * kChunksPerRow / 64;
-        constexpr int kBatch = kStores < 4 ? kStores : 4;                 // reads in flight before their stores
-        static_assert(64 % kChunksPerRow == 0 && kStores % kBatch == 0, "whole rows per store instruction");
-        static_assert(WM <= 64, "a wave's rows lie in one row of dS blocks");
-        const int srow = lane / kChunksPerRow, sc = lane % kChunksPerRow;
-        const uint32_t st_r = lds_addr(stage + srow * T::kDsStride + sc * 16);
-        half_t* const dst = ds_out + ds_block_offset(bh, x0 + wave * WM + srow, jt * BY + sc * 8, seq_q, seq_k);
-#pragma unroll
-        for (int i0 = 0; i0 < kStores; i0 += kBatch) {
-          f4v val[kBatch];
-#pragma unroll
-          for (int i = 0; i < kBatch; ++i) val[i] = lds_read_f4_async(st_r, (i0 + i) * kRowsPerInstr * T::kDsStride);
-          static_for<kBatch>([&](auto i_tag) {
-            constexpr int i = decltype(i_tag)::value;
-            lds_wait_younger<kBatch - 1 - i>(val[i]);
-            // rows of one store instruction lie in one 64-row block (kRowsPerInstr divides 64): 64 elements apart
-            __builtin_nontemporal_store(val[i], reinterpret_cast<f4v*>(dst + (size_t)(i0 + i) * kRowsPerInstr * 64));
-          });
-        }
+        if (g == 1) ds_fetch();
+        if (g == (G > 2 ? 2 : 1)) ds_store();
       }
     };
     h8 ef[RT][NT][2];
     pv_gemm_steps<RT, NT, DT, NCZ, PF, WPE == 1>(acc, ef, zaddr, zoff, [&](int g) {
-      if (g == 0) send_late();
+      ride_along(g);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) pack_group<NT>(ef[rt], tacc[rt], g);
     });
