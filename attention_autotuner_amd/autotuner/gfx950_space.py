@@ -169,6 +169,13 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
     """A configuration that is valid for every supported head size; used before/without tuning."""
     prefs = [(256, 64, 512, 2, 2, 2), (128, 64, 256, 2, 2, 2), (128, 64, 256, 1, 1, 2), (128, 64, 256, 1, 1, 1), (128, 32, 256, 1, 1, 1),
              (64, 32, 128, 1, 1, 1)]
+    if op == "ret" and dim_v == 512 and not ((seq_q and seq_q % 128) or (seq_k and seq_k % 64)):
+        # 32 rows x 512 columns per wave fill the 256 accumulation registers of a wave that has its SIMD to itself;
+        # the RetNet kernel is written so that this builds without scratch, and at d_qk 256 it leads every mask mode
+        cfg = RetConfig(128, 64, dim_qk, dim_v, dim_qk, 64, 1, 1, 1, 256, True, waves_per_eu=1)
+        cfg.set_fuse_type("register")
+        if forward_valid(cfg, arch):
+            return cfg
     for br, bc, nt, sq, sv, wpe in prefs:
         if (seq_q and seq_q % br) or (seq_k and seq_k % bc):
             continue
@@ -288,8 +295,11 @@ def backward_candidates(br, bc, dim_qk, dim_v):
 
 
 def default_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
-    for br, bc, nt, sy, sz, wpe in ((128, 32, 256, 3, 2, 1), (128, 32, 256, 2, 2, 1), (64, 32, 128, 2, 2, 1), (64, 32, 128, 1, 1, 1),
-                                    (64, 32, 128, 1, 1, 2), (64, 64, 128, 1, 1, 1)):
+    prefs = ((128, 32, 256, 3, 2, 1), (128, 32, 256, 2, 2, 1), (64, 32, 128, 2, 2, 1), (64, 32, 128, 1, 1, 1), (64, 32, 128, 1, 1, 2),
+             (64, 64, 128, 1, 1, 1))
+    if dim_v == 512:            # measured at d_qk 256: 64-row streamed tiles with single buffers lead the three-buffer ring of 32-row tiles
+        prefs = ((128, 64, 256, 1, 1, 1),) + prefs
+    for br, bc, nt, sy, sz, wpe in prefs:
         if any(s and (s % br or s % bc) for s in (seq_q, seq_k)):
             continue
         n = nt // WAVE
