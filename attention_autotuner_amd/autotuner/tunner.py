@@ -113,9 +113,9 @@ class RetBwdTunner(BaseTunner):
             return gfx950_space.backward_valid(config, self.arch)
         return _foreign_space(self.arch).backward_valid(config, self.arch)
 
-    def _kernel_matters(self, mangled):                   # ret_bwd_chain<..., PASS, WPE, DECAY>
+    def _kernel_matters(self, mangled):                   # ret_bwd_chain<..., PASS, WPE, DECAY, DS_OUT>; the dK-from-dS kernel has no flags
         flags = codegen.template_bools(mangled)
-        return not flags or flags[-1] == bool(self.decay)
+        return len(flags) != 2 or flags[0] == bool(self.decay)
 
     def tune(self, *a, **kw):
         if not _is_rocm(self.arch):

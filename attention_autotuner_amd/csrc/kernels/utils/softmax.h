@@ -11,15 +11,21 @@ namespace aat {
 // running sum and output are rescaled.
 constexpr float kLazyLog2 = 8.0f;
 
-// max over the lane's registers of NT score tiles
+// max over the lane's registers of NT score tiles: one v_max3_f32 per two values, four chains.  Written as the
+// instruction because hipcc re-associates fmaxf(m, fmaxf(a, b)) into two v_max_f32 and a v_max3_f32 per four
+// values (48 instructions for 64 values instead of 34).
+AAT_DEV float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
 template <int NT> AAT_DEV float lane_max(const f16v (&s)[NT]) {
-  float m = -INFINITY;
+  float m[4];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
+  for (int i = 0; i < 4; ++i) m[i] = fmaxf(s[0][2 * i], s[0][2 * i + 1]);
 #pragma unroll
-    for (int v = 0; v < 16; v += 2) m = fmaxf(m, fmaxf(s[t][v], s[t][v + 1]));  // v_max3_f32
-  }
-  return m;
+  for (int e = 8; e < NT * 16; e += 2) m[(e >> 1) & 3] = max3(m[(e >> 1) & 3], s[e >> 4][e & 15], s[e >> 4][(e & 15) + 1]);
+  return max3(fmaxf(m[0], m[1]), m[2], m[3]);
 }
 
 // Set S^T entries above the causal diagonal to -inf.  kv_base = first kv index of score tile 0,

@@ -217,7 +217,7 @@ def test_verify_reference_math_matches_the_oracle_and_rejects_a_perturbed_output
 
 # ---------------------------------------------------------------------- the compiler's resource report
 REMARKS = """
-x.hip:2:1: remark: Function Name: _ZN3aat13ret_bwd_chainILi256ELi512ELi512ELi128ELi32ELi256ELi3ELi2ELNS_7BwdPassE0ELi1ELb1EEEvPKDF16_ [-Rpass-analysis=kernel-resource-usage]
+x.hip:2:1: remark: Function Name: _ZN3aat13ret_bwd_chainILi256ELi512ELi512ELi128ELi32ELi256ELi3ELi2ELNS_7BwdPassE0ELi1ELb1ELb0EEEvPKDF16_ [-Rpass-analysis=kernel-resource-usage]
 x.hip:2:1: remark:     TotalSGPRs: 58 [-Rpass-analysis=kernel-resource-usage]
 x.hip:2:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]
 x.hip:2:1: remark:     AGPRs: 256 [-Rpass-analysis=kernel-resource-usage]
@@ -227,7 +227,7 @@ x.hip:2:1: remark:     Occupancy [waves/SIMD]: 1 [-Rpass-analysis=kernel-resourc
 x.hip:2:1: remark:     SGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
 x.hip:2:1: remark:     VGPRs Spill: 604 [-Rpass-analysis=kernel-resource-usage]
 x.hip:2:1: remark:     LDS Size [bytes/block]: 0 [-Rpass-analysis=kernel-resource-usage]
-x.hip:3:1: remark: Function Name: _ZN3aat13ret_bwd_chainILi256ELi512ELi512ELi128ELi32ELi256ELi3ELi2ELNS_7BwdPassE0ELi1ELb0EEEvPKDF16_ [-Rpass-analysis=kernel-resource-usage]
+x.hip:3:1: remark: Function Name: _ZN3aat13ret_bwd_chainILi256ELi512ELi512ELi128ELi32ELi256ELi3ELi2ELNS_7BwdPassE0ELi1ELb0ELb0EEEvPKDF16_ [-Rpass-analysis=kernel-resource-usage]
 x.hip:3:1: remark:     VGPRs: 250 [-Rpass-analysis=kernel-resource-usage]
 x.hip:3:1: remark:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=kernel-resource-usage]
 """
@@ -237,11 +237,11 @@ def test_resource_report_is_parsed_and_decides_what_the_tuner_times(tmp_path, mo
     usage = codegen.parse_resource_usage(REMARKS)
     assert [k["scratch_bytes"] for k in usage] == [2416, 16] and usage[0]["vgprs"] == 256 and usage[0]["vgpr_spills"] == 604
     assert usage[0]["occupancy"] == 1 and usage[0]["agprs"] == 256 and usage[0]["sgprs"] == 58
-    assert codegen.template_bools(usage[0]["kernel"]) == [True] and codegen.template_bools(usage[1]["kernel"]) == [False]
+    assert codegen.template_bools(usage[0]["kernel"]) == [True, False] and codegen.template_bools(usage[1]["kernel"]) == [False, False]
     assert codegen.template_bools("_ZN3aat21flashattn_fwd_regfuseILi128ELi128ELi256ELi64ELi512ELi2ELi2ELi2ELb0ELb1ELb0ELb0EEEvPKDF16_") == [False, True, False, False]
     assert codegen.template_bools("_Z6kernelPf") == []
     assert [k["scratch_bytes"] for k in codegen.spilling_kernels(usage)] == [2416]          # 16 bytes are below the threshold
-    assert codegen.spilling_kernels(usage, lambda name: not codegen.template_bools(name)[-1]) == []
+    assert codegen.spilling_kernels(usage, lambda name: not codegen.template_bools(name)[0]) == []
     assert codegen.spilling_kernels(None) == []
     # a decay tuner looks at the decay kernels of a library, a mask-tensor tuner at the others
     from attention_autotuner_amd.autotuner import RetBwdTunner
@@ -249,6 +249,7 @@ def test_resource_report_is_parsed_and_decides_what_the_tuner_times(tmp_path, mo
     arrays = make_tensors("ret_bwd", 1, 2, 256, 256, 256, 512, "meta")
     assert RetBwdTunner(ARCH, arrays, decay=True)._kernel_matters(usage[0]["kernel"])
     assert not RetBwdTunner(ARCH, arrays, causal=True)._kernel_matters(usage[0]["kernel"])
+    assert RetBwdTunner(ARCH, arrays, causal=True)._kernel_matters("_ZN3aat18ret_bwd_dk_from_dsILi256ELi128ELi64ELi256ELi2ELi2EEEvPKDF16_S2_PDF16_iiiiPKiii")
     attn = AttnTunner(ARCH, make_tensors("attn", 1, 2, 256, 256, 128, 128, "meta"), causal=True)
     name = "_ZN3aat21flashattn_fwd_regfuseILi128ELi128ELi256ELi64ELi512ELi2ELi2ELi2ELb0ELb%dELb0ELb0EEEvPKDF16_"
     assert attn._kernel_matters(name % 1) and not attn._kernel_matters(name % 0)
