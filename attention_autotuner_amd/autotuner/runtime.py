@@ -22,6 +22,20 @@ _ERRORS = {-2: "sequence lengths are not multiples of the configuration's tile (
            -3: "workspace missing or too small"}
 
 
+# A RetNet backward built with a stored dS asks for B*H*S_q*S_kv fp16 on top of the mask scan and works without them
+# (it then evaluates dS twice).  Beyond this many bytes the runtime does not grant the room on its own: a caller who
+# wants it there passes a workspace of workspace_size() bytes.
+MAX_DS_BYTES = int(os.environ.get("AAT_MAX_DS_BYTES", 2 << 30))
+
+
+def _wanted(config, need, B, H, Sq, Sk):
+    """Bytes of workspace the runtime provides when the caller's is missing or too small."""
+    ds_bytes = 2 * B * H * Sq * Sk
+    if getattr(config, "operation", "") == "ret_bwd" and getattr(config, "ds_rows", 0) and need >= ds_bytes > MAX_DS_BYTES:
+        return need - ds_bytes
+    return need
+
+
 def _grown(workspace, need, device, keep):
     """A workspace of ``need`` bytes.  ``keep``: the one handed in holds a mask scan an earlier launch left (mode
     "scanned") and is smaller than this library wants (a backward that also stores dS): its bytes move to the head of
@@ -68,7 +82,7 @@ class Runtime:
         B, H, Sq, Sk = int(q.shape[0]), int(q.shape[1]), int(q.shape[2]), int(k.shape[2])
         op = self.config.operation
         lib = library.load(self._path(), op)
-        need = int(lib.workspace_size(B, H, Sq, Sk))
+        need = _wanted(self.config, int(lib.workspace_size(B, H, Sq, Sk)), B, H, Sq, Sk)
         if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
             workspace = _grown(workspace, need, q.device, keep=causal == "scanned")
         ws_ptr = ctypes.c_void_p(workspace.data_ptr() if workspace is not None else 0)
@@ -107,7 +121,7 @@ class Runtime:
         B, H, Sq, Sk = int(q.shape[0]), int(q.shape[1]), int(q.shape[2]), int(k.shape[2])
         op = self.config.operation
         lib = library.load(self._path(), op)
-        need = int(lib.workspace_size(B, H, Sq, Sk))
+        need = _wanted(self.config, int(lib.workspace_size(B, H, Sq, Sk)), B, H, Sq, Sk)
         if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
             workspace = _grown(workspace, need, q.device, keep=causal == "scanned")
         args = [ctypes.c_void_p(t.data_ptr()) for t in torch_array] + [B, H, Sq, Sk]

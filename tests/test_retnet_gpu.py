@@ -491,3 +491,31 @@ def test_without_room_for_ds_the_library_evaluates_it_twice():
     # the scanning modes still need their ranges
     ptrs = [ctypes.c_void_p(x.data_ptr()) for x in (q, k, v, mask, do, r, *got["plain", "no workspace"], torch.zeros(1, device="cuda"))]
     assert libs[0].kernel_entry_ex(*ptrs, 1, 2, 256, 256, 3, None, 0, None) == -3
+
+
+def test_runtime_grants_the_room_for_ds_up_to_a_cap(monkeypatch):
+    """Beyond ``runtime.MAX_DS_BYTES`` the runtime hands the library the mask scan's bytes only and the library
+    evaluates dS twice: the results of the configuration without the stored dS."""
+    import parity_matrix
+    from attention_autotuner_amd.autotuner import runtime
+    t = parity_matrix.RET_BWD_STORED_DS[0]
+    with_ds, plain = parity_matrix.ret_bwd_stored_ds_config(*t), parity_matrix.ret_bwd_stored_ds_config(*t[:5], 0)
+    b, h, sq, sk = 1, 2, 256, 256
+    assert runtime._wanted(with_ds, 1000 + 2 * b * h * sq * sk, b, h, sq, sk) == 1000 + 2 * b * h * sq * sk
+    q, k, v, mask, do = (x.cuda() for x in _inputs(b, h, sq, sk, 256, 512, seed=9))
+    r = torch.full((b, h, sq), 20.0, device="cuda")
+    outs = {}
+    for name, cfg, cap in (("granted", with_ds, None), ("capped", with_ds, 1024), ("plain", plain, None)):
+        if cap is not None:
+            monkeypatch.setattr(runtime, "MAX_DS_BYTES", cap)
+            assert runtime._wanted(cfg, 1000 + 2 * b * h * sq * sk, b, h, sq, sk) == 1000
+        o = [torch.full_like(x, float("nan")) for x in (q, k, v)]
+        Runtime(ARCH, cfg).apply([q, k, v, mask, do, r, *o, torch.zeros(1, device="cuda")], causal=True)
+        torch.cuda.synchronize()
+        outs[name] = o
+    for a, c in zip(outs["capped"], outs["plain"]):
+        assert torch.equal(a, c)
+    assert torch.equal(outs["granted"][0], outs["plain"][0]) and torch.equal(outs["granted"][2], outs["plain"][2])
+    # dK of the granted run comes from the other kernel and from the dQ pass's rounding of dS: equal to the plain one only
+    # up to that rounding (its parity is test_backward_with_a_stored_ds_agrees_with_the_one_that_evaluates_it_twice's)
+    assert not torch.equal(outs["granted"][1], outs["plain"][1])
