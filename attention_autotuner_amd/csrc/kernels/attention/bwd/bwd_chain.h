@@ -277,7 +277,11 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
 
     // first contractions: s = Y1 X1^T (scores), p = Y2 X2^T (dP), both transposed (lane owns resident row)
     // the score tiles accumulate in vector registers when the outputs alone fill the accumulation registers
-    constexpr bool kVacc = WPE == 1 && RT * ((kOut1 ? DT : 0) + (kOut2 ? KT + NT : 0) + NT) * 16 > 256;
+    // ... and also when they fit next to the resident fragments anyway: a score tile in accumulation registers is
+    // read back one register at a time for the element-wise step (64 v_accvgpr_read per 64-row tile at d 128;
+    // -0.7 ... -1.0 % on the whole backward, same bits)
+    constexpr bool kFitsVec = RT * (KS + (kOut2 ? DS : 0)) * 4 + RT * NT * 32 + 72 <= 208;
+    constexpr bool kVacc = WPE == 1 && (kFitsVec || RT * ((kOut1 ? DT : 0) + (kOut2 ? KT + NT : 0) + NT) * 16 > 256);
     f16v s[RT][NT], dp[RT][kOut2 ? NT : 1];
     qk_gemm_steps<RT, NT, KS, NCK, PF, kVacc>(s, x1f, y1addr, off, [](int) {});
     if constexpr (kOut2) qk_gemm_steps<RT, NT, DS, NCD, PF, kVacc>(dp, x2f, y2addr, off, [](int) {});
