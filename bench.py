@@ -326,6 +326,12 @@ def retnet_measurements(aat, arch, mk, steps, warmup):
     res["retnet_fwd_bwd_b4h8s2048_dqk256_dv512"] = extra(t, (fwd_flops + bwd_flops) / 2, issued_ratio=issued_ratio("retnet_bwd", 1), flops_counted=half,
                                                          tflops_dense_count=round((fwd_flops + bwd_flops) / t.median / 1e9, 1))
     log(f"retnet fwd+bwd: {t.median:.4f} ms -> {(fwd_flops + bwd_flops) / t.median / 1e9:.1f} TFLOP/s (dense-mask FLOPs; zero tiles skipped)")
+    # a model applies one mask in every layer and step: the scan taken once and handed to every call
+    scan = aat.retnet_mask_scan(mask, arch)
+    t = time_launches(lambda: aat.RetNetAttnFunc(q, k, v, mask, arch, scan).backward(do), steps, warmup, before_each=reset)
+    res["retnet_fwd_bwd_scan_reused_b4h8s2048_dqk256_dv512"] = extra(t, (fwd_flops + bwd_flops) / 2, issued_ratio=issued_ratio("retnet_bwd", 1),
+                                                                     flops_counted=half)
+    log(f"retnet fwd+bwd, mask scan reused: {t.median:.4f} ms")
     t = time_launches(lambda: aat.RetNetAttnFunc(q, k, v, mask, arch, False).backward(do), steps, warmup, before_each=reset)
     res["retnet_fwd_bwd_dense_walk_b4h8s2048_dqk256_dv512"] = extra(t, fwd_flops + bwd_flops, issued_ratio=issued_ratio("retnet_bwd", 0))
     log(f"retnet fwd+bwd, dense walk: {t.median:.4f} ms -> {(fwd_flops + bwd_flops) / t.median / 1e9:.1f} TFLOP/s")

@@ -519,3 +519,24 @@ def test_runtime_grants_the_room_for_ds_up_to_a_cap(monkeypatch):
     # dK of the granted run comes from the other kernel and from the dQ pass's rounding of dS: equal to the plain one only
     # up to that rounding (its parity is test_backward_with_a_stored_ds_agrees_with_the_one_that_evaluates_it_twice's)
     assert not torch.equal(outs["granted"][1], outs["plain"][1])
+
+
+def test_a_mask_scan_taken_once_serves_later_calls():
+    """``retnet_mask_scan`` + ``RetNetAttnFunc(..., causal=scan)``: outputs and gradients have the bits of the call that scans
+    itself, whatever the mask looks like, and the scan is only read."""
+    b, h, sq, sk, dqk, dv = 2, 2, 256, 384, 64, 128
+    q, k, v, _, do = _inputs(b, h, sq, sk, dqk, dv, seed=51)
+    for name, mask in _masks(h, sq, sk, seed=52).items():
+        scan = aat.retnet_mask_scan(mask.cuda(), ARCH)
+        before = scan.clone()
+        outs = []
+        for causal in (None, scan, scan):
+            qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+            o = aat.RetNetAttnFunc(qc, kc, vc, mask.cuda(), ARCH, causal)
+            o.backward(do.cuda())
+            torch.cuda.synchronize()
+            outs.append((o.detach(), qc.grad, kc.grad, vc.grad))
+        for other in outs[1:]:
+            for a, c in zip(outs[0], other):
+                assert torch.equal(a, c), name
+        assert torch.equal(scan, before)                  # the calls only read it
