@@ -6,8 +6,8 @@ of block-resident rows and ``Bc`` the number of streamed rows per step of every 
 accepted for ABI compatibility and never touched: dQ is produced directly, without atomics.
 
 With ``ds_rows`` set the dQ pass runs before dK and stores its dS tiles in the workspace (behind the mask scan's
-ranges), and dK comes from the kernel that reads them back (dk_from_ds.h): the workspace is then needed in every
-mask mode, ``workspace_size`` says how much.
+ranges), and dK comes from the kernel that reads them back (dk_from_ds.h); ``workspace_size`` says how much room that
+takes, and without it the library runs the chained dK pass.
 """
 
 global_vars = r"""
