@@ -165,24 +165,41 @@ ret_bwd_dk_from_ds(const half_t* __restrict__ q, const half_t* __restrict__ ds, 
     const bool all_written = wlo <= x0 && x0 + BX <= whi;          // block-uniform
     const bool mine_written = my_kv >= wlo && my_kv < whi;
 
+    // The operand reads are issued as instructions with counted waits (tile_ops.h): in front of an LDS read it can see
+    // the compiler waits for every LDS-DMA copy in flight, i.e. for the next tile this one has just requested.
+    constexpr int PF = 2;
+    static_for<KSTEPS>([&](auto s_tag) {
+      constexpr int s = decltype(s_tag)::value;
+      h4 blo = lds_read_tr_h4_async(saddr, off + s * kSRow16);
+      h4 bhi = lds_read_tr_h4_async(saddr, off + s * kSRow16 + kSRow8);
+      h4 lo[PF], hi[PF];
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-      const h4 blo = lds_read_tr_h4_at(saddr + off + s * kSRow16);
-      const h4 bhi = lds_read_tr_h4_at(saddr + off + s * kSRow16 + kSRow8);
-      h8 bf = cat_h4(blo, bhi);
-      if (!all_written) {
-        if (!mine_written) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) bf[e] = (half_t)0.f;
+      for (int i = 0; i < PF && i < DT; ++i) {
+        lo[i] = lds_read_tr_h4_async(zaddr[i], off + s * kZRow16);
+        hi[i] = lds_read_tr_h4_async(zaddr[i], off + s * kZRow16 + kZRow8);
+      }
+      h8 bf;
+      static_for<DT>([&](auto dt_tag) {
+        constexpr int dt = decltype(dt_tag)::value;
+        h4 clo = lo[dt % PF], chi = hi[dt % PF];
+        if constexpr (dt + PF < DT) {
+          lo[dt % PF] = lds_read_tr_h4_async(zaddr[dt + PF], off + s * kZRow16);
+          hi[dt % PF] = lds_read_tr_h4_async(zaddr[dt + PF], off + s * kZRow16 + kZRow8);
         }
-      }
+        lds_wait_younger<2 * ((dt + PF < DT) ? PF : DT - 1 - dt)>(clo, chi);      // the B pair is older: it has landed too
+        if constexpr (dt == 0) {
+          asm volatile("" : "+v"(blo), "+v"(bhi));
+          bf = cat_h4(blo, bhi);
+          if (!all_written) {
+            if (!mine_written) {
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        const h4 lo = lds_read_tr_h4_at(zaddr[dt] + off + s * kZRow16);
-        const h4 hi = lds_read_tr_h4_at(zaddr[dt] + off + s * kZRow16 + kZRow8);
-        acc[0][dt] = mfma_32x32x16(cat_h4(lo, hi), bf, acc[0][dt]);
-      }
-    }
+              for (int e = 0; e < 8; ++e) bf[e] = (half_t)0.f;
+            }
+          }
+        }
+        acc[0][dt] = mfma_32x32x16(cat_h4(clo, chi), bf, acc[0][dt]);
+      });
+    });
   };
   for (int j = j_begin; j < j_end; j += NS) {
     static_for<NS>([&](auto k_tag) {
