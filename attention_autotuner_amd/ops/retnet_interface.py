@@ -75,6 +75,8 @@ class RetNetAttn(torch.autograd.Function):
         scan = None
         if reused is not None:
             scan = reused
+            assert scan.is_cuda and scan.dtype == torch.uint8 and scan.numel() >= rt.workspace_size(batch_size, nheads, seqlen_q, seqlen_k), \
+                "causal: a scan from retnet_mask_scan(mask, device_type) of a mask of this shape"
             rt.apply(arrays, causal="scanned", workspace=scan)
         elif causal is None:                   # the scan lands in `scan`; the backward reads it from there
             scan = torch.empty(rt.workspace_size(batch_size, nheads, seqlen_q, seqlen_k), dtype=torch.uint8, device=q.device)
