@@ -72,8 +72,8 @@ template <int Kd, int D, int Br, int Bc, int NT, int NSK, int NSV, int WPE, bool
 static void test_regfuse_attention(const ProblemShape& ps, const Buffers& b) {
   using T = aat::AttnFwdRegfuse<Kd, D, Br, Bc, NT, NSK, NSV>;
   if (ps.Sq % Br || ps.Sk % Bc) return;
-  auto plain = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, PIPE, false>;
-  auto causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, PIPE, true>;
+  auto plain = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, Bc, PIPE, false>;
+  auto causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, Bc, PIPE, true>;
   HIP_OK(hipFuncSetAttribute((const void*)plain, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
   HIP_OK(hipFuncSetAttribute((const void*)causal, hipFuncAttributeMaxDynamicSharedMemorySize, T::kSmemBytes));
   const float scale = 1.f / std::sqrt((float)Kd);
@@ -82,7 +82,7 @@ static void test_regfuse_attention(const ProblemShape& ps, const Buffers& b) {
   using TP = typename T::template Persist<WPE>;
   int resident = 0;
   if constexpr (TP::kOk && !PIPE) {
-    auto persist = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, false, false, false, true>;
+    auto persist = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, NT, NSK, NSV, WPE, Bc, false, false, false, true>;
     int per_cu = 0, cus = 0, dev = 0;
     HIP_OK(hipGetDevice(&dev));
     HIP_OK(hipFuncSetAttribute((const void*)persist, hipFuncAttributeMaxDynamicSharedMemorySize, TP::kSmemBytes));

@@ -23,13 +23,14 @@ constexpr int num_stages_v = {num_stages_v};     // LDS buffers for the V tile
 constexpr int waves_per_eu = {waves_per_eu};
 constexpr int kv_splits = {kv_splits};           // > 1: the kv range is cut into that many parts (non-causal only)
 constexpr bool sw_pipeline = {sw_pipeline};      // next tile's QK^T MFMAs interleaved with this tile's exponentials
+constexpr int unit_rows = sw_pipeline ? Bc : {BlockKSmem2};   // plain schedule: kv rows per scores -> softmax -> PV unit inside a tile of Bc rows
 constexpr float kReferenceScale = 0.125f;        // what the reference kernels hard-code
 
 using Traits = aat::AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v>;
 constexpr int shared_mem = Traits::kSmemBytes;
-const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, false>;
-const auto kernel_causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, true>;
-const auto kernel_split = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, sw_pipeline, false, true>;
+const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, sw_pipeline, false>;
+const auto kernel_causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, sw_pipeline, true>;
+const auto kernel_split = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, sw_pipeline, false, true>;
 constexpr int shared_mem_split = Traits::kSmemBytesSplit;
 
 // Persistent variant (a block walks several row blocks, prefetching across them): exists for two K and two V
@@ -44,7 +45,7 @@ using PersistTraits = Traits::Persist<waves_per_eu>;
 constexpr int shared_mem_persist = PersistTraits::kSmemBytes;
 template <bool OK> auto persistent_kernel() {{
   if constexpr (OK)
-    return &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, false, false, false, true>;
+    return &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, false, false, false, true>;
   else
     return static_cast<decltype(kernel)>(nullptr);
 }}

@@ -27,6 +27,11 @@
 #ifndef AAT_PF
 #define AAT_PF 2
 #endif
+#ifdef AAT_NOPRIO
+#define AAT_SETPRIO(x)
+#else
+#define AAT_SETPRIO(x) __builtin_amdgcn_s_setprio(x)
+#endif
 
 namespace aat {
 
@@ -121,7 +126,7 @@ template <bool CAUSAL, class F> AAT_DEV void run_tiles(F& tile, int n_full, int 
 // the copies only: memory operations complete in order, so "at most as many outstanding as stores were issued
 // after them" leaves the stores in flight.  Needs two K and two V buffers and an even number of kv tiles (the
 // buffer parity must wrap); plain schedule, non-causal, unsplit.
-template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int WPE = 1, bool PIPE = false,
+template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int WPE = 1, int BU = Bc, bool PIPE = false,
           bool CAUSAL = false, bool SPLIT = false, bool PERSIST = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k,
@@ -131,6 +136,15 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   using T = AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, WM = T::WM;
   constexpr int PF = AAT_PF;                     // operand prefetch distance, in MFMA steps
+  // Plain schedule: a kv tile of Bc rows (one copy, one barrier) is worked through in NU units of BU rows, each
+  // scores -> softmax -> PV, so the live score tile is RT * BU / 32 accumulator blocks whatever Bc is.
+  constexpr int NU = Bc / BU, NTU = BU / 32;
+  static_assert(Bc % BU == 0 && BU % 32 == 0, "a kv tile is a whole number of units of whole 32-row score tiles");
+  static_assert(NU == 1 || (NSK == 2 && NSV == 2), "units inside a tile: no barrier between the contractions, two K and two V buffers");
+  static_assert(NU == 1 || !PIPE, "the pipelined schedule has its own 32-row units");
+  // Where the output accumulators, the Q fragments and one unit's scores leave fewer than 40 of a wave's registers,
+  // the operand addresses of all contraction steps are derived from one register each (tile_ops.h: XA).
+  constexpr bool XA = WPE >= 2 && RT * (DT * 16 + KS * 4 + NTU * 16) + 40 > 512 / WPE;
   static_assert(!PIPE || T::kPipeOk, "the pipelined schedule needs 2+2 buffers and unit-aligned K copies");
   static_assert(!(SPLIT && CAUSAL), "kv splitting is for non-causal problems");
   using TP = typename T::template Persist<WPE>;
@@ -145,8 +159,8 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   const int n = lane & 31, h = lane >> 5;
 
   const int Tr = seq_q / Br;
-  typename T::KDma kdma;
-  typename T::VDma vdma;
+  TileDma<Bc, NCK, Nthreads, Swz::Rows16, 0, XA> kdma;
+  TileDma<Bc, NCV, Nthreads, Swz::Rows4, 0, XA> vdma;
   kdma.init(tid);
   vdma.init(tid);
   const int wave_base = wave * 64;
@@ -264,50 +278,54 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
           }
         }
 
-        // A wave none of whose rows sees any kv row of this tile (above the diagonal) only keeps the block's
-        // copies and barriers going: its P would be all zeros, which changes neither O nor l nor the maximum.
-        bool wave_sees = true;
-        if constexpr (MASKED) wave_sees = j * Bc <= q0 + wave * WM + WM - 1 + diag;
-
-        f16v sacc[RT][NT];
+        // A wave none of whose rows sees any kv row of a unit (above the diagonal) only keeps the block's copies
+        // and barriers going: its P would be all zeros, which changes neither O nor l nor the maximum.
         // The matrix phases run at a raised wave priority: with two or three waves on the SIMD the one that has
         // MFMAs to issue goes first and the others' softmax arithmetic fills the gaps, not the other way round
         // (causal forward at three waves per SIMD: -1.4 %; nothing at two).
-        if (wave_sees) {
-          __builtin_amdgcn_s_setprio(2);
-          qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
-          __builtin_amdgcn_s_setprio(0);
-        }
-        if constexpr (PERSIST) {
-          if (!more && has_next) load_q_frags_async<RT, KS, Kd>(qf, q_next);   // the last scores of this row block are done; waited for at (A)
-        }
-        if (wave_sees) {
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) {
-            if constexpr (MASKED) causal_mask<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
-            const float mc = lazy_max_step<NT, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
-            exp_tile<NT>(sacc[rt], c2, mc);
-            if constexpr (MASKED) zero_masked<NT>(sacc[rt], j * Bc, q_lim0 + rt * 32, h);
-          }
-        }
+        static_for<NU>([&](auto unit_tag) {
+          constexpr int U = decltype(unit_tag)::value;
+          const int kv0 = j * Bc + U * BU;           // first kv row of the unit
+          bool wave_sees = true;
+          if constexpr (MASKED) wave_sees = kv0 <= q0 + wave * WM + WM - 1 + diag;
 
-        // (B) with one buffer: V_j must have landed / K buffer must be free before K_{j+1} is fetched.
-        if constexpr (NSV == 1 || NSK == 1) {
-          if constexpr (NSV == 1) wait_vmcnt<0>();
-          block_sync();
-          if constexpr (NSK == 1) {
-            if (more) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf, wave_base);
+          f16v sacc[RT][NTU];
+          if (wave_sees) {
+            AAT_SETPRIO(2);
+            qk_gemm_steps<RT, NTU, KS, NCK, PF, false, XA>(sacc, qf, kaddr, (NSK == 2 ? PAR * T::kKBytes : 0) + U * NTU * T::kUnitK, [](int) {});
+            AAT_SETPRIO(0);
           }
-        }
-        if (wave_sees) {
-          h8 pf[RT][NT][2];
-          __builtin_amdgcn_s_setprio(2);
-          pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
+          if constexpr (PERSIST && U == NU - 1) {
+            if (!more && has_next) load_q_frags_async<RT, KS, Kd>(qf, q_next);   // the last scores of this row block are done; waited for at (A)
+          }
+          if (wave_sees) {
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) pack_p_group<NT>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
-          });
-          __builtin_amdgcn_s_setprio(0);
-        }
+            for (int rt = 0; rt < RT; ++rt) {
+              if constexpr (MASKED) causal_mask<NTU>(sacc[rt], kv0, q_lim0 + rt * 32, h);
+              const float mc = lazy_max_step<NTU, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
+              exp_tile<NTU, XA>(sacc[rt], c2, mc);
+              if constexpr (MASKED) zero_masked<NTU>(sacc[rt], kv0, q_lim0 + rt * 32, h);
+            }
+          }
+
+          // (B) with one buffer: V_j must have landed / K buffer must be free before K_{j+1} is fetched.
+          if constexpr (NSV == 1 || NSK == 1) {
+            if constexpr (NSV == 1) wait_vmcnt<0>();
+            block_sync();
+            if constexpr (NSK == 1) {
+              if (more) kdma.issue(kg + (size_t)(j + 1) * T::kKBytes, kbuf, wave_base);
+            }
+          }
+          if (wave_sees) {
+            h8 pf[RT][NTU][2];
+            AAT_SETPRIO(2);
+            pv_gemm_steps<RT, NTU, DT, NCV, PF, false, XA>(oacc, pf, vaddr, (NSV == 2 ? PAR * T::kVBytes : 0) + U * NTU * T::kUnitV, [&](int g) {
+#pragma unroll
+              for (int rt = 0; rt < RT; ++rt) pack_p_group<NTU, XA>(pf[rt], sacc[rt], g, l_run[rt]);   // per-lane partial sums
+            });
+            AAT_SETPRIO(0);
+          }
+        });
       };
       run_tiles<CAUSAL>(kv_tile, n_full, n_tiles);
     } else {

@@ -170,7 +170,11 @@ template <int N, int I = 0, class F> AAT_DEV void static_for(F&& f) {
 // threads cover whole rows per instruction (NT % NC == 0): then a thread keeps its chunk column and
 // only the swizzle term can change from one instruction to the next, with a short period.
 // AUX: cache-policy bits of the load (2 = non-temporal: data read once).
-template <int ROWS, int NC, int NT, Swz MODE, int AUX = 0>
+// SADDR: the copy instruction is written out in its scalar-base form (64-bit base in SGPRs, one 32-bit per-lane
+// offset) with its own write of M0; the builtin form adds the per-lane offset to the base as a 64-bit vector add per
+// instruction and keeps the offsets as register pairs.  A kernel must issue all its copies one way or the other: the
+// compiler does not know that the asm form has changed M0.
+template <int ROWS, int NC, int NT, Swz MODE, int AUX = 0, bool SADDR = false>
 struct TileDma {
   static constexpr int kChunks = ROWS * NC;
   static_assert(kChunks % NT == 0, "tile chunks must divide evenly over the block's threads");
@@ -214,6 +218,13 @@ struct TileDma {
     uint64_t base = (uint64_t)(uintptr_t)(kRegular ? g + (size_t)i * kRowsPerIter * pitch : g);
     asm volatile("" : "+s"(base));                     // keep the uniform part in SGPRs (saddr form)
     const uint32_t lane_off = loff[kRegular ? i % kDistinct : i];
+    if constexpr (SADDR) {
+      static_assert(AUX == 0 || !SADDR, "the scalar-base form is written without cache-policy bits");
+      const uint32_t dst = __builtin_amdgcn_readfirstlane(
+          (uint32_t)(uintptr_t)(AAT_AS3 char*)(lds + (i * NT + wave_base) * 16));
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off), "s"(base) : "memory");
+      return;
+    }
     __builtin_amdgcn_global_load_lds((const AAT_AS1 void*)(uintptr_t)(base + lane_off),
                                      (AAT_AS3 void*)(lds + (i * NT + wave_base) * 16), 16, 0, AUX);
   }

@@ -94,11 +94,18 @@ AAT_DEV float lazy_max_step(const f16v (&s)[NT], float& m_run, float& l_run, f16
 }
 
 // s <- exp2(s*c2 - mc) in place (masked entries hold -inf and come out as 0 for any positive scale).
-template <int NT> AAT_DEV void exp_tile(f16v (&s)[NT], float c2, float mc) {
+// FENCED: a scheduling barrier after every four entries, for kernels without a register to spare: left alone the
+// scheduler lifts the multiply-adds of a whole tile above its exponentials and the results land in new registers.
+template <int NT, bool FENCED = false> AAT_DEV void exp_tile(f16v (&s)[NT], float c2, float mc) {
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[t][v] = fast_exp2(__builtin_fmaf(s[t][v], c2, -mc));
+    for (int v = 0; v < 16; ++v) {
+      s[t][v] = fast_exp2(__builtin_fmaf(s[t][v], c2, -mc));
+      if constexpr (FENCED) {
+        if (v % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+      }
+    }
 }
 
 // exp of `count` consecutive entries (flattened index e = 16*tile + v) of a row group, in place.
@@ -117,7 +124,10 @@ template <int NT> AAT_DEV void exp_range(f16v (&s)[NT], int e0, int count, float
 // gfx950 the dot instructions share the matrix pipe's issue path: next to a wave that streams MFMAs each
 // v_dot2c_f32_f16 of the other wave of the SIMD was measured at ~90 cycles instead of 4.5 (8 of them turned
 // a 450-cycle stretch of exponentials and conversions into 1150 cycles), and a wave's own MFMAs wait for them too.
-template <int NT> AAT_DEV void pack_p_group(h8 (&pf)[NT][2], const f16v (&s)[NT], int g, float& sum) {
+// PIN: the updated sum is tied to this point of the program.  Otherwise the compiler is free to sink the additions
+// to the sum's next use -- the rescale test of the NEXT unit -- and the sixteen unrounded P values they read stay
+// live across that unit's first contraction, which is where a kernel short of registers is shortest.
+template <int NT, bool PIN = false> AAT_DEV void pack_p_group(h8 (&pf)[NT][2], const f16v (&s)[NT], int g, float& sum) {
   const int t = g >> 1, half = g & 1;
   h8 r;
   float s0 = s[t][8 * half] + s[t][8 * half + 1], s1 = s[t][8 * half + 2] + s[t][8 * half + 3];
@@ -130,6 +140,7 @@ template <int NT> AAT_DEV void pack_p_group(h8 (&pf)[NT][2], const f16v (&s)[NT]
   s0 += s[t][8 * half + 4] + s[t][8 * half + 5];
   s1 += s[t][8 * half + 6] + s[t][8 * half + 7];
   sum += s0 + s1;
+  if constexpr (PIN) asm volatile("" : "+v"(sum));
   pf[t][half] = r;
 }
 

@@ -88,6 +88,16 @@ AAT_DEV h8 lds_read_h8_async(uint32_t base, int imm) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(base + hi), "i"(imm & 0xffff));
   return v;
 }
+// The same read at address base ^ x (x a compile-time constant): the operand addresses of a swizzled tile differ
+// from one contraction step to the next by an XOR of the chunk bits, so one address register plus a one-cycle
+// v_xor_b32 into a short-lived temporary serves every step where registers are scarce.
+AAT_DEV h8 lds_read_h8_async_xor(uint32_t base, int x, int imm) {
+  h8 v;
+  uint32_t t;
+  const uint32_t hi = (uint32_t)imm & ~0xffffu;
+  asm volatile("v_xor_b32 %1, %3, %2\n\tds_read_b128 %0, %1 offset:%4" : "=v"(v), "=&v"(t) : "v"(base + hi), "n"(x), "i"(imm & 0xffff));
+  return v;
+}
 // Wait until at most N LDS operations issued after the one that produced `v` are outstanding.  The
 // operand ties the wait to the value, so no consumer of `v` can be scheduled above it.
 template <int N> AAT_DEV void lds_wait_younger(h8& v) {
@@ -117,6 +127,12 @@ AAT_DEV h4 lds_read_tr_h4_async(uint32_t base, int imm) {
   const uint32_t hi = (uint32_t)imm & ~0xffffu;
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(base + hi), "i"(imm & 0xffff));
   return v;
+}
+// Both transposing reads of one 16-row step (rows +0 and +8) at address base ^ x.
+AAT_DEV void lds_read_tr_h4_pair_async_xor(h4& lo, h4& hi, uint32_t base, int x, int imm_lo, int imm_hi) {
+  uint32_t t;
+  asm volatile("v_xor_b32 %2, %4, %3\n\tds_read_b64_tr_b16 %0, %2 offset:%5\n\tds_read_b64_tr_b16 %1, %2 offset:%6"
+               : "=v"(lo), "=&v"(hi), "=&v"(t) : "v"(base), "n"(x), "i"(imm_lo), "i"(imm_hi));
 }
 template <int N> AAT_DEV void lds_wait_younger(h4& a, h4& b) {
   static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
@@ -150,18 +166,28 @@ AAT_DEV void mfma_settle(f16v& c) { asm volatile("s_nop 15\n\ts_nop 7" : "+v"(c)
 // S^T = K Q^T over one kv tile.  kaddr[ks] = LDS address of this lane's chunk for k-step ks in score
 // tile 0 of the K buffer (tile nt adds nt*32 rows).  side(step) runs after the MFMA group of each step.
 // VACC: accumulate in vector registers through hand-written MFMAs (see mfma_32x32x16_vacc).
-template <int RT, int NT, int KS, int NCK, int PF, bool VACC = false, class Side>
+// XA: only kaddr[0] is used; step ks reads at kaddr[0] ^ (ks % 8) << 5 (the Rows16 swizzle XORs the chunk index
+// 2 ks + h with row bits, so the steps' addresses differ by exactly that).
+template <int RT, int NT, int KS, int NCK, int PF, bool VACC = false, bool XA = false, class Side>
 AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const uint32_t (&kaddr)[KS],
                            int buf_off, Side&& side) {
+  static_assert(!(XA && VACC), "xor addressing is for kernels that fit the unified register file");
   constexpr int S = NT * KS;
   constexpr int kTileStride = 32 * NCK * 16;
   // With rows of whole 16-chunk groups the swizzle only permutes chunks inside a group, so k-step ks
   // sits 256 bytes per group behind k-step ks % 8: eight address registers serve any contraction width.
   constexpr bool kFold = NCK % 16 == 0 && KS > 8;
+  static_assert(!XA || NCK % 16 == 0 || NCK == 8, "xor addressing: the swizzle must act on whole bits of the chunk index");
   auto read = [&](int i) {
     const int ks = i % KS;
-    return lds_read_h8_async(kFold ? kaddr[ks % 8] : kaddr[ks],
-                             (kFold ? (ks / 8) * 256 : 0) + buf_off + (i / KS) * kTileStride);
+    if constexpr (XA) {
+      const int imm = (NCK % 16 == 0 ? (ks / 8) * 256 : 0) + buf_off + (i / KS) * kTileStride;
+      if (ks % 8 == 0) return lds_read_h8_async(kaddr[0], imm);
+      return lds_read_h8_async_xor(kaddr[0], (ks % 8) << 5, imm);
+    } else {
+      return lds_read_h8_async(kFold ? kaddr[ks % 8] : kaddr[ks],
+                               (kFold ? (ks / 8) * 256 : 0) + buf_off + (i / KS) * kTileStride);
+    }
   };
   if constexpr (!VACC) {
 #pragma unroll
@@ -175,14 +201,23 @@ AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const u
   sched_fence();
   static_for<S>([&](auto step_tag) {
     constexpr int step = decltype(step_tag)::value;
-    h8 cur = ring[step % PF];
-    if constexpr (step + PF < S) ring[step % PF] = read(step + PF);
-    lds_wait_younger<(step + PF < S) ? PF : S - 1 - step>(cur);
+    if constexpr (XA) {
+      // Scarce registers: the ring slot is consumed where it is and refilled behind its MFMAs (a matrix instruction
+      // has read its operands long before an LDS read issued after it returns), so PF slots are all there is.
+      lds_wait_younger<(step + PF - 1 < S) ? PF - 1 : S - 1 - step>(ring[step % PF]);
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      if constexpr (!VACC) sacc[rt][step / KS] = mfma_32x32x16(cur, qf[rt][step % KS], sacc[rt][step / KS]);
-      else if constexpr (step % KS == 0) mfma_32x32x16_vacc_first(sacc[rt][step / KS], cur, qf[rt][step % KS]);
-      else mfma_32x32x16_vacc(sacc[rt][step / KS], cur, qf[rt][step % KS]);
+      for (int rt = 0; rt < RT; ++rt) sacc[rt][step / KS] = mfma_32x32x16(ring[step % PF], qf[rt][step % KS], sacc[rt][step / KS]);
+      if constexpr (step + PF < S) ring[step % PF] = read(step + PF);
+    } else {
+      h8 cur = ring[step % PF];
+      if constexpr (step + PF < S) ring[step % PF] = read(step + PF);
+      lds_wait_younger<(step + PF < S) ? PF : S - 1 - step>(cur);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if constexpr (!VACC) sacc[rt][step / KS] = mfma_32x32x16(cur, qf[rt][step % KS], sacc[rt][step / KS]);
+        else if constexpr (step % KS == 0) mfma_32x32x16_vacc_first(sacc[rt][step / KS], cur, qf[rt][step % KS]);
+        else mfma_32x32x16_vacc(sacc[rt][step / KS], cur, qf[rt][step % KS]);
+      }
     }
     side(step);
     sched_fence();
@@ -242,7 +277,9 @@ AAT_DEV void pv_gemm_steps_hl(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const u
 // for d-tile dt, kv rows 0..3 (+4h) of the V buffer.  pack(g) must fill pf[*][g/2][g%2] (the P operand of
 // kv rows 16g .. 16g+15); it is called one group ahead of use, between MFMAs.
 // BLIND: as in pv_gemm_steps_hl.
-template <int RT, int NT, int DT, int NCV, int PF, bool BLIND = false, class Pack>
+// XA: only vaddr[0] is used; d-tile dt reads at vaddr[0] ^ (dt % 4) << 6 (the Rows4 swizzle XORs the chunk-group
+// bits with row bits); implies hand-issued reads with counted waits.
+template <int RT, int NT, int DT, int NCV, int PF, bool BLIND = false, bool XA = false, class Pack>
 AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint32_t (&vaddr)[DT], int buf_off,
                            Pack&& pack) {
   constexpr int G = NT * 2;              // groups of 16 kv rows
@@ -252,31 +289,49 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
   // is four chunks wide: d-tile dt sits 256 bytes per group behind d-tile dt % 4, so four address registers
   // serve any output width (the others are never read and cost nothing).
   constexpr bool kFold = NCV % 16 == 0 && DT > 4;
-  static_assert(!BLIND || 2 * PF < 16, "two reads per step in flight, counted by a 4-bit counter");
-  auto read = [&](int i, int half) {
-    return lds_read_tr_h4_either<BLIND>(kFold ? vaddr[(i % DT) % 4] : vaddr[i % DT],
-                                (kFold ? ((i % DT) / 4) * 256 : 0) + buf_off + (i / DT) * kRow16 + half * kRow8);
-  };
+  static_assert(!(BLIND || XA) || 2 * PF < 16, "two reads per step in flight, counted by a 4-bit counter");
+  static_assert(!XA || NCV % 16 == 0 || NCV == 8, "xor addressing: the swizzle must act on whole bits of the chunk index");
+  constexpr bool kHand = BLIND || XA;
   h4 lo[PF], hi[PF];
+  auto read = [&](int i, int slot) {
+    const int dt = i % DT;
+    if constexpr (XA) {
+      const int imm = (NCV % 16 == 0 ? (dt / 4) * 256 : 0) + buf_off + (i / DT) * kRow16;
+      if (dt % 4 == 0) {
+        lo[slot] = lds_read_tr_h4_async(vaddr[0], imm);
+        hi[slot] = lds_read_tr_h4_async(vaddr[0], imm + kRow8);
+      } else {
+        const int far = (imm + kRow8 > 0xffff) ? (imm & ~0x7fff) : 0;     // beyond the 16-bit offset field: one add
+        lds_read_tr_h4_pair_async_xor(lo[slot], hi[slot], vaddr[0] + (uint32_t)far, (dt % 4) << 6, imm - far, imm - far + kRow8);
+      }
+    } else {
+      const uint32_t a = kFold ? vaddr[dt % 4] : vaddr[dt];
+      const int imm = (kFold ? (dt / 4) * 256 : 0) + buf_off + (i / DT) * kRow16;
+      lo[slot] = lds_read_tr_h4_either<BLIND>(a, imm);
+      hi[slot] = lds_read_tr_h4_either<BLIND>(a, imm + kRow8);
+    }
+  };
 #pragma unroll
-  for (int i = 0; i < PF && i < S; ++i) {
-    lo[i] = read(i, 0);
-    hi[i] = read(i, 1);
-  }
+  for (int i = 0; i < PF && i < S; ++i) read(i, i);
   pack(0);
   sched_fence();
   static_for<S>([&](auto step_tag) {
     constexpr int step = decltype(step_tag)::value;
     constexpr int g = step / DT, dt = step % DT;
-    h4 clo = lo[step % PF], chi = hi[step % PF];
-    if constexpr (step + PF < S) {
-      lo[step % PF] = read(step + PF, 0);
-      hi[step % PF] = read(step + PF, 1);
-    }
-    lds_wait_younger_either<BLIND, 2 * ((step + PF < S) ? PF : S - 1 - step)>(clo, chi);
-    const h8 vf = cat_h4(clo, chi);
+    if constexpr (XA) {                      // slots consumed in place and refilled behind their MFMAs (qk_gemm_steps)
+      lds_wait_younger<2 * ((step + PF - 1 < S) ? PF - 1 : S - 1 - step)>(lo[step % PF], hi[step % PF]);
+      const h8 vf = cat_h4(lo[step % PF], hi[step % PF]);
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
+      for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
+      if constexpr (step + PF < S) read(step + PF, step % PF);
+    } else {
+      h4 clo = lo[step % PF], chi = hi[step % PF];
+      if constexpr (step + PF < S) read(step + PF, step % PF);
+      lds_wait_younger_either<kHand, 2 * ((step + PF < S) ? PF : S - 1 - step)>(clo, chi);
+      const h8 vf = cat_h4(clo, chi);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
+    }
     if constexpr (dt == 0 && g + 1 < G) pack(g + 1);
     sched_fence();
   });
