@@ -45,8 +45,12 @@ def _stream_ptr():
 class BaseTunner:
     operation = None                  # config operation name ("attn", ...)
 
-    def __init__(self, arch, torch_array, op_name, causal=False, softmax_scale=None, decay=False):
+    def __init__(self, arch, torch_array, op_name, causal=False, softmax_scale=None, decay=False, mask_mode=None):
         self.arch = arch
+        # RetNet only: the mask mode the operator will launch with when that is not plain causal / dense ("scan":
+        # the library scans the caller's mask for zero tiles).  Candidates are timed and verified in that mode, on the
+        # caller's own mask, which need not be zero above the diagonal; the cache entry is the causal walk's.
+        self.mask_mode = mask_mode
         self.decay = bool(decay)                  # RetNet only: torch_array[3] is log2(gamma) [H], not a mask
         self.torch_array = torch_array
         self.op_name = op_name
@@ -110,29 +114,49 @@ class BaseTunner:
 
     def _ex_args(self):
         """Operator-specific scalar arguments between the sizes and the workspace."""
+        if self.mask_mode is not None:
+            from .runtime import mask_mode
+            return [ctypes.c_int(mask_mode(self.mask_mode))]
         return [ctypes.c_int(int(self.causal))]
 
-    def profile(self, libname, device="cuda:0"):
-        """Mean milliseconds of one launch of ``libname`` on this tuner's tensors (FAILED on error)."""
+    def _workspace(self, lib, config):
+        """(tensor or None, bytes): the workspace the runtime would grant ``config`` for this problem -- a stored dS
+        beyond the runtime's limit is withheld there too, so what is timed is what will be launched.  Raises
+        torch.cuda.OutOfMemoryError like any allocation."""
+        from .runtime import _wanted
+        s = self.problem_shape
+        need = int(lib.workspace_size(s["B"], s["H"], s["Sq"], s["Sk"]))
+        if config is not None:
+            need = _wanted(config, need, s["B"], s["H"], s["Sq"], s["Sk"])
+        ws = torch.empty(need, dtype=torch.uint8, device=self.torch_array[0].device) if need else None
+        return ws, need
+
+    def profile(self, libname, device="cuda:0", config=None):
+        """Mean milliseconds of one launch of ``libname`` on this tuner's tensors (FAILED on error, and when the
+        workspace the candidate asks for cannot be allocated)."""
         lib = library.load(libname, self.operation)
         s = self.problem_shape
-        need = lib.workspace_size(s["B"], s["H"], s["Sq"], s["Sk"])
-        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=self.torch_array[0].device) if need else None
+        try:
+            ws, need = self._workspace(lib, config)
+        except torch.cuda.OutOfMemoryError:
+            return FAILED
         ptrs = [ctypes.c_void_p(t.data_ptr()) for t in self.torch_array]
         entry = lib.profile_decay if self.decay else lib.profile_ex
         ms = entry(*ptrs, s["B"], s["H"], s["Sq"], s["Sk"], *([] if self.decay else self._ex_args()),
                    ctypes.c_void_p(ws.data_ptr() if ws is not None else 0), ctypes.c_size_t(need), _stream_ptr())
         return FAILED if ms < 0 else float(ms)
 
-    def verify(self, libname):
+    def verify(self, libname, config=None):
         """Run ``libname`` once on this tuner's tensors and compare its outputs with torch math."""
         if not hasattr(self, "_reference"):
             scale = None if len(self._ex_args()) == 1 else self._ex_args()[0].value
             self._reference = verify.reference_outputs(self.operation, self.torch_array, scale, self.causal, self.decay)
         lib = library.load(libname, self.operation)
         s = self.problem_shape
-        need = lib.workspace_size(s["B"], s["H"], s["Sq"], s["Sk"])
-        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=self.torch_array[0].device) if need else None
+        try:
+            ws, need = self._workspace(lib, config)
+        except torch.cuda.OutOfMemoryError:
+            return False
         for idx in self._reference:
             self.torch_array[idx].zero_()
         ptrs = [ctypes.c_void_p(t.data_ptr()) for t in self.torch_array]
@@ -226,7 +250,7 @@ class BaseTunner:
                 # the compiler says this candidate keeps part of its working set in scratch memory: not worth timing
                 self.rejected_spills[res.config] = max(k.get("scratch_bytes", 0) for k in spills)
                 continue
-            ms = self.profile(res.lib_name)
+            ms = self.profile(res.lib_name, config=res.config)
             if ms == FAILED and self.verbose:
                 pprint.pprint(res.config)
                 print("profile runtime error")
@@ -237,7 +261,7 @@ class BaseTunner:
             libs = {res.config: res.lib_name for res in results}
             best = None
             for cfg in sorted((c for c, ms in timings.items() if ms < FAILED), key=timings.get):
-                if self.verify(libs[cfg]):
+                if self.verify(libs[cfg], config=cfg):
                     best, best_ms = cfg, timings[cfg]
                     break
                 timings[cfg] = FAILED                     # fast but wrong: never cache it

@@ -15,7 +15,7 @@ class NoValidConfigError(ValueError):
 
 WAVE = 64
 MFMA_M = 32
-BR_LIST = (64, 128, 256)
+BR_LIST = (64, 128, 256, 512)
 BC_LIST = (32, 64, 128)
 THREADS = (128, 256, 512)
 STAGES = ((1, 1), (2, 2), (2, 1), (1, 2))
@@ -32,6 +32,14 @@ def rows_per_wave(cfg):
 def blocks_per_cu(cfg):
     """Resident blocks per CU implied by the occupancy target (4 SIMDs per CU)."""
     return max(1, (cfg.waves_per_eu * 4) // _waves(cfg))
+
+
+def unit_rows(cfg):
+    """kv rows of one scores -> softmax -> PV unit of the register-fused attention forward (plain schedule):
+    ``BlockKSmem2``, a divisor of Bc; the whole tile everywhere else."""
+    if cfg.operation == "attn" and cfg.fuse_type == "register" and not getattr(cfg, "sw_pipeline", 0):
+        return getattr(cfg, "BlockKSmem2", cfg.Bc) or cfg.Bc
+    return cfg.Bc
 
 
 def dma_divisible(cfg):
@@ -61,9 +69,10 @@ def forward_reg_estimate(cfg):
         o_regs = cfg.Br * cfg.D // (nw * 64)
         return rt1 * (cfg.Kd // 16) * 4 + rt1 * nt1 * 16 + o_regs + 48
     rt = rows_per_wave(cfg) // MFMA_M
+    unit = unit_rows(cfg)
     q_regs = rt * (cfg.Kd // 16) * 4
-    s_regs = rt * (cfg.Bc // 32) * 16
-    p_regs = rt * (cfg.Bc // 32) * 4            # fp16 P, built while the fp32 scores retire
+    s_regs = rt * (unit // 32) * 16
+    p_regs = rt * (unit // 32) * 4              # fp16 P, built while the fp32 scores retire
     if cfg.fuse_type == "register":
         o_regs = rt * (cfg.D // 32) * 16
     else:
@@ -73,7 +82,9 @@ def forward_reg_estimate(cfg):
         s_regs *= 2                                   # current and next score tile are both live
     # a count of what must be live, not a prediction of what the register allocator achieves: candidates that
     # pass it and still spill are rejected by the tuning loop from the compiler's own resource report
-    return q_regs + s_regs + p_regs + o_regs + 32
+    # (a kernel this close to its budget derives its operand addresses from one register each and keeps two-slot
+    # operand rings: 24 registers besides the tiles)
+    return q_regs + s_regs + p_regs + o_regs + (24 if unit < cfg.Bc else 32)
 
 
 def forward_likely_spills(cfg):
@@ -105,6 +116,11 @@ def forward_valid(cfg, arch):
     elif cfg.Nthreads % WAVE or cfg.Br % (MFMA_M * _waves(cfg)):
         return False
     if cfg.Bc % 32 or cfg.Kd % 64 or cfg.D % 64:
+        return False
+    unit = unit_rows(cfg)
+    if unit % 32 or cfg.Bc % unit:
+        return False
+    if unit < cfg.Bc and not (cfg.num_stages_qk == 2 and cfg.num_stages_v == 2):   # no barrier between the contractions of a unit
         return False
     if _waves(cfg) > 4 * cfg.waves_per_eu:           # the block itself needs that many waves per SIMD
         return False
@@ -143,6 +159,13 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
                     if op == "attn" and fuse == "register" and (st_qk, st_v) == (2, 2):
                         piped = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, 2, 2, nthreads, True, waves_per_eu=wpe, sw_pipeline=1)
                         out.append(piped.set_fuse_type(fuse))
+                    if op == "attn" and fuse == "register" and (st_qk, st_v) == (2, 2) and br // (nthreads // WAVE) >= 2 * MFMA_M:
+                        # two or more 32-row groups per wave: a kv tile worked through in 32-row units keeps one
+                        # small score tile live, which is what lets such a wave share its SIMD with a second one
+                        for unit in (32, 64):
+                            if unit < bc:
+                                u = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, unit, 2, 2, nthreads, True, waves_per_eu=wpe)
+                                out.append(u.set_fuse_type(fuse))
                     if op == "attn" and fuse == "register" and with_splits and st_qk == st_v:
                         for ns in KV_SPLITS:   # long kv, few query rows: cut the kv range so every CU gets work
                             sp = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, waves_per_eu=wpe, kv_splits=ns)
@@ -203,7 +226,7 @@ def default_forward_config(op, dim_qk, dim_v, arch, seq_q=None, seq_k=None):
 # ---- backward (RetNet) ---------------------------------------------------------------------------------
 # Three passes of one chained-contraction kernel (dV, dK, dQ).  Br = block-resident rows, Bc = streamed rows
 # per step, for every pass; both sequence lengths must divide by both.
-BWD_BR_LIST = (64, 128, 256)
+BWD_BR_LIST = (64, 128, 256, 512)
 BWD_BC_LIST = (32, 64)
 
 
@@ -312,7 +335,7 @@ def default_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
 
 # ---- backward (attention) ------------------------------------------------------------------------------
 # A column kernel (dV, dK) and a row kernel (dQ) share Br (resident rows) and Bc (streamed rows per step).
-ATTN_BWD_BR_LIST = (64, 128, 256)
+ATTN_BWD_BR_LIST = (64, 128, 256, 512)
 ATTN_BWD_BC_LIST = (32, 64)
 
 

@@ -1,9 +1,9 @@
-"""Tile / wave / buffer variants the GPU parity suite runs to show that every configuration computes the
-same thing.  ``parity_configs()`` lists them so the build step can compile them ahead of time (nothing is
-compiled inside a GPU test)."""
-from attention_autotuner_amd.arch import MI355X
-from attention_autotuner_amd.autotuner import gfx950_space
-from attention_autotuner_amd.autotuner.configs import AttnBwdConfig, AttnConfig, RetBwdConfig, RetConfig
+"""Tile / wave / buffer variants beyond the shipping set: the matrix a parity suite runs to show that every
+configuration computes the same thing.  ``parity_configs()`` lists them so that a build step can compile them ahead
+of time (``prebuilt.build_all(extra=parity_configs())``; nothing is compiled inside a GPU test)."""
+from ..arch import MI355X
+from . import gfx950_space
+from .configs import AttnBwdConfig, AttnConfig, RetBwdConfig, RetConfig
 
 # attention forward, register-fused: (Br, Bc, Nthreads, K buffers, V buffers, waves per SIMD) for every head-size pair below
 PARITY_TILES = [
@@ -12,6 +12,13 @@ PARITY_TILES = [
     (256, 64, 512, 2, 2, 2), (128, 32, 256, 2, 2, 3), (128, 64, 256, 1, 1, 3),
 ]
 PARITY_DIMS = [(64, 64), (128, 128), (64, 128), (256, 256), (192, 192)]
+# ... with a kv tile worked through in units (two or more 32-row groups per wave): (Br, Bc, unit rows, Nthreads, waves per SIMD)
+UNIT_TILES = [(512, 128, 32, 512, 2), (512, 64, 32, 512, 2), (256, 64, 32, 256, 2), (256, 128, 64, 256, 1), (128, 64, 32, 128, 1)]
+UNIT_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64)]
+
+
+def unit_config(br, bc, unit, nt, wpe, dqk, dv):
+    return AttnConfig(br, bc, dqk, dv, dqk, unit, 2, 2, nt, True, waves_per_eu=wpe).set_fuse_type("register")
 # attention forward, LDS-fused: (Br, Bc, Nthreads, K bufs, V bufs, W1N, W2N, waves/SIMD)
 SHARED_TILES = [(128, 64, 256, 2, 2, 1, 4, 2), (64, 64, 256, 1, 1, 2, 4, 2), (64, 64, 256, 2, 1, 2, 2, 2), (64, 64, 256, 1, 1, 2, 4, 1)]
 SHARED_DIMS = [(64, 64), (128, 128), (256, 512)]
@@ -51,6 +58,12 @@ def ret_shared_wide_one_wave():
 RET_BWD_STORED_DS = [(256, 512, 128, 64, 256, 128), (256, 512, 128, 64, 256, 256), (256, 512, 128, 32, 256, 256), (64, 128, 64, 32, 128, 128)]
 
 
+# ... and with two or three Y/mask buffers and one or two Z buffers: the dS stores then stay in flight across tile
+# boundaries next to the ring's copies, under different wait counts (last element: (Y buffers, Z buffers))
+RET_BWD_STORED_DS_STAGED = [(256, 512, 128, 32, 256, 128, (2, 2)), (256, 512, 128, 32, 256, 256, (2, 1)),
+                            (64, 128, 64, 32, 128, 128, (3, 2)), (128, 128, 128, 32, 256, 128, (3, 2)), (256, 256, 128, 32, 256, 128, (3, 2))]
+
+
 def ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, ds_rows, stages=(1, 1)):
     n = nt // 64
     return RetBwdConfig(br, bc, dqk, dv, n, n, n, n, nt, True, BlockKSmem=dqk, num_stages_qk=stages[0], num_stages_mask=stages[0],
@@ -73,6 +86,8 @@ def parity_configs(arch=None):
     out.append(ret_shared_wide_one_wave())
     for t in RET_BWD_STORED_DS:
         out += [ret_bwd_stored_ds_config(*t), ret_bwd_stored_ds_config(*t[:5], 0)]      # and the same passes without it
+    for t in RET_BWD_STORED_DS_STAGED:
+        out += [ret_bwd_stored_ds_config(*t[:6], stages=t[6]), ret_bwd_stored_ds_config(*t[:5], 0, stages=t[6])]
     out += [attn_bwd_split_config(*t) for t in ATTN_BWD_SPLIT_TILES]
     out.append(AttnBwdConfig(64, 64, 128, 128, 128, 2, row_waves_per_eu=2, row_Bc=32))      # row kernel with a tile height of its own
     for br, bc, nt, st in ATTN_BWD_TILES:
@@ -89,6 +104,11 @@ def parity_configs(arch=None):
                 piped = AttnConfig(br, bc, dqk, dv, dqk, bc, 2, 2, nt, True, waves_per_eu=wpe, sw_pipeline=1).set_fuse_type("register")
                 if gfx950_space.forward_valid(piped, arch):
                     out.append(piped)
+    for dqk, dv in UNIT_DIMS:
+        for t in UNIT_TILES:
+            cfg = unit_config(*t, dqk, dv)
+            if gfx950_space.forward_valid(cfg, arch):
+                out.append(cfg)
     for dqk, dv, ns in SPLIT_VARIANTS:
         out.append(AttnConfig(128, 64, dqk, dv, dqk, 64, 2, 2, 256, True, waves_per_eu=2, kv_splits=ns).set_fuse_type("register"))
     for dqk, dv in SHARED_DIMS:

@@ -90,15 +90,15 @@ class AttnTunner(_ForwardTunner):
 class RetTunner(_ForwardTunner):
     operation = "ret"
 
-    def __init__(self, arch, torch_array, causal=False, decay=False):
-        super().__init__(arch, torch_array, "retnet", causal=causal or decay, decay=decay)
+    def __init__(self, arch, torch_array, causal=False, decay=False, mask_mode=None):
+        super().__init__(arch, torch_array, "retnet", causal=causal or decay, decay=decay, mask_mode=mask_mode)
 
 
 class RetBwdTunner(BaseTunner):
     operation = "ret_bwd"
 
-    def __init__(self, arch, torch_array, causal=False, decay=False):
-        super().__init__(arch, torch_array, "retnet_bwd", causal=causal or decay, decay=decay)
+    def __init__(self, arch, torch_array, causal=False, decay=False, mask_mode=None):
+        super().__init__(arch, torch_array, "retnet_bwd", causal=causal or decay, decay=decay, mask_mode=mask_mode)
         if _is_rocm(arch):
             self.Br_list = list(getattr(gfx950_space, "BWD_BR_LIST", (64, 128)))
             self.Bc_list = list(getattr(gfx950_space, "BWD_BC_LIST", (32, 64, 128)))

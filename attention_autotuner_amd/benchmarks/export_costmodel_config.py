@@ -5,14 +5,14 @@ the reference runs Nsight Compute once per candidate and reads "Elapsed Cycles";
 counter run (GRBM_GUI_ACTIVE, busy cycles summed over the 8 XCDs) covers every candidate, because the
 candidates are separately built libraries that one process can launch back to back.
 
-    python -m attention_autotuner_amd.benchmarks.export_costmodel_config attn 4 32 2048 2048 128 128 [--causal] [--limit N] [--out FILE]
+    python -m attention_autotuner_amd.benchmarks.export_costmodel_config attn 4 32 2048 2048 128 128 [--causal] [--limit N] [--only-built] [--out FILE]
 
 The outer invocation builds the candidate libraries, starts itself under ``rocprofv3 --pmc`` with
 ``--run-candidates`` (that inner process launches every candidate twice: one warm-up, one counted),
 matches the counter rows to the candidates by dispatch order and writes a JSON list of
 
     {"config": {...}, "cost_model_config": [[Sq, Sk, dqk, dv], [Br, Bc, BlockK, D], [wave tile of the first
-     contraction], [wave tile of the second], B, H], "cycles": int, "lds_bytes": int, "registers": int}
+     contraction], [wave tile of the second], B, H], "causal": bool, "cycles": int, "lds_bytes": int, "registers": int}
 
 in the tuple layout of the reference's exporter (wave tiles are (rows, columns, 16): the rows and
 columns one wave computes per step and the MFMA k depth).
@@ -36,12 +36,16 @@ TUNERS = {"attn": "AttnTunner", "ret": "RetTunner"}
 XCDS = 8
 
 
-def candidates(op, dims, causal, limit):
+def candidates(op, dims, causal, limit, only_built=False):
+    """The tuner's candidates for the problem (unsplit ones: one kernel per launch); ``only_built``: those whose
+    library is already in the build directory (a machine without a compiler, or a process that must not start one)."""
     from ..autotuner import tunner
     b, h, sq, sk, dqk, dv = dims
     arrays = make_tensors(op, b, h, sq, sk, dqk, dv, "meta")
     t = getattr(tunner, TUNERS[op])(MI355X(), arrays, causal=causal)
     cfgs = [c for c in t.get_tuned_configs() if t._fits_problem(c) and getattr(c, "kv_splits", 1) == 1]
+    if only_built:
+        cfgs = [c for c in cfgs if os.path.exists(codegen.library_path(c))]
     return cfgs[:limit] if limit else cfgs
 
 
@@ -57,7 +61,7 @@ def cost_model_tuple(cfg, dims):
     return [[sq, sk, dqk, dv], [cfg.Br, cfg.Bc, cfg.BlockKSmem, cfg.D], list(tile1), list(tile2), b, h]
 
 
-def run_candidates(op, dims, causal, limit):
+def run_candidates(op, dims, causal, limit, only_built=False):
     """Inner mode (under rocprofv3): launch every candidate library twice."""
     import ctypes
     b, h, sq, sk, dqk, dv = dims
@@ -65,7 +69,7 @@ def run_candidates(op, dims, causal, limit):
     ptrs = [ctypes.c_void_p(t.data_ptr()) for t in arrays]
     extra = [ctypes.c_float(dqk ** -0.5), ctypes.c_int(int(causal))] if op == "attn" else [ctypes.c_int(int(causal))]
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    for cfg in candidates(op, dims, causal, limit):
+    for cfg in candidates(op, dims, causal, limit, only_built):
         path = codegen.library_path(cfg)
         if not os.path.exists(path):
             continue
@@ -84,20 +88,25 @@ def main(argv=None):
     ap.add_argument("dims", type=int, nargs=6, metavar="N", help="B H Sq Sk dqk dv")
     ap.add_argument("--causal", action="store_true")
     ap.add_argument("--limit", type=int, default=0, help="only the first N candidates")
+    ap.add_argument("--only-built", action="store_true", help="only candidates whose library is already built (nothing is compiled)")
     ap.add_argument("--out", default=None)
     ap.add_argument("--run-candidates", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args(argv)
     if args.run_candidates:
-        run_candidates(args.op, args.dims, args.causal, args.limit)
+        run_candidates(args.op, args.dims, args.causal, args.limit, args.only_built)
         return 0
 
     arch = MI355X()
-    cfgs = candidates(args.op, args.dims, args.causal, args.limit)
-    libs = codegen.compile_parallel(cfgs, arch, timeout=300)
-    cfgs = [c for c, l in zip(cfgs, libs) if l is not None]
+    cfgs = candidates(args.op, args.dims, args.causal, args.limit, args.only_built)
+    if not cfgs:
+        raise RuntimeError("no candidate library to count")
+    if not args.only_built:
+        libs = codegen.compile_parallel(cfgs, arch, timeout=300)
+        cfgs = [c for c, l in zip(cfgs, libs) if l is not None]
     out_dir = tempfile.mkdtemp(prefix="aat_costmodel_", dir=os.environ.get("TMPDIR", "/tmp"))
     inner = [sys.executable, "-m", "attention_autotuner_amd.benchmarks.export_costmodel_config", args.op,
-             *map(str, args.dims), "--run-candidates", "--limit", str(args.limit)] + (["--causal"] if args.causal else [])
+             *map(str, args.dims), "--run-candidates", "--limit", str(args.limit)] + (["--causal"] if args.causal else []) + \
+            (["--only-built"] if args.only_built else [])
     cmd = ["rocprofv3", "--pmc", "GRBM_GUI_ACTIVE", "--output-format", "csv", "-d", out_dir, "-o", "cm", "--", *inner]
     res = subprocess.run(cmd, capture_output=True, text=True, timeout=1800)
     launched = [l.split(" ", 1)[1] for l in res.stdout.splitlines() if l.startswith("LAUNCHED ")]
@@ -116,7 +125,7 @@ def main(argv=None):
     records = []
     for i, name in enumerate(launched):
         cfg = by_name[name]
-        records.append({"config": cfg.to_dict(), "cost_model_config": cost_model_tuple(cfg, args.dims),
+        records.append({"config": cfg.to_dict(), "cost_model_config": cost_model_tuple(cfg, args.dims), "causal": bool(args.causal),
                         "cycles": int(float(rows[2 * i + 1]["Counter_Value"]) / XCDS),
                         "lds_bytes": gfx950_space.forward_lds_bytes(cfg), "registers": gfx950_space.forward_reg_estimate(cfg)})
     out = args.out or f"{args.op}_{args.dims[4]}_{args.dims[5]}_costmodel.json"

@@ -88,7 +88,9 @@ static void test_regfuse_attention(const ProblemShape& ps, const Buffers& b) {
     HIP_OK(hipFuncSetAttribute((const void*)persist, hipFuncAttributeMaxDynamicSharedMemorySize, TP::kSmemBytes));
     HIP_OK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)persist, NT, TP::kSmemBytes));
     HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-    if (!ps.causal && (ps.Sk / Bc) % 2 == 0 && ps.Sk <= 1792 && items > per_cu * cus) resident = per_cu * cus;
+    hipFuncAttributes attr;                        // as the library: never a build of the persistent kernel that spills
+    HIP_OK(hipFuncGetAttributes(&attr, (const void*)persist));
+    if (attr.localSizeBytes == 0 && !ps.causal && (ps.Sk / Bc) % 2 == 0 && ps.Sk <= 1792 && items > per_cu * cus) resident = per_cu * cus;
     if (resident > 0) {
       auto t = aat_bench::do_bench([&] {
         persist<<<dim3(resident), dim3(NT), TP::kSmemBytes, 0>>>(b.q, b.k, b.v, b.o, nullptr, ps.H, ps.Sk, ps.Sq, scale,

@@ -59,7 +59,12 @@ int resident_blocks() {{
   int blocks = cached[dev].load(std::memory_order_relaxed);
   if (blocks == 0) {{
     int per_cu = 0, cus = 0;
-    if (aat::allow_lds(kernel_persist, shared_mem_persist) != hipSuccess ||
+    // The persistent kernel requests the next row block's Q fragments into live registers behind the compiler's back
+    // and waits for them a tile later.  That is sound only while those registers stay registers: a build whose
+    // allocator spilled anything (scratch bytes per lane != 0) may have parked a fragment in memory before it arrived.
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kernel_persist)) != hipSuccess || attr.localSizeBytes != 0 ||
+        aat::allow_lds(kernel_persist, shared_mem_persist) != hipSuccess ||
         hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel_persist), Nthreads, shared_mem_persist) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || per_cu <= 0 || cus <= 0)
       blocks = -1;

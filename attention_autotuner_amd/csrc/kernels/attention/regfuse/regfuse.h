@@ -71,7 +71,11 @@ struct AttnFwdRegfuse {
     static constexpr int kSmemBytes = kFit > kMainBytes ? kFit : kMainBytes;
     static constexpr int kInSpare = (kSmemBytes - kMainBytes) / kStageWave;
     static constexpr int kInK = kKBytes / kStageWave, kInV = kVBytes / kStageWave;
-    static constexpr bool kOk = NSK == 2 && NSV == 2 && kInSpare + kInK + kInV >= NW;
+    // WPE >= 2: the next row block's Q fragments are requested into live registers behind the compiler's back.  With the
+    // unified register file of two or more waves per SIMD those registers stay where they are; a wave that owns the
+    // split file (256 vector + 256 accumulation registers) has its fragments moved between the two classes at the
+    // compiler's discretion, and a copy made before the data has arrived carries stale values.
+    static constexpr bool kOk = NSK == 2 && NSV == 2 && WPE >= 2 && kInSpare + kInK + kInV >= NW;
     static constexpr bool kSharesBuffers = kInSpare < NW;   // then every wave must be done with the last tile first
     static constexpr int kOutputStores = RT * D / 16;       // 16-byte-per-lane store instructions of one output tile
     static_assert(kOutputStores + RT < 64, "vmcnt is a 6-bit counter");

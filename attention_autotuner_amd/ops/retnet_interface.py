@@ -69,7 +69,9 @@ class RetNetAttn(torch.autograd.Function):
         reused = causal if torch.is_tensor(causal) else None      # a scan taken earlier (retnet_mask_scan)
         if reused is not None:
             causal = None
-        tuner = RetTunner(arch=device_type, torch_array=arrays, causal=causal is None or bool(causal))
+        # ... but a tuning run on a cache miss times and verifies its candidates in the mode launched here, on this mask
+        tuner = RetTunner(arch=device_type, torch_array=arrays, causal=causal is None or bool(causal),
+                          mask_mode="scan" if causal is None else None)
         cc = resolve(tuner, lambda: gfx950_space.default_forward_config("ret", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
         rt = Runtime(device_type, cc)
         scan = None
@@ -104,7 +106,8 @@ class RetNetAttn(torch.autograd.Function):
         # touch it (dQ is produced directly), so a token buffer stands in for the [B,H,S_q,d_qk] tensor.
         dq_accum = torch.zeros(1, device=q.device, dtype=torch.float32)
         arrays = [q, k, v, mask, do, r, dq, dk, dv, dq_accum]
-        tuner = RetBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal is None or bool(ctx.causal))
+        tuner = RetBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal is None or bool(ctx.causal),
+                             mask_mode="scan" if ctx.mask_scan is not None else None)
         cc = resolve(tuner, lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
         if ctx.mask_scan is not None:
             Runtime(device_type, cc).apply(arrays, causal="scanned", workspace=ctx.mask_scan)

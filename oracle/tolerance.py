@@ -80,3 +80,28 @@ def assert_close_rounded_operand(got, ref, terms, what=""):
           f"{lit_large:.2f} ulp over the {n_large} entries above")
     assert ok, (what, worst, ratio)
     return worst, ratio
+
+
+def literal_rule_report(got, ref, what="", atol=ATOL):
+    """The contract's bound read literally -- |err| <= ``atol`` for EVERY entry, whatever its magnitude -- against ``ref``:
+    prints and returns how many entries exceed it, the largest error, and the band of positions (second-to-last and
+    last dimension) the exceeding entries lie in.  A measurement, not an assertion: see the header for why fp16 cannot
+    hold that bound above |ref| = 4 and why rounded operands exceed it on rows that see one or two kv positions."""
+    got = got.detach().float().cpu()
+    ref = ref.detach().float().cpu()
+    err = (got - ref).abs()
+    over = err > atol
+    n = int(over.sum().item())
+    out = {"entries": err.numel(), "exceeding": n, "max_err": err.max().item()}
+    if n:
+        idx = over.nonzero()
+        out["rows"] = (int(idx[:, -2].min()), int(idx[:, -2].max()))
+        out["cols"] = (int(idx[:, -1].min()), int(idx[:, -1].max()))
+        out["min_abs_ref_of_exceeding"] = ref[over].abs().min().item()
+        small = over & (ref.abs() < SMALL)
+        out["exceeding_with_abs_ref_below_4"] = int(small.sum().item())
+        out["max_err_with_abs_ref_below_4"] = err[small].max().item() if small.any() else 0.0
+    print(f"{what}: literal |err| <= {atol:g} for every entry: {n} of {err.numel()} exceed it, max |err| {out['max_err']:.3e}"
+          + (f", rows {out['rows'][0]}..{out['rows'][1]}, columns {out['cols'][0]}..{out['cols'][1]}, smallest |ref| among them "
+             f"{out['min_abs_ref_of_exceeding']:.3f}, {out['exceeding_with_abs_ref_below_4']} of them with |ref| < 4 (max |err| there {out['max_err_with_abs_ref_below_4']:.3e})" if n else ""))
+    return out

@@ -8,7 +8,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 TESTS = os.path.dirname(os.path.abspath(__file__))
 if TESTS not in sys.path:
-    sys.path.insert(0, TESTS)               # reference_space, parity_matrix
+    sys.path.insert(0, TESTS)               # reference_space
 
 # Tests never start a tuning run implicitly: a cache miss falls back to the default configuration.
 os.environ.setdefault("AAT_TUNE_ON_MISS", "0")

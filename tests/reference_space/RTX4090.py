@@ -1,24 +1,9 @@
-"""NVIDIA RTX 4090 limits (enumeration checks only, see A100.py)."""
-from attention_autotuner_amd.arch import Arch
+"""The package's RTX 4090 descriptor with the reference's NVIDIA search space attached (enumeration checks only,
+see A100.py)."""
+from attention_autotuner_amd.arch import RTX4090 as _RTX4090
 
 from . import legacy_space
 
 
-class RTX4090(Arch):
-    reg_cap = 65536
-    smem_cap = 100 * 1024
-    max_smem_usage = 100 * 1024
-    compute_max_core = 128
-    warp_size = 32
-    sm_partition = 4
-    transaction_size = (32, 128)
-    bandwidth = (1008, 0)
-    platform = "CUDA"
-    compute_capability = "89"
-    register_per_thread = 255
-    cutlass_mma = (16, 8, 16)
+class RTX4090(_RTX4090):
     search_space = legacy_space        # the tuners enumerate a non-ROCm descriptor with the space it brings along
-
-    def __init__(self):
-        super().__init__()
-        self.cutlass_mma = type(self).cutlass_mma

@@ -16,7 +16,7 @@ import attention_autotuner_amd as aat
 from attention_autotuner_amd.arch import MI355X
 from attention_autotuner_amd.autotuner import Runtime, codegen, gfx950_space, library, prebuilt
 from attention_autotuner_amd.autotuner.configs import AttnBwdConfig
-import parity_matrix
+from attention_autotuner_amd.autotuner import prebuilt_extra as parity_matrix
 from oracle import ref_op, tolerance
 
 pytestmark = pytest.mark.gpu

@@ -92,3 +92,36 @@ def test_tuner_prunes_with_the_shipped_model_and_not_without(monkeypatch):
     monkeypatch.setenv("AAT_TUNE_PRUNE", "0")
     exhaustive = AttnTunner(MI355X(), _meta(4, 32, 2048), causal=True)
     assert exhaustive.cost_model is None and exhaustive.prune(cfgs) == cfgs
+
+
+@pytest.mark.gpu
+def test_cycle_exporter_counts_prebuilt_candidates_in_the_reference_tuple_layout(tmp_path):
+    """benchmarks/export_costmodel_config.py end to end on a few libraries that are already built: one rocprofv3 counter
+    run, one record per candidate in the tuple layout of reference python/tests/export_costmodel_config.py:31-56
+    (``Nwarps`` there counts 32-lane warps, here 64-lane waves), cycles that a fit can read back."""
+    import json
+    import subprocess
+    import sys
+    out = tmp_path / "export.json"
+    dims = (1, 8, 512, 512, 128, 128)
+    env = dict(os.environ, AAT_NO_JIT="1", TMPDIR=str(tmp_path))
+    done = subprocess.run([sys.executable, "-m", "attention_autotuner_amd.benchmarks.export_costmodel_config", "attn",
+                           *map(str, dims), "--only-built", "--limit", "4", "--out", str(out)],
+                          capture_output=True, text=True, timeout=300, env=env,
+                          cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert done.returncode == 0, done.stdout[-2000:] + done.stderr[-2000:]
+    records = json.loads(out.read_text())
+    assert len(records) == 4
+    b, h, sq, sk, dqk, dv = dims
+    for r in records:
+        c = r["config"]
+        nw = c["Nthreads"] // 64
+        w1n, w2n = (c["warps_mma1_n"], c["warps_mma_n"]) if c["fuse_type"] == "shared" else (1, 1)
+        assert r["cost_model_config"] == [[sq, sk, dqk, dv], [c["Br"], c["Bc"], c["BlockKSmem"], c["D"]],
+                                          [c["Br"] // (nw // w1n), c["Bc"] // w1n, 16], [c["Br"] // (nw // w2n), c["D"] // w2n, 16], b, h]
+        # 1 x 8 x 512 x 512 x (128 + 128) x 2 flop at no more than 2.5 PFLOP/s and 2.4 GHz, and nowhere near a millisecond
+        assert 1000 < r["cycles"] < 2_000_000 and r["causal"] is False
+        assert r["lds_bytes"] > 0 and r["registers"] > 0
+    samples = costmodel.samples_from_export(str(out))
+    assert [s[1] for s in samples] == [(b, h, sq, sk)] * 4 and all(s[3] == r["cycles"] for s, r in zip(samples, records))
+    assert np.isfinite(costmodel.CostModel(unit="cycles").fit(samples).weights).all()

@@ -142,6 +142,9 @@ def test_mi355x_space_is_valid_and_nonempty():
                 nw = c.Nthreads // 64
                 assert nw % c.warps_mma1_n == 0 and nw % c.warps_mma_n == 0
                 assert c.Bc % (32 * c.warps_mma1_n) == 0 and dv % (32 * c.warps_mma_n) == 0
-            assert c.BlockKSmem == dqk and c.BlockKSmem2 == c.Bc
+            assert c.BlockKSmem == dqk and c.Bc % c.BlockKSmem2 == 0
+            if c.BlockKSmem2 != c.Bc:     # units inside a kv tile: plain register-fused schedule, two or more row groups per wave
+                assert c.fuse_type == "register" and not c.sw_pipeline and (c.num_stages_qk, c.num_stages_v) == (2, 2)
+                assert c.BlockKSmem2 % 32 == 0 and c.Br // (c.Nthreads // 64) >= 64
     with pytest.raises(RuntimeError):
         AttnTunner(A100(), _fake_arrays(64, 64)).tune()

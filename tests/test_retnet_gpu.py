@@ -18,6 +18,7 @@ import torch
 import attention_autotuner_amd as aat
 from attention_autotuner_amd.arch import MI355X
 from attention_autotuner_amd.autotuner import RetBwdConfig, RetConfig, Runtime, codegen, gfx950_space, library
+from attention_autotuner_amd.autotuner import prebuilt_extra as parity_matrix
 from oracle import ref_op, tolerance
 
 pytestmark = pytest.mark.gpu
@@ -79,12 +80,12 @@ def test_config3_forward_b4_h8_s2048_dqk256_dv512_and_r():
     cfg = gfx950_space.default_forward_config("ret", 256, 512, ARCH, 2048, 2048)
     for causal in (False, True):            # the decay mask is lower-triangular: skipping tiles must not change anything
         Runtime(ARCH, cfg).apply(arrays + [o, r], causal=causal)
-        for b, h in ((0, 0), (2, 5), (3, 7)):
-            o_ref, r_ref = ref_op.retnet_ref(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], mask[h:h + 1], return_r=True)
-            ok, ex = _close(o[b:b + 1, h:h + 1], o_ref)
-            assert ok, (causal, b, h, ex)
-            rel = ((r[b, h].cpu() - r_ref[0, 0]).abs() / r_ref[0, 0]).max().item()
-            assert rel <= 1e-3, (causal, b, h, rel)
+        for b in range(4):                  # every (batch, head) slice, one batch element (all 8 heads and their mask rows) at a time
+            o_ref, r_ref = ref_op.retnet_ref(q[b:b + 1], k[b:b + 1], v[b:b + 1], mask, return_r=True)
+            ok, ex = _close(o[b:b + 1], o_ref)
+            assert ok, (causal, b, ex)
+            rel = ((r[b].cpu() - r_ref[0]).abs() / r_ref[0]).max().item()
+            assert rel <= 1e-3, (causal, b, rel)
     # size-independent properties on the whole problem
     assert torch.isfinite(o.float()).all()
     assert (r >= 1).all()
@@ -94,9 +95,24 @@ def test_config3_forward_b4_h8_s2048_dqk256_dv512_and_r():
 def test_config4_forward_backward_b4_h8_s2048_dqk256_dv512(causal):
     q, k, v, mask, do = _inputs(4, 8, 2048, 2048, 256, 512, seed=4)
     o, dq, dk, dv_ = _run(q, k, v, mask, do, causal=causal)
-    for b, h in ((0, 0), (3, 7)):
-        sl = (slice(b, b + 1), slice(h, h + 1))
-        _grads_close(f"config 4 ({b},{h})", (dq[sl], dk[sl], dv_[sl]), q[sl], k[sl], v[sl], mask[h:h + 1], do[sl])
+    over = {}
+    for b in range(4):                      # every (batch, head) slice, one batch element at a time
+        sl = slice(b, b + 1)
+        tolerance.assert_close(o[sl].detach(), ref_op.retnet_ref(q[sl], k[sl], v[sl], mask), f"config 4 batch {b} o")
+        _grads_close(f"config 4 batch {b}", (dq[sl], dk[sl], dv_[sl]), q[sl], k[sl], v[sl], mask, do[sl])
+        # the contract's 2e-3 read literally, for every entry, against the exact fp32 form: measured, printed, bounded below
+        for name, g, want in zip(("dq", "dk", "dv"), (dq[sl], dk[sl], dv_[sl]), ref_op.retnet_bwd_ref(q[sl], k[sl], v[sl], mask, do[sl])):
+            rep = tolerance.literal_rule_report(g, want, f"config 4 batch {b} {name} vs exact fp32 form")
+            over.setdefault(name, []).append(rep)
+    # what exceeds the literal bound is a thin set: fewer than one entry in ten thousand, all of them on the first eight rows
+    # of the decay mask, where a gradient entry is a handful of products -- most too large for fp16 to hold 2e-3 at all
+    # (|ref| >= 4: up to 2e-2 at |ref| > 32, less than one fp16 ulp there), the rest within 8e-3 (6.6e-3 measured, on an entry
+    # whose large terms cancel: the rounded-operand bound 2^-11 T of the check above scales with the terms, not with the result)
+    for name, reps in over.items():
+        total, n = sum(r["entries"] for r in reps), sum(r["exceeding"] for r in reps)
+        assert n <= 1e-4 * total, (name, n, total)
+        assert all(r.get("max_err_with_abs_ref_below_4", 0.0) <= 8e-3 for r in reps), (name, [r.get("max_err_with_abs_ref_below_4") for r in reps])
+        assert all(r["rows"][1] <= 7 for r in reps if r["exceeding"]), (name, [r.get("rows") for r in reps])
     # linearity in dO on the whole problem: grad(2*dO) == 2*grad(dO) up to fp16 rounding of the outputs
     if not causal:
         return
@@ -151,7 +167,6 @@ def test_one_wave_forward_with_256_accumulators_at_dqk256_dv512(which):
     256 accumulation registers of a wave that has its SIMD to itself, rescaled in place when the lazy normaliser moves
     (the sums of |S| pass 256 within the first tiles here).  It is built without a byte of scratch and must be right
     for every way of handing over the mask."""
-    import parity_matrix
     cfg = parity_matrix.ret_register_wide() if which == "register" else parity_matrix.ret_shared_wide_one_wave()
     assert gfx950_space.forward_valid(cfg, ARCH) and os.path.exists(codegen.library_path(cfg))
     report = [k for k in codegen.resource_usage(codegen.library_path(cfg)) if "ret_fwd_" in k["kernel"]]
@@ -428,14 +443,13 @@ def _bwd_through(cfg, arrays, mode, scan_of=None, decay=False):
     return outs
 
 
-@pytest.mark.parametrize("dqk,dv,br,bc,nt,ds_rows", __import__("parity_matrix").RET_BWD_STORED_DS)
+@pytest.mark.parametrize("dqk,dv,br,bc,nt,ds_rows,stages", [t + ((1, 1),) for t in parity_matrix.RET_BWD_STORED_DS] + parity_matrix.RET_BWD_STORED_DS_STAGED)
 @pytest.mark.parametrize("sq,sk", [(256, 256), (256, 512), (512, 256)])
-def test_backward_with_a_stored_ds_agrees_with_the_one_that_evaluates_it_twice(dqk, dv, br, bc, nt, ds_rows, sq, sk):
+def test_backward_with_a_stored_ds_agrees_with_the_one_that_evaluates_it_twice(dqk, dv, br, bc, nt, ds_rows, stages, sq, sk):
     """The dQ pass writes only the dS tiles it walks, so the workspace is full of NaN elsewhere and the dK kernel must
     take exactly the written part: dense, causal-promise and scanned walks of a decay mask, a banded mask, S_q != S_kv."""
-    import parity_matrix
-    with_ds = parity_matrix.ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, ds_rows)
-    plain = parity_matrix.ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, 0)
+    with_ds = parity_matrix.ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, ds_rows, stages)
+    plain = parity_matrix.ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, 0, stages)
     assert gfx950_space.backward_valid(with_ds, ARCH) and os.path.exists(codegen.library_path(with_ds))
     b, h = 2, 3
     q, k, v, do, gamma, exact = _decay_problem(b, h, sq, sk, dqk, dv, seed=sq + sk + ds_rows)
@@ -463,7 +477,6 @@ def test_backward_with_a_stored_ds_agrees_with_the_one_that_evaluates_it_twice(d
 def test_without_room_for_ds_the_library_evaluates_it_twice():
     """The reference-signature entry points have no workspace to give, and a caller of the others may give a small one or
     none: dK then comes from the chained pass, and the results are those of the library built without the stored dS."""
-    import parity_matrix
     t = parity_matrix.RET_BWD_STORED_DS[0]
     libs = [library.load(Runtime(ARCH, parity_matrix.ret_bwd_stored_ds_config(*t[:5], rows))._path(), "ret_bwd") for rows in (t[5], 0)]
     q, k, v, mask, do = (x.cuda() for x in _inputs(1, 2, 256, 256, 256, 512, seed=5))
@@ -496,7 +509,6 @@ def test_without_room_for_ds_the_library_evaluates_it_twice():
 def test_runtime_grants_the_room_for_ds_up_to_a_cap(monkeypatch):
     """Beyond ``runtime.MAX_DS_BYTES`` the runtime hands the library the mask scan's bytes only and the library
     evaluates dS twice: the results of the configuration without the stored dS."""
-    import parity_matrix
     from attention_autotuner_amd.autotuner import runtime
     t = parity_matrix.RET_BWD_STORED_DS[0]
     with_ds, plain = parity_matrix.ret_bwd_stored_ds_config(*t), parity_matrix.ret_bwd_stored_ds_config(*t[:5], 0)

@@ -6,7 +6,7 @@ import os
 
 import pytest
 
-import parity_matrix
+from attention_autotuner_amd.autotuner import prebuilt_extra as parity_matrix
 import torch
 
 from attention_autotuner_amd.arch import MI355X
@@ -106,3 +106,68 @@ def test_a_library_that_is_not_built_is_compiled_on_this_machine_and_runs(tmp_pa
     for causal in (False, True):
         rt.apply([q.cuda(), k.cuda(), v.cuda(), o], causal=causal)
         assert (o.float().cpu() - ref_op.attention_ref(q, k, v, None, causal)).abs().max().item() <= 2e-3
+
+
+def test_default_operator_call_on_a_dense_mask_tunes_in_the_mode_it_launches(tmp_path, monkeypatch):
+    """``RetNetAttnFunc(q, k, v, mask, arch)`` as the reference calls it (reference python/tests/test_runtime.py:38-62:
+    a dense N(0,1) mask), with an empty tuning cache and tuning on a miss: the operator launches the scanning walk,
+    so the tuners it starts must time and verify their candidates in that mode on this mask -- under the causal
+    promise every candidate would fail the guard on a mask that is not zero above the diagonal.  Candidates are
+    restricted to libraries built ahead of time (nothing compiles here)."""
+    import attention_autotuner_amd as aat
+    from attention_autotuner_amd.autotuner import base_tunner
+    from attention_autotuner_amd.autotuner.tunner import RetTunner
+    from attention_autotuner_amd.ops import _resolve
+    from oracle import ref_op, tolerance
+    monkeypatch.setenv("AAT_TUNE_ON_MISS", "1")
+    monkeypatch.setattr(base_tunner, "DEFAULT_CACHE_DIR", str(tmp_path / "cache"))
+    monkeypatch.setattr(_resolve, "DEFAULT_LOG_DIR", str(tmp_path / "logs"))
+    fwd = [c for c in parity_matrix.parity_configs(ARCH) if c.operation == "ret" and (c.Kd, c.D) == (128, 128)
+           and os.path.exists(codegen.library_path(c))]
+    bwd = []
+    for seq in (None, 128, 64):
+        c = gfx950_space.default_backward_config(128, 128, ARCH, seq, seq)
+        if c not in bwd and os.path.exists(codegen.library_path(c)):
+            bwd.append(c)
+    assert len(fwd) >= 2 and bwd
+    monkeypatch.setattr(RetTunner, "get_tuned_configs", lambda self: fwd)
+    monkeypatch.setattr(RetBwdTunner, "get_tuned_configs", lambda self: bwd)
+    g = torch.Generator().manual_seed(0)
+    q, k, v, do = (torch.randn(1, 2, 256, 128, generator=g).half() for _ in range(4))
+    mask = torch.randn(2, 256, 256, generator=g).half()                # dense: nothing to skip, nothing promised
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = aat.RetNetAttnFunc(qc, kc, vc, mask.cuda(), ARCH)
+    o.backward(do.cuda())
+    torch.cuda.synchronize()
+    tolerance.assert_close(o.detach(), ref_op.retnet_ref(q, k, v, mask), "tuned on a miss, dense mask: o")
+    for name, got, want in zip(("dq", "dk", "dv"), (qc.grad, kc.grad, vc.grad),
+                               ref_op.retnet_bwd_ref(q, k, v, mask, do, operand_dtype=torch.float16)):
+        tolerance.assert_close(got, want, f"tuned on a miss, dense mask: {name}")
+    written = sorted(os.listdir(tmp_path / "cache"))
+    assert written == ["best_config_retnet_MI355X_128_128_b1h2q256k256_c1.json",
+                       "best_config_retnet_bwd_MI355X_128_128_b1h2q256k256_c1.json"], written
+    logs = sorted(os.listdir(tmp_path / "logs"))
+    assert logs == ["profile_result_ret_128_128.txt", "profile_result_ret_bwd_128_128.txt"], logs
+
+
+def test_a_stored_ds_beyond_the_runtime_limit_is_timed_as_it_will_be_launched(monkeypatch):
+    """The tuner grants a candidate the workspace the runtime would: above the runtime's dS limit the room for a stored dS
+    is withheld in both, so such a candidate is timed on the chained passes it will actually run."""
+    from attention_autotuner_amd.autotuner import library, runtime
+    cfg = parity_matrix.ret_bwd_stored_ds_config(64, 128, 64, 32, 128, 128)
+    lib_path = codegen.library_path(cfg)
+    assert os.path.exists(lib_path)
+    arrays = make_tensors("ret_bwd", 1, 2, 256, 256, 64, 128, "cuda")
+    tuner = RetBwdTunner(ARCH, arrays, causal=True)
+    lib = library.load(lib_path, "ret_bwd")
+    full = int(lib.workspace_size(1, 2, 256, 256))
+    ds_bytes = 2 * 1 * 2 * 256 * 256
+    assert tuner._workspace(lib, cfg)[1] == full and full > ds_bytes
+    monkeypatch.setattr(runtime, "MAX_DS_BYTES", ds_bytes - 1)
+    assert tuner._workspace(lib, cfg)[1] == full - ds_bytes
+    assert tuner.profile(lib_path, config=cfg) < base_tunner_failed() and tuner.verify(lib_path, config=cfg)
+
+
+def base_tunner_failed():
+    from attention_autotuner_amd.autotuner import base_tunner
+    return base_tunner.FAILED
