@@ -163,13 +163,40 @@ def samples_from_tuning_log(path, op, dim_qk, dim_v, shape, causal=False, failed
     return out
 
 
-def samples_from_export(path):
-    """(cfg, shape, causal, cycles) from the JSON of ``benchmarks/export_costmodel_config.py``."""
+def samples_from_export(path, max_scratch_bytes=None):
+    """(cfg, shape, causal, cycles) from the JSON of ``benchmarks/export_costmodel_config.py``.  ``max_scratch_bytes``:
+    leave out the candidates whose library keeps more than that per lane in scratch memory -- the tuning loop does not
+    time those either, and their cycle counts (ten times the rest) would be all a least-squares fit sees."""
     with open(path) as f:
         records = json.load(f)
     out = []
     for r in records:
+        if max_scratch_bytes is not None and (r.get("scratch_bytes") or 0) > max_scratch_bytes:
+            continue
         cfg = supported_configs[r["config"]["operation"]].from_dict(r["config"])
         (sq, sk, _, _), _, _, _, b, h = r["cost_model_config"]
         out.append((cfg, (b, h, sq, sk), bool(r.get("causal", False)), float(r["cycles"])))
     return out
+
+
+def main(argv=None):
+    """``python -m attention_autotuner_amd.autotuner.costmodel fit EXPORT.json [EXPORT.json ...] --out MODEL.json``:
+    fit on the cycle counts of one or more exporter runs (candidates that spill left out) and write the model."""
+    import argparse
+    from . import codegen
+    ap = argparse.ArgumentParser()
+    ap.add_argument("command", choices=["fit"])
+    ap.add_argument("exports", nargs="+")
+    ap.add_argument("--out", required=True)
+    args = ap.parse_args(argv)
+    samples = [s for path in args.exports for s in samples_from_export(path, codegen.MAX_SCRATCH_BYTES)]
+    model = CostModel(unit="cycles").fit(samples)
+    model.save(args.out)
+    print(json.dumps({"samples": len(samples), "out": args.out, "rank_of_best": model.rank_of_best(samples)}))
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+    sys.exit(main())
+

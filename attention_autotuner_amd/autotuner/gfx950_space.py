@@ -19,6 +19,7 @@ BR_LIST = (64, 128, 256, 512)
 BC_LIST = (32, 64, 128)
 THREADS = (128, 256, 512)
 STAGES = ((1, 1), (2, 2), (2, 1), (1, 2))
+KV_SPLITS = (2, 4, 8, 16)
 
 
 def _waves(cfg):
@@ -138,7 +139,6 @@ def forward_valid(cfg, arch):
     return forward_reg_estimate(cfg) <= arch.register_per_thread // cfg.waves_per_eu
 
 
-KV_SPLITS = (2, 4, 8, 16)
 
 
 def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "shared"), with_splits=False):
@@ -164,8 +164,9 @@ def forward_candidates(op, br, bc, dim_qk, dim_v, fuse_types=("register", "share
                         # small score tile live, which is what lets such a wave share its SIMD with a second one
                         for unit in (32, 64):
                             if unit < bc:
-                                u = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, unit, 2, 2, nthreads, True, waves_per_eu=wpe)
-                                out.append(u.set_fuse_type(fuse))
+                                for ns in (1,) + (KV_SPLITS if with_splits else ()):
+                                    u = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, unit, 2, 2, nthreads, True, waves_per_eu=wpe, kv_splits=ns)
+                                    out.append(u.set_fuse_type(fuse))
                     if op == "attn" and fuse == "register" and with_splits and st_qk == st_v:
                         for ns in KV_SPLITS:   # long kv, few query rows: cut the kv range so every CU gets work
                             sp = AttnConfig(br, bc, dim_qk, dim_v, dim_qk, bc, st_qk, st_v, nthreads, True, waves_per_eu=wpe, kv_splits=ns)

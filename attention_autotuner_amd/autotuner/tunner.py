@@ -53,8 +53,9 @@ class _ForwardTunner(BaseTunner):
         flags = codegen.template_bools(mangled)
         if self.operation == "ret":                       # <..., DECAY>
             return not flags or flags[-1] == bool(self.decay)
-        if "flashattn_fwd_regfuse" in mangled and len(flags) == 4:     # <..., PIPE, CAUSAL, SPLIT, PERSIST>
-            return flags[1] == bool(self.causal)
+        if "flashattn_fwd_regfuse" in mangled and len(flags) == 5:     # <..., PIPE, CAUSAL, SPLIT, PERSIST, PAIR>
+            # the persistent and the paired variant are not launched from a build that spills (the wrapper asks the runtime)
+            return flags[1] == bool(self.causal) and not flags[3] and not flags[4]
         if "flashattn_fwd_smemfuse" in mangled and flags:              # <..., CAUSAL>
             return flags[-1] == bool(self.causal)
         return True

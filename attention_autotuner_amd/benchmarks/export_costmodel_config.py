@@ -12,7 +12,8 @@ The outer invocation builds the candidate libraries, starts itself under ``rocpr
 matches the counter rows to the candidates by dispatch order and writes a JSON list of
 
     {"config": {...}, "cost_model_config": [[Sq, Sk, dqk, dv], [Br, Bc, BlockK, D], [wave tile of the first
-     contraction], [wave tile of the second], B, H], "causal": bool, "cycles": int, "lds_bytes": int, "registers": int}
+     contraction], [wave tile of the second], B, H], "causal": bool, "cycles": int, "dispatches": int, "scratch_bytes": int,
+     "lds_bytes": int, "registers": int}
 
 in the tuple layout of the reference's exporter (wave tiles are (rows, columns, 16): the rows and
 columns one wave computes per step and the MFMA k depth).
@@ -37,13 +38,13 @@ XCDS = 8
 
 
 def candidates(op, dims, causal, limit, only_built=False):
-    """The tuner's candidates for the problem (unsplit ones: one kernel per launch); ``only_built``: those whose
+    """The tuner's candidates for the problem; ``only_built``: those whose
     library is already in the build directory (a machine without a compiler, or a process that must not start one)."""
     from ..autotuner import tunner
     b, h, sq, sk, dqk, dv = dims
     arrays = make_tensors(op, b, h, sq, sk, dqk, dv, "meta")
     t = getattr(tunner, TUNERS[op])(MI355X(), arrays, causal=causal)
-    cfgs = [c for c in t.get_tuned_configs() if t._fits_problem(c) and getattr(c, "kv_splits", 1) == 1]
+    cfgs = [c for c in t.get_tuned_configs() if t._fits_problem(c)]
     if only_built:
         cfgs = [c for c in cfgs if os.path.exists(codegen.library_path(c))]
     return cfgs[:limit] if limit else cfgs
@@ -61,6 +62,19 @@ def cost_model_tuple(cfg, dims):
     return [[sq, sk, dqk, dv], [cfg.Br, cfg.Bc, cfg.BlockKSmem, cfg.D], list(tile1), list(tile2), b, h]
 
 
+def dispatches_per_launch(cfg, dims, causal):
+    """Kernels one launch of ``cfg`` enqueues: a kv-splitting attention configuration runs its split kernel and the
+    merge (csrc/kernels/attention/regfuse/profile_code.py: ``split_applies``), everything else one kernel."""
+    ns = getattr(cfg, "kv_splits", 1)
+    return 2 if (cfg.operation == "attn" and ns > 1 and not causal and (dims[3] // cfg.Bc) % ns == 0) else 1
+
+
+def scratch_bytes(cfg):
+    """Largest per-lane scratch of any kernel in the configuration's library (the compiler's report), or None."""
+    usage = codegen.resource_usage(codegen.library_path(cfg))
+    return max((k.get("scratch_bytes", 0) for k in usage), default=0) if usage else None
+
+
 def run_candidates(op, dims, causal, limit, only_built=False):
     """Inner mode (under rocprofv3): launch every candidate library twice."""
     import ctypes
@@ -74,8 +88,10 @@ def run_candidates(op, dims, causal, limit, only_built=False):
         if not os.path.exists(path):
             continue
         lib = library.load(path, op)
+        need = int(lib.workspace_size(b, h, sq, sk))
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device="cuda")
         for _ in range(2):
-            rc = lib.kernel_entry_ex(*ptrs, b, h, sq, sk, *extra, ctypes.c_void_p(0), ctypes.c_size_t(0), stream)
+            rc = lib.kernel_entry_ex(*ptrs, b, h, sq, sk, *extra, ctypes.c_void_p(ws.data_ptr() if need else 0), ctypes.c_size_t(need), stream)
             if rc != 0:
                 raise RuntimeError(f"{cfg}: kernel_entry_ex returned {rc}")
         torch.cuda.synchronize()
@@ -118,15 +134,19 @@ def main(argv=None):
         with open(path) as f:
             rows += [r for r in csv.DictReader(f) if r["Counter_Name"] == "GRBM_GUI_ACTIVE" and "aat" in r["Kernel_Name"]]
     rows.sort(key=lambda r: int(r["Dispatch_Id"]))
-    # one kernel per launch for unsplit forward configurations: two dispatches per candidate, keep the second
-    if len(rows) != 2 * len(launched):
-        raise RuntimeError(f"{len(rows)} counted dispatches for {len(launched)} candidates")
+    # every candidate was launched twice (warm-up, counted): the cycles of a launch are those of its kernels together
     by_name = {str(c): c for c in cfgs}
-    records = []
-    for i, name in enumerate(launched):
+    per_launch = [dispatches_per_launch(by_name[name], args.dims, args.causal) for name in launched]
+    if len(rows) != 2 * sum(per_launch):
+        raise RuntimeError(f"{len(rows)} counted dispatches for {len(launched)} candidates ({sum(per_launch)} kernels per round)")
+    records, at = [], 0
+    for name, k in zip(launched, per_launch):
         cfg = by_name[name]
+        counted = rows[at + k:at + 2 * k]
+        at += 2 * k
         records.append({"config": cfg.to_dict(), "cost_model_config": cost_model_tuple(cfg, args.dims), "causal": bool(args.causal),
-                        "cycles": int(float(rows[2 * i + 1]["Counter_Value"]) / XCDS),
+                        "cycles": int(sum(float(r["Counter_Value"]) for r in counted) / XCDS), "dispatches": k,
+                        "scratch_bytes": scratch_bytes(cfg),
                         "lds_bytes": gfx950_space.forward_lds_bytes(cfg), "registers": gfx950_space.forward_reg_estimate(cfg)})
     out = args.out or f"{args.op}_{args.dims[4]}_{args.dims[5]}_costmodel.json"
     with open(out, "w") as f:

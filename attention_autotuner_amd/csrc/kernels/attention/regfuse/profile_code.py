@@ -30,6 +30,7 @@ using Traits = aat::AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_s
 constexpr int shared_mem = Traits::kSmemBytes;
 const auto kernel = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, sw_pipeline, false>;
 const auto kernel_causal = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, sw_pipeline, true>;
+const auto kernel_causal_paired = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, sw_pipeline, true, false, false, true>;
 const auto kernel_split = &aat::flashattn_fwd_regfuse<Kd, D, Br, Bc, Nthreads, num_stages_qk, num_stages_v, waves_per_eu, unit_rows, sw_pipeline, false, true>;
 constexpr int shared_mem_split = Traits::kSmemBytesSplit;
 
@@ -75,6 +76,30 @@ int resident_blocks() {{
   return blocks > 0 ? blocks : 0;
 }}
 
+// Whether `n` equal workgroups come out as whole rounds over the workgroups the chip holds at this configuration's
+// occupancy (registers: waves_per_eu waves per SIMD; the LDS may allow fewer, which this does not look at).
+bool pairs_fill_the_chip(int n) {{
+  static std::atomic<int> cus_of[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  int cus = cus_of[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {{
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = -1;
+    cus_of[dev].store(cus, std::memory_order_relaxed);
+  }}
+  if (cus <= 0) return false;
+  // a build of the paired kernel that keeps part of its working set in scratch memory (the second pass costs registers)
+  // loses more than the pairing gains: the one-row-block-per-workgroup kernel stands in
+  static const bool paired_spills = [] {{
+    hipFuncAttributes attr;
+    return hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kernel_causal_paired)) != hipSuccess || attr.localSizeBytes != 0;
+  }}();
+  if (paired_spills) return false;
+  const int per_cu = waves_per_eu * 4 * 64 / Nthreads > 0 ? waves_per_eu * 4 * 64 / Nthreads : 1;
+  const int resident = cus * per_cu;
+  return n % resident == 0 || n >= 8 * resident;
+}}
+
 size_t split_workspace_bytes(int B, int H, int Seq_q) {{
   return kv_splits > 1 ? (size_t)kv_splits * B * H * Seq_q * (D + 1) * sizeof(float) : 0;
 }}
@@ -111,7 +136,13 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, int B, int
   static const hipError_t lds_ok_causal = aat::allow_lds(kernel_causal, shared_mem);
   if (lds_ok != hipSuccess) return lds_ok;
   if (lds_ok_causal != hipSuccess) return lds_ok_causal;
-  (causal ? kernel_causal : kernel)<<<dim3(items), dim3(Nthreads), shared_mem, stream>>>(
+  // causal, an even number of row blocks per head: half the grid, every workgroup walks a long and a short row block --
+  // where those workgroups fill the chip a whole number of times (or many times over); a last round that is one third
+  // full costs more than the equal lengths and the shared K/V stream gain
+  const bool paired = causal && (Seq_q / Br) % 2 == 0 && pairs_fill_the_chip(items / 2);
+  static const hipError_t lds_ok_paired = aat::allow_lds(kernel_causal_paired, shared_mem);
+  if (lds_ok_paired != hipSuccess) return lds_ok_paired;
+  (paired ? kernel_causal_paired : causal ? kernel_causal : kernel)<<<dim3(paired ? items / 2 : items), dim3(Nthreads), shared_mem, stream>>>(
       reinterpret_cast<const aat::half_t*>(q), reinterpret_cast<const aat::half_t*>(k),
       reinterpret_cast<const aat::half_t*>(v), reinterpret_cast<aat::half_t*>(o), lse, H, Seq_k, Seq_q,
       softmax_scale, nullptr, nullptr, 0);

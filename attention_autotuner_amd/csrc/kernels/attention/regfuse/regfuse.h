@@ -53,12 +53,10 @@ struct AttnFwdRegfuse {
   static constexpr int kKBytes = Bc * Kd * 2, kVBytes = Bc * D * 2;
   static constexpr int kUnitK = 32 * Kd * 2, kUnitV = 32 * D * 2;   // bytes of one 32-row unit
   static constexpr int kOStride = D * 2 + 16;   // epilogue staging row stride (bytes)
-  static constexpr int kOStride32 = D * 4 + 16; // same, for the fp32 partial outputs of a kv split
   static constexpr int kMainBytes = NSK * kKBytes + NSV * kVBytes;
   static constexpr int kEpiBytes = Br * kOStride;
   static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
-  static constexpr int kEpiBytesSplit = Br * kOStride32;
-  static constexpr int kSmemBytesSplit = kMainBytes > kEpiBytesSplit ? kMainBytes : kEpiBytesSplit;
+  static constexpr int kSmemBytesSplit = kMainBytes;   // the partial outputs of a kv split are stored without staging
   // Persistent blocks (PERSIST) stage their output tiles where the copies of the next row block's first kv
   // tile do not land: behind the K/V buffers as far as the LDS budget of a block goes, then in the second K
   // and the second V buffer (the last kv tile of a row block has parity 1, the prefetch goes to parity 0).
@@ -131,14 +129,14 @@ template <bool CAUSAL, class F> AAT_DEV void run_tiles(F& tile, int n_full, int 
 // after them" leaves the stores in flight.  Needs two K and two V buffers and an even number of kv tiles (the
 // buffer parity must wrap); plain schedule, non-causal, unsplit.
 template <int Kd, int D, int Br, int Bc, int Nthreads, int NSK, int NSV, int WPE = 1, int BU = Bc, bool PIPE = false,
-          bool CAUSAL = false, bool SPLIT = false, bool PERSIST = false>
+          bool CAUSAL = false, bool SPLIT = false, bool PERSIST = false, bool PAIR = false>
 __global__ void __launch_bounds__(Nthreads) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k,
                       const half_t* __restrict__ v, half_t* __restrict__ o, float* __restrict__ lse,
                       int H, int seq_k, int seq_q, float softmax_scale, float* __restrict__ part_o = nullptr,
                       float* __restrict__ part_lse = nullptr, int n_items = 0) {
   using T = AttnFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV>;
-  constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, WM = T::WM;
+  constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, WM = T::WM, NW = T::NW;
   constexpr int PF = AAT_PF;                     // operand prefetch distance, in MFMA steps
   // Plain schedule: a kv tile of Bc rows (one copy, one barrier) is worked through in NU units of BU rows, each
   // scores -> softmax -> PV, so the live score tile is RT * BU / 32 accumulator blocks whatever Bc is.
@@ -149,6 +147,12 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
   // Where the output accumulators, the Q fragments and one unit's scores leave fewer than 40 of a wave's registers,
   // the operand addresses of all contraction steps are derived from one register each (tile_ops.h: XA).
   constexpr bool XA = WPE >= 2 && RT * (DT * 16 + KS * 4 + NTU * 16) + 40 > 512 / WPE;
+  // Causal, two 32-row groups per wave: wave w owns groups w and 2 NW - 1 - w of the block's 2 NW, an early and a late
+  // one.  In the tiles the diagonal crosses a group needs the kv rows up to its own, so with contiguous rows the last
+  // wave works through the whole diagonal region while the first is done after one unit and waits at every barrier;
+  // dealt out this way every wave has 2 NW + 1 group-units to do there.  A unit the late group sees and the early one
+  // does not runs the contractions for the late group alone.
+  constexpr bool ILV = CAUSAL && RT == 2 && !PIPE && NSK == 2 && NSV == 2;
   static_assert(!PIPE || T::kPipeOk, "the pipelined schedule needs 2+2 buffers and unit-aligned K copies");
   static_assert(!(SPLIT && CAUSAL), "kv splitting is for non-causal problems");
   using TP = typename T::template Persist<WPE>;
@@ -181,18 +185,30 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     for (int dt = 0; dt < DT; ++dt) vaddr[dt] = lds_addr(vbuf + voff[dt]);
   }
 
-  const float c2 = softmax_scale * kLog2e;
+  const float c2 = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, softmax_scale * kLog2e)));   // wave-uniform: a scalar register
   const int diag = seq_k - seq_q;               // kv index allowed for query i is <= i + diag
 
-  // One pass per row block: a single one unless PERSIST.
+  // One pass per row block: a single one unless PERSIST -- or PAIR (a variant of the causal kernel): then the grid is half
+  // the row blocks and block p of a head walks row block Tr-1-p and then row block p.  The two lengths add up to the same
+  // for every p, so every workgroup does the same amount of work whatever order the dispatcher hands them out in, and
+  // the workgroups of a head run side by side on one XCD and share its K/V stream in L2 (dealing single row blocks out
+  // longest-first over all heads of an XCD balances as well, but interleaves sixteen heads in every L2).
   bool prefetched = false;                      // Q fragments and kv tile 0 of this row block were requested by the previous pass
+  static_assert(!PAIR || (CAUSAL && !PERSIST && !SPLIT), "pairs of row blocks: the causal walk");
+  int pass = 0;
   for (int vb = blockIdx.x;; vb += gridDim.x) {
     const int tile = PERSIST ? xcd_remap(vb, n_items) : xcd_remap(vb, (int)gridDim.x);
     int bh = tile / Tr, rb = tile % Tr;
-    if constexpr (CAUSAL) {                       // long rows first, over all heads of the XCD
-      const TileId t = causal_tile(vb, (int)gridDim.x, Tr, true);
-      bh = t.bh;
-      rb = t.blk;
+    if constexpr (CAUSAL) {
+      if constexpr (PAIR) {
+        const int half = Tr / 2;
+        bh = tile / half;
+        rb = pass == 0 ? Tr - 1 - tile % half : tile % half;
+      } else {                                    // long rows first, over all heads of the XCD
+        const TileId t = causal_tile(vb, (int)gridDim.x, Tr, true);
+        bh = t.bh;
+        rb = t.blk;
+      }
     }
     const int q0 = rb * Br;
     int n_tiles = seq_k / Bc;
@@ -216,7 +232,10 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     const char* kg = reinterpret_cast<const char*>(k + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * Kd);
     const char* vg = reinterpret_cast<const char*>(v + ((size_t)bh * seq_k + (size_t)tile0 * Bc) * D);
 
-    if (!prefetched) load_q_frags<RT, KS, Kd>(qf, q + ((size_t)bh * seq_q + q0 + wave * WM + n) * Kd + 8 * h);
+    // first row of the wave's first 32-row group inside the block, and the distance to its second group
+    const int wrow0 = ILV ? 32 * wave : wave * WM;
+    const int group_rows = ILV ? 32 * (2 * NW - 1 - 2 * wave) : 32;
+    if (!prefetched) load_q_frags<RT, KS, Kd>(qf, q + ((size_t)bh * seq_q + q0 + wrow0 + n) * Kd + 8 * h, group_rows);
     // PERSIST: where the next row block of this block starts (tile numbers map to (head, row block) as above)
     const int vb_next = vb + (int)gridDim.x;
     const bool has_next = PERSIST && vb_next < n_items;
@@ -234,7 +253,7 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] = zero16();
     }
-    const int q_lim0 = q0 + wave * WM + n + diag;   // last kv index row n of row group 0 may see
+    const int q_lim0 = q0 + wrow0 + n + diag;       // last kv index row n of row group 0 may see
 
     if constexpr (!PIPE) {
       // ============================ plain schedule =================================================
@@ -242,6 +261,7 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
         kdma.issue(kg, kbuf, wave_base);
         if constexpr (NSV == 2) vdma.issue(vg, vbuf, wave_base);
       }
+      if (!prefetched) wait_vmcnt0_visible();        // the Q fragments are in (cdna4.h); tile 0 is waited for next anyway
       // `parity_tag` carries j & 1 as a compile-time value so that every LDS address of the tile is a
       // per-lane constant plus an immediate.
       auto kv_tile = [&](const int j, auto parity_tag, auto masked_tag) {
@@ -290,6 +310,44 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
         static_for<NU>([&](auto unit_tag) {
           constexpr int U = decltype(unit_tag)::value;
           const int kv0 = j * Bc + U * BU;           // first kv row of the unit
+          if constexpr (ILV) {
+            // One body for both row groups; in a unit the early group no longer sees (and the late one does) its
+            // MFMAs, its softmax step and its packing are branched around one by one.
+            bool on0 = true, on1 = true;
+            if constexpr (MASKED) {
+              const int last_early = q0 + wrow0 + 31 + diag;            // last kv row the early group sees
+              on0 = kv0 <= last_early;
+              on1 = kv0 <= last_early + group_rows;
+            }
+            if (on1) {
+              f16v sacc[RT][NTU];
+              AAT_SETPRIO(2);
+              qk_gemm_steps<RT, NTU, KS, NCK, PF, false, XA, MASKED && XA>(sacc, qf, kaddr, PAR * T::kKBytes + U * NTU * T::kUnitK, [](int) {}, on0);
+              AAT_SETPRIO(0);
+#pragma unroll
+              for (int rt = 0; rt < RT; ++rt) {
+                if (rt != 0 || on0 || !(MASKED && XA)) {
+                  const int q_lim = q_lim0 + rt * group_rows;
+                  // only the unit the group's own diagonal runs through has anything to mask (wave-uniform)
+                  const bool crosses = MASKED && kv0 + BU - 1 > q0 + wrow0 + rt * group_rows + diag;
+                  if (crosses) causal_mask<NTU>(sacc[rt], kv0, q_lim, h);
+                  const float mc = lazy_max_step<NTU, DT>(sacc[rt], m_run[rt], l_run[rt], oacc[rt], c2);
+                  exp_tile<NTU, XA>(sacc[rt], c2, mc);
+                  if (crosses) zero_masked<NTU>(sacc[rt], kv0, q_lim, h);
+                }
+              }
+              h8 pf[RT][NTU][2];
+              AAT_SETPRIO(2);
+              pv_gemm_steps<RT, NTU, DT, NCV, PF, false, XA, MASKED && XA>(oacc, pf, vaddr, PAR * T::kVBytes + U * NTU * T::kUnitV, [&](int g) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                  if (rt != 0 || on0 || !(MASKED && XA)) pack_p_group<NTU, XA>(pf[rt], sacc[rt], g, l_run[rt]);
+                }
+              }, on0);
+              AAT_SETPRIO(0);
+            }
+            return;
+          }
           bool wave_sees = true;
           if constexpr (MASKED) wave_sees = kv0 <= q0 + wave * WM + WM - 1 + diag;
 
@@ -430,7 +488,7 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     for (int rt = 0; rt < RT; ++rt) {
       const float l_tot = pair_sum(l_run[rt]);
       inv[rt] = l_tot > 0.f ? fast_rcp(l_tot) : 0.f;
-      const size_t row = (size_t)bh * seq_q + q0 + wave * WM + rt * 32 + n;
+      const size_t row = (size_t)bh * seq_q + q0 + wrow0 + rt * group_rows + n;
       const float row_lse = l_tot > 0.f ? m_run[rt] * softmax_scale + __logf(l_tot) : -INFINITY;
       if constexpr (SPLIT) {
         if (h == 0) part_lse[(size_t)blockIdx.y * gridDim.x * Br + row] = row_lse;   // gridDim.x * Br = B*H*S_q
@@ -440,16 +498,22 @@ flashattn_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k
     }
     if constexpr (SPLIT) {
       const size_t rows_total = (size_t)gridDim.x * Br;
-      store_o_tile<RT, DT, D, T::kOStride32, float>(
-          oacc, inv, smem + wave * WM * T::kOStride32,
-          part_o + ((size_t)blockIdx.y * rows_total + (size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+      store_o_rows_f32<RT, DT, D>(oacc, inv, part_o + ((size_t)blockIdx.y * rows_total + (size_t)bh * seq_q + q0 + wave * WM) * D, lane);
     } else if constexpr (PERSIST) {
       store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + TP::stage_offset(wave),
                                            o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
     } else {
       // transposed through LDS for 16-byte coalesced stores
       store_o_tile<RT, DT, D, T::kOStride>(oacc, inv, smem + wave * WM * T::kOStride,
-                                           o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+                                           o + ((size_t)bh * seq_q + q0 + wrow0) * D, lane, group_rows);
+    }
+    if constexpr (PAIR) {
+      if (pass == 0) {
+        pass = 1;
+        vb -= (int)gridDim.x;                      // the same workgroup id again
+        block_sync();                              // every wave has read its output tile out of the staging area
+        continue;
+      }
     }
     if (!has_next) break;
     prefetched = true;

@@ -63,6 +63,12 @@ template <int N> AAT_DEV void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 AAT_DEV void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// vmcnt(0) as an instruction the compiler can see.  Its own bookkeeping of outstanding loads does not read the waits
+// written in asm: fragments loaded ahead of a loop stay "possibly in flight" at the loop header for good, and it guards
+// their first use in the loop body with counted vmcnt waits on every iteration -- which, in hardware, also wait for the
+// LDS-DMA copies of the next tile issued a moment earlier (vmcnt(0) by the last fragment: no overlap left).  One visible
+// wait between those loads and the loop settles the books.
+AAT_DEV void wait_vmcnt0_visible() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0), expcnt and lgkmcnt untouched
 // Workgroup barrier that makes this thread's finished LDS traffic (ds ops and, when the caller has
 // already waited on vmcnt, LDS-DMA writes) visible to the other waves of the block.
 AAT_DEV void block_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }

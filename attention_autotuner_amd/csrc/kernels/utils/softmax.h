@@ -29,15 +29,16 @@ template <int NT> AAT_DEV float lane_max(const f16v (&s)[NT]) {
 }
 
 // Set S^T entries above the causal diagonal to -inf.  kv_base = first kv index of score tile 0,
-// q_lim = last kv index this lane's query row may see.
+// q_lim = last kv index this lane's query row may see.  Register v of tile t holds kv index
+// kv_base + 32 t + 4 h + (8 (v / 4) + v % 4): the lane-dependent part goes into one per-lane limit and every entry is
+// then a comparison of that limit with a literal and a select -- no kv index per entry in a register, no branch.
+AAT_DEV int causal_lane_limit(int kv_base, int q_lim, int h) { return q_lim - kv_base - 4 * h; }
 template <int NT> AAT_DEV void causal_mask(f16v (&s)[NT], int kv_base, int q_lim, int h) {
+  const int lim = causal_lane_limit(kv_base, q_lim, h);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int kv = kv_base + 32 * t + c_row(v, h);
-      if (kv > q_lim) s[t][v] = -INFINITY;
-    }
+    for (int v = 0; v < 16; ++v) s[t][v] = (32 * t + c_row(v, 0) > lim) ? -INFINITY : s[t][v];
   }
 }
 
@@ -45,13 +46,11 @@ template <int NT> AAT_DEV void causal_mask(f16v (&s)[NT], int kv_base, int q_lim
 // score is already 0 for any positive scale; this pass makes the result exact for scale 0 as well,
 // where -inf * 0 would otherwise leave a NaN.
 template <int NT> AAT_DEV void zero_masked(f16v (&p)[NT], int kv_base, int q_lim, int h) {
+  const int lim = causal_lane_limit(kv_base, q_lim, h);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int kv = kv_base + 32 * t + c_row(v, h);
-      if (kv > q_lim) p[t][v] = 0.f;
-    }
+    for (int v = 0; v < 16; ++v) p[t][v] = (32 * t + c_row(v, 0) > lim) ? 0.f : p[t][v];
   }
 }
 

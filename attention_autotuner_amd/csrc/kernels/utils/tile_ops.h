@@ -9,13 +9,14 @@ namespace aat {
 
 // Q rows of this wave as MFMA B operands, straight from global memory.
 // qrow points at element [first row of the wave + n][8*h] of a row-major [*, Kd] matrix.
+// group_rows: rows from one 32-row group of the wave to the next (32: the wave's rows are contiguous).
 template <int RT, int KS, int Kd>
-AAT_DEV void load_q_frags(h8 (&qf)[RT][KS], const half_t* qrow) {
+AAT_DEV void load_q_frags(h8 (&qf)[RT][KS], const half_t* qrow, int group_rows = 32) {
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      qf[rt][ks] = *reinterpret_cast<const h8*>(qrow + (size_t)rt * 32 * Kd + 16 * ks);
+      qf[rt][ks] = *reinterpret_cast<const h8*>(qrow + (size_t)rt * group_rows * Kd + 16 * ks);
 }
 
 // The same loads issued behind the compiler's back, into registers that already hold fragments: for a
@@ -168,9 +169,14 @@ AAT_DEV void mfma_settle(f16v& c) { asm volatile("s_nop 15\n\ts_nop 7" : "+v"(c)
 // VACC: accumulate in vector registers through hand-written MFMAs (see mfma_32x32x16_vacc).
 // XA: only kaddr[0] is used; step ks reads at kaddr[0] ^ (ks % 8) << 5 (the Rows16 swizzle XORs the chunk index
 // 2 ks + h with row bits, so the steps' addresses differ by exactly that).
-template <int RT, int NT, int KS, int NCK, int PF, bool VACC = false, bool XA = false, class Side>
+// GATE0: the MFMAs of row group 0 are issued only when `group0_on` (wave-uniform) is set -- a causal wave whose early
+// group no longer sees the unit while its late group does.  One code path with a branch around single instructions
+// rather than a second instantiation for the late group alone: with two bodies the allocator no longer keeps the
+// accumulator tuples in the same registers on both and reconciles them through scratch memory.
+template <int RT, int NT, int KS, int NCK, int PF, bool VACC = false, bool XA = false, bool GATE0 = false, class Side>
 AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const uint32_t (&kaddr)[KS],
-                           int buf_off, Side&& side) {
+                           int buf_off, Side&& side, bool group0_on = true) {
+  static_assert(!GATE0 || (XA && RT == 2), "the gate is built into the in-place operand ring of two row groups");
   static_assert(!(XA && VACC), "xor addressing is for kernels that fit the unified register file");
   constexpr int S = NT * KS;
   constexpr int kTileStride = 32 * NCK * 16;
@@ -206,7 +212,9 @@ AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const u
       // has read its operands long before an LDS read issued after it returns), so PF slots are all there is.
       lds_wait_younger<(step + PF - 1 < S) ? PF - 1 : S - 1 - step>(ring[step % PF]);
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) sacc[rt][step / KS] = mfma_32x32x16(ring[step % PF], qf[rt][step % KS], sacc[rt][step / KS]);
+      for (int rt = 0; rt < RT; ++rt) {
+        if (!GATE0 || rt != 0 || group0_on) sacc[rt][step / KS] = mfma_32x32x16(ring[step % PF], qf[rt][step % KS], sacc[rt][step / KS]);
+      }
       if constexpr (step + PF < S) ring[step % PF] = read(step + PF);
     } else {
       h8 cur = ring[step % PF];
@@ -279,9 +287,11 @@ AAT_DEV void pv_gemm_steps_hl(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const u
 // BLIND: as in pv_gemm_steps_hl.
 // XA: only vaddr[0] is used; d-tile dt reads at vaddr[0] ^ (dt % 4) << 6 (the Rows4 swizzle XORs the chunk-group
 // bits with row bits); implies hand-issued reads with counted waits.
-template <int RT, int NT, int DT, int NCV, int PF, bool BLIND = false, bool XA = false, class Pack>
+// GATE0, group0_on: as in qk_gemm_steps.
+template <int RT, int NT, int DT, int NCV, int PF, bool BLIND = false, bool XA = false, bool GATE0 = false, class Pack>
 AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint32_t (&vaddr)[DT], int buf_off,
-                           Pack&& pack) {
+                           Pack&& pack, bool group0_on = true) {
+  static_assert(!GATE0 || (XA && RT == 2), "the gate is built into the in-place operand ring of two row groups");
   constexpr int G = NT * 2;              // groups of 16 kv rows
   constexpr int S = G * DT;
   constexpr int kRow16 = 16 * NCV * 16, kRow8 = 8 * NCV * 16;
@@ -322,7 +332,9 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
       lds_wait_younger<2 * ((step + PF - 1 < S) ? PF - 1 : S - 1 - step)>(lo[step % PF], hi[step % PF]);
       const h8 vf = cat_h4(lo[step % PF], hi[step % PF]);
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
+      for (int rt = 0; rt < RT; ++rt) {
+        if (!GATE0 || rt != 0 || group0_on) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
+      }
       if constexpr (step + PF < S) read(step + PF, step % PF);
     } else {
       h4 clo = lo[step % PF], chi = hi[step % PF];
@@ -340,9 +352,10 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
 // Epilogue: scale the wave's O^T accumulators per row, convert (fp16 with RNE, or fp32 as is),
 // transpose through a wave-private LDS staging area and store rows with 16-byte coalesced writes.
 // ostage: wave-private LDS, WM rows of O_STRIDE bytes.  og: global pointer to the wave's first output row.
+// group_rows: rows in global memory from one 32-row group of the wave to the next (32: contiguous).
 template <int RT, int DT, int D, int O_STRIDE, class OutT = half_t>
 AAT_DEV void store_o_tile(const f16v (&oacc)[RT][DT], const float (&row_scale)[RT], char* ostage, OutT* og,
-                          int lane) {
+                          int lane, int group_rows = 32) {
   constexpr int kElem = (int)sizeof(OutT);
   constexpr int kChunksPerRow = D * kElem / 16, WM = RT * 32;
   const int n = lane & 31, h = lane >> 5;
@@ -383,7 +396,34 @@ AAT_DEV void store_o_tile(const f16v (&oacc)[RT][DT], const float (&row_scale)[R
     const int idx = t * 64 + lane;
     const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
     const u4v val = *reinterpret_cast<const u4v*>(ostage + row * O_STRIDE + c * 16);
-    *reinterpret_cast<u4v*>(reinterpret_cast<char*>(og) + ((size_t)row * kChunksPerRow + c) * 16) = val;
+    const size_t grow = (size_t)(row / 32) * group_rows + row % 32;
+    *reinterpret_cast<u4v*>(reinterpret_cast<char*>(og) + (grow * kChunksPerRow + c) * 16) = val;
+  }
+}
+
+// fp32 output straight from the accumulators, no staging: a lane holds four consecutive columns of one row per
+// accumulator group, so it stores 16-byte pieces (the two lanes of a row write neighbouring pieces).  Slower per tile
+// than the staged, row-contiguous stores (about twice), which does not matter for the once-per-block partial output of a
+// kv split, and it needs no LDS: a split block then occupies what its K/V buffers take and nothing more.
+template <int RT, int DT, int D>
+AAT_DEV void store_o_rows_f32(const f16v (&oacc)[RT][DT], const float (&row_scale)[RT], float* og, int lane) {
+  const int n = lane & 31, h = lane >> 5;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const float sc = row_scale[rt];
+    float* row = og + (size_t)(rt * 32 + n) * D + 4 * h;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      f16v blk = oacc[rt][dt];
+      if constexpr (RT * DT * 16 >= 256) asm volatile("" : "+a"(blk));
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f4v w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = blk[4 * g + e] * sc;
+        *reinterpret_cast<f4v*>(row + 32 * dt + 8 * g) = w;
+      }
+    }
   }
 }
 

@@ -21,10 +21,18 @@ RUNS = {                                                  # file -> (shape, caus
     "attn_b4h32q2048k2048_c0_128_128_later.txt": ((4, 32, 2048, 2048), False),
     "attn_b4h32q2048k2048_c1_128_128_later.txt": ((4, 32, 2048, 2048), True),
 }
+# ... and again with the candidates that work a kv tile through in units (two 32-row groups per wave, Br up to 512) and,
+# for the long-kv problem, the kv-splitting candidates: new kernels, new winners
+RUNS_WITH_UNITS = {
+    "attn_b4h32q2048k2048_c0_128_128_units.txt": ((4, 32, 2048, 2048), False),
+    "attn_b4h32q2048k2048_c1_128_128_units.txt": ((4, 32, 2048, 2048), True),
+    "attn_b1h32q256k16384_c0_128_128_units.txt": ((1, 32, 256, 16384), False),
+}
+EXPORTS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "costmodel_export")
 
 
 def _samples(name):
-    shape, causal = RUNS[name]
+    shape, causal = {**RUNS, **RUNS_WITH_UNITS}[name]
     return costmodel.samples_from_tuning_log(os.path.join(LOGS, name), "attn", 128, 128, shape, causal)
 
 
@@ -70,9 +78,32 @@ def test_model_fitted_on_one_run_keeps_the_winner_of_the_others():
         assert model.rank_of_best(runs) < len(keep), name                  # the measured winner survives the cut
         assert times[keep].min() == times.min(), name
         assert np.corrcoef(pred, times)[0, 1] > 0.8, name                  # and the model follows the measurements overall
-    # the model shipped next to the tuning cache is this fit
+
+
+def test_shipped_model_is_the_fit_on_exported_cycles_and_keeps_every_recorded_winner():
+    """The model next to the tuning cache is fitted on the cycle counts of benchmarks/export_costmodel_config.py (three
+    problems: the headline, its causal variant, the long-kv shape with its kv-splitting candidates; candidates the
+    compiler reports as spilling left out, as in the tuning loop).  Ranking by counted cycles must keep the measured
+    winner of every recorded tuning run -- timed in milliseconds on other boxes, six of them with kernels older than the
+    export."""
+    exports = sorted(os.path.join(EXPORTS, f) for f in os.listdir(EXPORTS) if f.endswith(".json"))
+    assert len(exports) == 3
+    samples = [s for path in exports for s in costmodel.samples_from_export(path, max_scratch_bytes=64)]
+    assert len(samples) > 700 and any(getattr(s[0], "kv_splits", 1) > 1 for s in samples) and any(s[2] for s in samples)
+    model = costmodel.CostModel(unit="cycles").fit(samples)
     shipped = costmodel.CostModel.load(os.path.join(AttnTunner(MI355X(), _meta(4, 32, 2048)).cache_path, "costmodel_attn.json"))
     np.testing.assert_allclose(shipped.weights, model.weights, rtol=1e-6)
+    assert shipped.unit == "cycles"
+    for name in list(RUNS) + list(RUNS_WITH_UNITS):
+        runs = _samples(name)
+        times = np.array([s[3] for s in runs])
+        pred = np.array([shipped.predict(*s[:3]) for s in runs])
+        keep = np.argsort(pred)[:max(AttnTunner.keep_min, int(len(runs) * AttnTunner.keep_fraction + 0.999))]
+        assert times[keep].min() == times.min(), (name, shipped.rank_of_best(runs))
+        assert np.corrcoef(pred, times)[0, 1] > 0.8, name
+    # the spilling candidates are in the export (ten times the cycles of the rest) and would be all a fit sees
+    everything = [s for path in exports for s in costmodel.samples_from_export(path)]
+    assert len(everything) > len(samples) + 100
 
 
 def _meta(b, h, s, d=128):
