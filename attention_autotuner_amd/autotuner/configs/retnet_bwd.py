@@ -6,7 +6,9 @@ class RetBwdConfig(BaseConfig):
 
     On MI355X the gradient is three passes (dV, dK, dQ) of one chained-contraction kernel: ``Br`` is the
     number of block-resident rows and ``Bc`` the number of streamed rows per step of every pass;
-    ``num_stages_qk`` / ``num_stages_dv`` are the LDS buffer counts of the two streams.  The ``mmawarpsN*``
+    ``num_stages_qk`` / ``num_stages_dv`` are the LDS buffer counts of the two streams of the dV pass, and
+    ``num_stages_ds`` / ``num_stages_dq`` the same counts for the passes that contract over d_v first (dQ, and dK
+    where it is a chained pass): their streamed tiles are d_v wide.  The ``mmawarpsN*``
     fields (how the reference splits its warps along the N side of each contraction) are carried for
     file compatibility; every wave here owns whole rows.
 

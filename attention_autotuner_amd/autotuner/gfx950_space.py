@@ -242,14 +242,16 @@ def backward_dv_cols(cfg):
 
 
 def _backward_passes(cfg):
-    """(first-contraction width, output columns per block) of the dV, dK and dQ passes."""
-    return ((cfg.Kd, backward_dv_cols(cfg)), (cfg.D, cfg.Kd), (cfg.D, cfg.Kd))
+    """(first-contraction width, output columns per block, buffers of the first stream, of the second) of the dV, dK
+    and dQ passes."""
+    return ((cfg.Kd, backward_dv_cols(cfg), cfg.num_stages_qk, cfg.num_stages_dv),
+            (cfg.D, cfg.Kd, cfg.num_stages_ds, cfg.num_stages_dq), (cfg.D, cfg.Kd, cfg.num_stages_ds, cfg.num_stages_dq))
 
 
 def backward_lds_bytes(cfg):
     worst = 0
-    for kx, dzb in _backward_passes(cfg):
-        main = cfg.num_stages_qk * (cfg.Bc * kx * 2 + cfg.Br * cfg.Bc * 2) + cfg.num_stages_dv * cfg.Bc * dzb * 2
+    for kx, dzb, sy, sz in _backward_passes(cfg):
+        main = sy * (cfg.Bc * kx * 2 + cfg.Br * cfg.Bc * 2) + sz * cfg.Bc * dzb * 2
         worst = max(worst, main, cfg.Br * (dzb * 2 + 16))
     return worst
 
@@ -258,7 +260,7 @@ def backward_reg_estimate(cfg):
     """(vector registers, accumulation registers) of the hungriest pass."""
     rt = cfg.Br // _waves(cfg) // MFMA_M
     vec = acc = 0
-    for kx, dzb in _backward_passes(cfg):
+    for kx, dzb, _, _ in _backward_passes(cfg):
         vec = max(vec, rt * (kx // 16) * 4 + rt * (cfg.Bc // 32) * 24 + 64)
         acc = max(acc, rt * (dzb // 32) * 16)
     return vec, acc
@@ -275,7 +277,7 @@ def backward_valid(cfg, arch):
         if ds_rows not in DS_ROWS or cfg.Br % DS_TILE or cfg.waves_per_eu != 1:
             return False
         # the row pass stages a dS tile behind its stream buffers; the dK kernel holds two (Q tile, dS tile) pairs
-        row_lds = cfg.num_stages_qk * (cfg.Bc * cfg.D * 2 + cfg.Br * cfg.Bc * 2) + cfg.num_stages_dv * cfg.Bc * cfg.Kd * 2
+        row_lds = cfg.num_stages_ds * (cfg.Bc * cfg.D * 2 + cfg.Br * cfg.Bc * 2) + cfg.num_stages_dq * cfg.Bc * cfg.Kd * 2
         if row_lds + cfg.Br * (cfg.Bc * 2 + 16) > arch.smem_cap:
             return False
         if 2 * DS_TILE * (cfg.Kd + ds_rows) * 2 > arch.smem_cap:
@@ -284,9 +286,12 @@ def backward_valid(cfg, arch):
         return False
     if nw > 4 * cfg.waves_per_eu:
         return False
-    if cfg.num_stages_qk not in (1, 2, 3) or cfg.num_stages_dv not in (1, 2):
-        return False
-    if cfg.num_stages_qk == 3 and cfg.num_stages_dv != 2:      # the three-buffer schedule prefetches Z one tile ahead
+    for sy, sz in ((cfg.num_stages_qk, cfg.num_stages_dv), (cfg.num_stages_ds, cfg.num_stages_dq)):
+        if sy not in (1, 2, 3) or sz not in (1, 2):
+            return False
+        if sy == 3 and sz != 2:      # the three-buffer schedule prefetches Z one tile ahead
+            return False
+    if cfg.num_stages_mask != cfg.num_stages_qk:               # the mask tile travels with the first stream
         return False
     nt = cfg.Nthreads
     for cols in (cfg.Kd, cfg.D, backward_dv_cols(cfg), cfg.Br):   # every streamed tile must split evenly over the threads
@@ -302,19 +307,24 @@ def backward_valid(cfg, arch):
     return vec + acc <= arch.register_per_thread // cfg.waves_per_eu
 
 
+BWD_STAGES = ((1, 1), (2, 2), (2, 1), (3, 2))       # (buffers of the first stream, of the second) of a pass
+
+
 def backward_candidates(br, bc, dim_qk, dim_v):
+    """Every combination of buffer counts for the dV pass and for the d_v-contracting passes: where d_v differs from
+    d_qk the two kinds of pass stream tiles of different widths and the best counts differ with them."""
     out = []
     for nthreads in (128, 256, 512):
-        for st_y, st_z in ((1, 1), (2, 2), (2, 1), (3, 2)):
-            for wpe in (1, 2):
-                n = nthreads // WAVE
-                out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, BlockKSmem=dim_qk,
-                                        num_stages_qk=st_y, num_stages_mask=st_y, num_stages_dv=st_z, waves_per_eu=wpe))
-                if wpe == 1:          # ... and with dS stored by the dQ pass for a dK kernel of its own (needs the workspace)
-                    for ds_rows in DS_ROWS:
-                        out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, BlockKSmem=dim_qk,
-                                                num_stages_qk=st_y, num_stages_mask=st_y, num_stages_dv=st_z,
-                                                waves_per_eu=wpe, ds_rows=ds_rows))
+        for st_y, st_z in BWD_STAGES:
+            for st_ds, st_dq in (BWD_STAGES if dim_qk != dim_v else ((st_y, st_z),)):
+                for wpe in (1, 2):
+                    n = nthreads // WAVE
+                    kw = dict(BlockKSmem=dim_qk, num_stages_qk=st_y, num_stages_mask=st_y, num_stages_dv=st_z,
+                              num_stages_ds=st_ds, num_stages_dq=st_dq, waves_per_eu=wpe)
+                    out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, **kw))
+                    if wpe == 1:          # ... and with dS stored by the dQ pass for a dK kernel of its own (needs the workspace)
+                        for ds_rows in DS_ROWS:
+                            out.append(RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nthreads, True, ds_rows=ds_rows, **kw))
     return out
 
 
@@ -328,7 +338,7 @@ def default_backward_config(dim_qk, dim_v, arch, seq_q=None, seq_k=None):
             continue
         n = nt // WAVE
         cfg = RetBwdConfig(br, bc, dim_qk, dim_v, n, n, n, n, nt, True, BlockKSmem=dim_qk, num_stages_qk=sy,
-                           num_stages_mask=sy, num_stages_dv=sz, waves_per_eu=wpe)
+                           num_stages_mask=sy, num_stages_dv=sz, num_stages_ds=sy, num_stages_dq=sz, waves_per_eu=wpe)
         if backward_valid(cfg, arch):
             return cfg
     raise NoValidConfigError(f"no default ret_bwd configuration fits dim_qk={dim_qk} dim_v={dim_v} seq=({seq_q},{seq_k})")

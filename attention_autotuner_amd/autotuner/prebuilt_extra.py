@@ -67,7 +67,7 @@ RET_BWD_STORED_DS_STAGED = [(256, 512, 128, 32, 256, 128, (2, 2)), (256, 512, 12
 def ret_bwd_stored_ds_config(dqk, dv, br, bc, nt, ds_rows, stages=(1, 1)):
     n = nt // 64
     return RetBwdConfig(br, bc, dqk, dv, n, n, n, n, nt, True, BlockKSmem=dqk, num_stages_qk=stages[0], num_stages_mask=stages[0],
-                        num_stages_dv=stages[1], waves_per_eu=1, ds_rows=ds_rows)
+                        num_stages_dv=stages[1], num_stages_ds=stages[0], num_stages_dq=stages[1], waves_per_eu=1, ds_rows=ds_rows)
 
 
 def parity_configs(arch=None):

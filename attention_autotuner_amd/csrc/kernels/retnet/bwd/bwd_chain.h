@@ -28,6 +28,7 @@
 #pragma once
 #include <type_traits>
 
+#include "../../utils/acc_file.h"
 #include "../../utils/cdna4.h"
 #include "../../utils/mask_extents.h"
 #include "../../utils/retention.h"
@@ -91,9 +92,15 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
               int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr,
               const int* __restrict__ extents = nullptr, half_t* __restrict__ ds_out = nullptr) {
   static_assert(!DS_OUT || PASS == BwdPass::Row, "dS is written by the row pass");
-  if constexpr (DECAY) causal = 1;
   using T = RetBwdChain<KX, DZ, DZB, BX, BY, Nthreads, NSY, NSZ, PASS>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCY = T::NCY, NCZ = T::NCZ, NCM = T::NCM, WM = T::WM;
+  // An output tile that fills the accumulation file (one wave per SIMD, 32 rows x 512 columns: the dV pass at d_v 512)
+  // lives there by number, outside the compiler's allocation (utils/acc_file.h): with the tile as a C++ value the
+  // variants with more than one buffer per stream -- one loop body per ring slot -- come out with the sixteen tuples
+  // placed differently from body to body and hundreds of bytes of scratch traffic per tile to reconcile them.
+  constexpr bool kNumbered = WPE == 1 && RT * DT * 16 == 256;
+  if constexpr (kNumbered) acc_claim_all();
+  if constexpr (DECAY) causal = 1;
   constexpr int PF = AAT_PF;
   constexpr bool COL = PASS == BwdPass::Col;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -186,11 +193,15 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   }
   const float* rg = r + (size_t)bh * seq_q;       // COL pass: r of the streamed query rows
 
-  f16v acc[RT][DT];
+  f16v acc[RT][DT];                               // unused when the tile lives in numbered registers
+  if constexpr (kNumbered) {
+    acc_zero<0, 256>();
+  } else {
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = zero16();
+      for (int dt = 0; dt < DT; ++dt) acc[rt][dt] = zero16();
+  }
 
   // Streamed tiles travel through rings of NSY (Y + mask) and NSZ (Z) LDS buffers; `st` is a ring slot.
   // Step j of the walk (j_begin <= j < j_end) works on streamed tile tile_of(j).  A row pass walks its kv tiles
@@ -250,8 +261,10 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
       // copies four of them back in front of every MFMA.
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
+        if constexpr (!kNumbered) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(acc[rt][dt]));
+          for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(acc[rt][dt]));
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(xf[rt][ks]));
       }
@@ -368,19 +381,37 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
     static_assert(!DS_OUT || kStores <= 8, "reads of the staging area in flight");
     char* const stage = smem + T::kMainBytes + wave * WM * T::kDsStride;
     f4v staged[kStores];
+    // The two lanes of a row hold alternate 8-byte pieces of it (kv 8g + 4h .. + 3).  Written as they are, the 32 rows
+    // of an instruction land 36 banks apart and collide four at a time.  The lanes first trade pieces (one
+    // v_permlane32_swap per register: the lower lane gives its piece of group 2k+1 for the upper lane's piece of
+    // group 2k), so each holds 16 contiguous bytes, kv 16k + 8h .. + 7, and writes them with one conflict-free
+    // 16-byte instruction: half the LDS writes, no conflicts, two swaps per write.
     const auto ds_stage = [&]() {
-      const uint32_t st_w = lds_addr(stage + n * T::kDsStride + 8 * h);
+      const uint32_t st_w = lds_addr(stage + n * T::kDsStride + 16 * h);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const h2 a = pack_rne(tacc[rt][t][4 * g], tacc[rt][t][4 * g + 1]);
-            const h2 b = pack_rne(tacc[rt][t][4 * g + 2], tacc[rt][t][4 * g + 3]);
-            h4 w;
-            w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
-            asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(st_w), "v"(w), "i"(rt * 32 * T::kDsStride + (32 * t + 8 * g) * 2));
+          for (int k2 = 0; k2 < 2; ++k2) {
+            uint32_t lo[2], hi[2];                       // the pieces of groups 2k and 2k+1, two halfs per register
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+              const h2 a = pack_rne(tacc[rt][t][8 * k2 + 2 * i], tacc[rt][t][8 * k2 + 2 * i + 1]);
+              const h2 b = pack_rne(tacc[rt][t][8 * k2 + 4 + 2 * i], tacc[rt][t][8 * k2 + 4 + 2 * i + 1]);
+              __builtin_memcpy(&lo[i], &a, 4);
+              __builtin_memcpy(&hi[i], &b, 4);
+            }
+            u4v w;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+              // result[0]: {lower lanes keep lo, upper lanes get the lower lanes' hi}; result[1]: {lower lanes get the
+              // upper lanes' lo, upper lanes keep hi}
+              const u2v sw = __builtin_amdgcn_permlane32_swap(lo[i], hi[i], false, false);
+              w[i] = sw[0];
+              w[2 + i] = sw[1];
+            }
+            asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(st_w), "v"(w), "i"(rt * 32 * T::kDsStride + (32 * t + 16 * k2) * 2));
           }
     };
     const auto ds_fetch = [&]() {
@@ -416,11 +447,13 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
       }
     };
     h8 ef[RT][NT][2];
-    pv_gemm_steps<RT, NT, DT, NCZ, PF, WPE == 1>(acc, ef, zaddr, zoff, [&](int g) {
+    const auto pack_e = [&](int g) {
       ride_along(g);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) pack_group<NT>(ef[rt], tacc[rt], g);
-    });
+    };
+    if constexpr (kNumbered) pv_gemm_steps_numbered<RT, NT, DT, NCZ, PF, 0>(ef, zaddr, zoff, pack_e, [](int) {});
+    else pv_gemm_steps<RT, NT, DT, NCZ, PF, WPE == 1>(acc, ef, zaddr, zoff, pack_e);
     if constexpr (COL) {
 #pragma unroll
       for (int i = 0; i < NT * 4; ++i) rv[i] = rv_next[i];
@@ -435,28 +468,28 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
     });
   }
 
+  if constexpr (kNumbered) acc_settle();
   wait_vmcnt<0>();
   block_sync();
-  float one[RT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) one[rt] = 1.f;
   // the staging rows are DZB wide; the global rows are DZ wide
   {
     char* const ostage = smem + wave * WM * T::kOStride;
     half_t* og = out + ((size_t)bh * seq_x + x0 + wave * WM) * DZ + dz0;
     constexpr int kChunksPerRow = DZB / 8;
+    static_for<RT * DT>([&](auto i_tag) {
+      constexpr int rt = decltype(i_tag)::value / DT, dt = decltype(i_tag)::value % DT;
+      f16v blk;
+      if constexpr (kNumbered) blk = acc_read16<16 * (rt * DT + dt)>();
+      else blk = acc[rt][dt];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const h2 a = pack_rne(acc[rt][dt][4 * g] * one[rt], acc[rt][dt][4 * g + 1]);
-          const h2 b = pack_rne(acc[rt][dt][4 * g + 2], acc[rt][dt][4 * g + 3]);
-          h4 w;
-          w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
-          *reinterpret_cast<h4*>(ostage + (rt * 32 + n) * T::kOStride + (32 * dt + 8 * g + 4 * h) * 2) = w;
-        }
+      for (int g = 0; g < 4; ++g) {
+        const h2 a = pack_rne(blk[4 * g], blk[4 * g + 1]);
+        const h2 b = pack_rne(blk[4 * g + 2], blk[4 * g + 3]);
+        h4 w;
+        w[0] = a[0]; w[1] = a[1]; w[2] = b[0]; w[3] = b[1];
+        *reinterpret_cast<h4*>(ostage + (rt * 32 + n) * T::kOStride + (32 * dt + 8 * g + 4 * h) * 2) = w;
+      }
+    });
     wait_lgkm0();
     constexpr int kChunks = WM * kChunksPerRow;
 #pragma unroll

@@ -25,6 +25,10 @@ constexpr int D = {D};
 constexpr int Nthreads = {Nthreads};
 constexpr int num_stages_qk = {num_stages_qk};   // LDS buffers of the first-contraction stream (+ mask)
 constexpr int num_stages_dv = {num_stages_dv};   // LDS buffers of the second-contraction stream
+// the same two counts for the passes that contract over d_v first (dQ, and dK when it is a chained pass): their streamed
+// tiles are d_v wide, twice the dV pass's at d_v = 2 d_qk, so they often cannot afford what the dV pass can
+constexpr int num_stages_ds = {num_stages_ds};
+constexpr int num_stages_dq = {num_stages_dq};
 constexpr int waves_per_eu = {waves_per_eu};
 constexpr int ds_rows = {ds_rows};               // 0, or kv rows per block of the dK kernel that reads a stored dS
 constexpr bool kStoredDs = ds_rows != 0;
@@ -37,18 +41,18 @@ constexpr int DKB = Kd;
 
 using aat::BwdPass;
 using TV = aat::RetBwdChain<Kd, D, DVB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col>;
-using TK = aat::RetBwdChain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col>;
-using TQ = aat::RetBwdChain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row>;
+using TK = aat::RetBwdChain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Col>;
+using TQ = aat::RetBwdChain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Row>;
 const auto kernel_dv = &aat::ret_bwd_chain<Kd, D, DVB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu>;
-const auto kernel_dk = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu>;
-const auto kernel_dq = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row, waves_per_eu>;
+const auto kernel_dk = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Col, waves_per_eu>;
+const auto kernel_dq = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Row, waves_per_eu>;
 const auto decay_dv = &aat::ret_bwd_chain<Kd, D, DVB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu, true>;
-const auto decay_dk = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Col, waves_per_eu, true>;
-const auto decay_dq = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row, waves_per_eu, true>;
+const auto decay_dk = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Col, waves_per_eu, true>;
+const auto decay_dq = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Row, waves_per_eu, true>;
 // stored dS: the row pass that writes it (the plain one again in a library without it), the dK kernel that reads it
 using TKD = aat::RetBwdDk<Kd, kDkRows, kDkTile, kDkRows * 2, kDkStages>;
-const auto kernel_dq_ds = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row, waves_per_eu, false, kStoredDs>;
-const auto decay_dq_ds = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_qk, num_stages_dv, BwdPass::Row, waves_per_eu, true, kStoredDs>;
+const auto kernel_dq_ds = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Row, waves_per_eu, false, kStoredDs>;
+const auto decay_dq_ds = &aat::ret_bwd_chain<D, Kd, DKB, Br, Bc, Nthreads, num_stages_ds, num_stages_dq, BwdPass::Row, waves_per_eu, true, kStoredDs>;
 const auto kernel_dk_ds = &aat::ret_bwd_dk_from_ds<Kd, kDkRows, kDkTile, kDkRows * 2, kDkStages, kDkWaves>;
 static_assert(!kStoredDs || Br % kDkTile == 0, "a query tile of the dK kernel lies inside one block of the row pass");
 

@@ -10,6 +10,7 @@
 #pragma once
 #include <type_traits>
 
+#include "../../utils/acc_file.h"
 #include "../../utils/cdna4.h"
 #include "../../utils/mask_extents.h"
 #include "../../utils/retention.h"
@@ -52,6 +53,10 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
                 const half_t* __restrict__ mask, half_t* __restrict__ o, float* __restrict__ r, int H,
                 int seq_k, int seq_q, int causal, const float* __restrict__ lg2gamma = nullptr,
                 const int* __restrict__ extents = nullptr) {
+  // One wave per SIMD: the output tile lives in the accumulation registers by number (utils/acc_file.h), the score
+  // tile in vector registers through hand-written matrix instructions, and the compiler allocates the rest.
+  constexpr bool kNumbered = WPE == 1;
+  if constexpr (kNumbered) acc_claim_all();
   if constexpr (DECAY) causal = 1;
   using T = RetFwdRegfuse<Kd, D, Br, Bc, Nthreads, NSK, NSV, NSM>;
   constexpr int RT = T::RT, NT = T::NT, KS = T::KS, DT = T::DT, NCK = T::NCK, NCV = T::NCV, NCM = T::NCM, WM = T::WM;
@@ -121,22 +126,12 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
         maddr[rt][i] = lds_addr(mbuf + lds_chunk_off<NCM, Swz::Rows16>(wave * WM + rt * 32 + n, i) + 8 * h);
   }
 
-  f16v oacc[RT][DT];
   RetentionRow row[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     row[rt].big_r = 0.f;
     row[rt].r_ref = 1.f;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      oacc[rt][dt] = zero16();
-      // One wave per SIMD: the zeros go into accumulation registers here.  As literals they also reach the epilogue
-      // on the path of a block without kv tiles, and the compiler then keeps that copy of the whole tile in vector
-      // registers across the main loop.
-      if constexpr (WPE == 1) asm volatile("" : "+a"(oacc[rt][dt]));
-    }
   }
-
   auto issue_km = [&](int j, int par) {          // K tile j and mask tile j travel together
     kdma.issue(kg + (size_t)j * T::kKBytes, kbuf + (NSK == 2 ? par * T::kKBytes : 0), wave_base);
     if constexpr (!DECAY) mdma.issue(mg + (size_t)j * Bc * 2, mbuf + (NSM == 2 ? par * T::kMBytes : 0), wave_base);
@@ -145,23 +140,120 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
     issue_km(0, 0);
     if constexpr (NSV == 2) vdma.issue(vg, vbuf, wave_base);
   }
+
+  if constexpr (kNumbered) {
+    static_assert(RT * DT * 16 <= 256, "a wave's output tile fills at most the accumulation file");
+    acc_zero<0, RT * DT * 16>();
+    // The copies of a tile are issued one instruction at a time between the matrix steps: a burst of them fills the
+    // memory pipeline's queue, and the wave -- the only one on its SIMD -- stands still with an idle matrix pipe until
+    // the queue has taken the last of them.
+    constexpr int KI = T::KDma::kIters, VI = T::VDma::kIters, MI = DECAY ? 0 : T::MDma::kIters;
+    auto issue_km_one = [&](int j, int par, int i) {          // instruction i of the K copy followed by the mask copy
+      if (i < KI) kdma.issue_one(i, kg + (size_t)j * T::kKBytes, kbuf + (NSK == 2 ? par * T::kKBytes : 0), wave_base);
+      else if constexpr (!DECAY) mdma.issue_one(i - KI, mg + (size_t)j * Bc * 2, mbuf + (NSM == 2 ? par * T::kMBytes : 0), wave_base);
+    };
+    // One loop body for both buffer parities: the parity is a run-time value that moves the operand addresses and the
+    // copy destinations.
+    int par = 0;
+    for (int j = 0; j < n_tiles; ++j) {
+      const bool more = (j + 1 < n_tiles);
+      // (A) K_j, mask_j (and with two V buffers V_j) have landed; every wave is past iteration j-1.
+      wait_vmcnt<0>();
+      block_sync();
+      f16v sacc[RT][NT];
+      // between the steps of the first contraction: V_j into a single V buffer, K_j+1 and mask_j+1 into second buffers
+      qk_gemm_steps<RT, NT, KS, NCK, PF, true>(sacc, qf, kaddr, 0, [&](int step) {
+        constexpr int kSteps = NT * KS, kOwnV = NSV == 1 ? VI : 0, kCopies = kOwnV + (NSK == 2 ? KI + MI : 0);
+        constexpr int kPer = (kCopies + kSteps - 1) / kSteps;
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+          const int i = step * kPer + u;
+          if (i < kOwnV) vdma.issue_one(i, vg + (size_t)j * T::kVBytes, vbuf, wave_base);
+          else if (i < kCopies && more) issue_km_one(j + 1, par ^ 1, i - kOwnV);
+        }
+      });
+      static_for<RT>([&](auto rt_tag) {
+        constexpr int rt = decltype(rt_tag)::value;
+        if constexpr (DECAY) {
+          const int own0 = q0 + wave * WM + rt * 32 + diag;              // q + diag of the group's first row
+          const auto one = [](int, int) { return 1.0f; };
+          if ((j + 1) * Bc - 1 > own0) decay.template apply<true>(sacc[rt], own0 + n - j * Bc, one);
+          else decay.template apply<false>(sacc[rt], own0 + n - j * Bc, one);
+        } else {
+          if constexpr (kFoldMask) apply_mask_folded_blind<NT>(sacc[rt], maddr[rt][0]);
+          else apply_mask<NT>(sacc[rt], maddr[rt], 0);
+        }
+        // the matrix instructions that last wrote the output tile are a whole score contraction back
+        retention_step_with<NT>(sacc[rt], row[rt], [&](float alpha) { acc_scale<16 * rt * DT, 16 * DT>(alpha); });
+      });
+      // (B) with one buffer: V_j must have landed / K and mask buffers must be free before the next fetch.
+      if constexpr (NSV == 1 || NSK == 1) {
+        if constexpr (NSV == 1) wait_vmcnt<0>();
+        block_sync();
+      }
+      h8 pf[RT][NT][2];
+      // between the steps of the second contraction: K_j+1 and mask_j+1 into single buffers (free since (B)), V_j+1 into
+      // the second V buffer (free since (A))
+      pv_gemm_steps_numbered<RT, NT, DT, NCV, PF, 0>(pf, vaddr, 0, [&](int g) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) pack_group<NT>(pf[rt], sacc[rt], g);
+      }, [&](int step) {
+        constexpr int kSteps = 2 * NT * DT, kKm = NSK == 1 ? KI + MI : 0, kCopies = kKm + (NSV == 2 ? VI : 0);
+        constexpr int kEvery = (kCopies > 0 && kSteps >= 2 * kCopies) ? kSteps / kCopies : 1;     // few copies: spread out
+        constexpr int kPer = (kCopies * kEvery + kSteps - 1) / kSteps;
+        if (step % kEvery != 0 || !more) return;
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+          const int i = (step / kEvery) * kPer + u;
+          if (i < kKm) issue_km_one(j + 1, 0, i);
+          else if (i < kCopies) vdma.issue_one(i - kKm, vg + (size_t)(j + 1) * T::kVBytes, vbuf + (par ^ 1) * T::kVBytes, wave_base);
+        }
+      });
+      // the next tile reads the other buffers
+      if constexpr (NSK == 2) {
+        const int dk = par ? -T::kKBytes : T::kKBytes;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kaddr[ks] += dk;
+      }
+      if constexpr (NSV == 2) {
+        const int dv = par ? -T::kVBytes : T::kVBytes;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vaddr[dt] += dv;
+      }
+      if constexpr (NSM == 2 && !DECAY) {
+        const int dm = par ? -T::kMBytes : T::kMBytes;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int i = 0; i < (kFoldMask ? 1 : NT * 4); ++i) maddr[rt][i] += dm;
+      }
+      par ^= 1;
+    }
+    acc_settle();
+    wait_vmcnt<0>();
+    block_sync();
+    float scale[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const float r_fin = fmaxf(row[rt].big_r, 1.0f);
+      scale[rt] = row[rt].r_ref * fast_rcp(r_fin);
+      if (h == 0) r[(size_t)bh * seq_q + q0 + wave * WM + rt * 32 + n] = r_fin;
+    }
+    store_o_tile_numbered<RT, DT, D, T::kOStride, 0>(scale, smem + wave * WM * T::kOStride,
+                                                     o + ((size_t)bh * seq_q + q0 + wave * WM) * D, lane);
+    return;
+  }
+
+  f16v oacc[RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] = zero16();
   auto kv_tile = [&](const int j, auto parity_tag) {
     constexpr int PAR = decltype(parity_tag)::value;
     char* const vcur = vbuf + (NSV == 2 ? PAR * T::kVBytes : 0);
     const bool more = (j + 1 < n_tiles);
 
-    if constexpr (WPE == 1) {
-      // Above 256 registers the file is split into 256 vector and 256 accumulation registers: keep the
-      // output accumulators in the accumulation half and the Q fragments in the vector half, or the
-      // allocator parks Q there and copies four registers back in front of every MFMA.
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[rt][ks]));
-      }
-    }
     // (A) K_j, mask_j (and with two V buffers V_j) have landed; every wave is past iteration j-1.
     wait_vmcnt<0>();
     block_sync();
@@ -172,9 +264,7 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
     }
 
     f16v sacc[RT][NT];
-    // the score tile accumulates in vector registers when the outputs fill the accumulation registers
-    constexpr bool kVacc = WPE == 1 && RT * (DT + NT) * 16 > 256;
-    qk_gemm_steps<RT, NT, KS, NCK, PF, kVacc>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
+    qk_gemm_steps<RT, NT, KS, NCK, PF>(sacc, qf, kaddr, NSK == 2 ? PAR * T::kKBytes : 0, [](int) {});
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       if constexpr (DECAY) {
@@ -186,7 +276,7 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
         if constexpr (kFoldMask) apply_mask_folded<NT>(sacc[rt], maddr[rt][0], NSM == 2 ? PAR * T::kMBytes : 0);
         else apply_mask<NT>(sacc[rt], maddr[rt], NSM == 2 ? PAR * T::kMBytes : 0);
       }
-      retention_step<NT, DT, WPE == 1>(sacc[rt], row[rt], oacc[rt]);
+      retention_step<NT, DT>(sacc[rt], row[rt], oacc[rt]);
     }
 
     // (B) with one buffer: V_j must have landed / K and mask buffers must be free before the next fetch.
@@ -198,7 +288,7 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
       }
     }
     h8 pf[RT][NT][2];
-    pv_gemm_steps<RT, NT, DT, NCV, PF, WPE == 1>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
+    pv_gemm_steps<RT, NT, DT, NCV, PF>(oacc, pf, vaddr, NSV == 2 ? PAR * T::kVBytes : 0, [&](int g) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) pack_group<NT>(pf[rt], sacc[rt], g);
     });
@@ -211,12 +301,6 @@ ret_fwd_regfuse(const half_t* __restrict__ q, const half_t* __restrict__ k, cons
   }
 
   // ---- epilogue -------------------------------------------------------------------------------------
-  if constexpr (WPE == 1) {        // the accumulators leave the loop where the MFMAs left them (see kv_tile)
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) asm volatile("" : "+a"(oacc[rt][dt]));
-  }
   wait_vmcnt<0>();
   block_sync();
   float scale[RT];

@@ -52,6 +52,28 @@ AAT_DEV void apply_mask_folded(f16v (&s)[NT], uint32_t chunk0, int buf_off) {
   }
 }
 
+// apply_mask_folded with the reads issued behind the compiler's back.  In front of an LDS read it can see, the compiler
+// waits for every LDS-DMA copy in flight (it takes them for writes the read may depend on): the copy of the next tile,
+// threaded between the matrix steps before this point, would be waited for here.
+template <int NT>
+AAT_DEV void apply_mask_folded_blind(f16v (&s)[NT], uint32_t chunk0) {
+  h4 m[NT * 4];
+#pragma unroll
+  for (int i = 0; i < NT * 4; ++i) {
+    const uint32_t a = chunk0 ^ (uint32_t)(i << 4);
+    asm volatile("ds_read_b64 %0, %1" : "=v"(m[i]) : "v"(a));
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)");
+#pragma unroll
+  for (int i = 0; i < NT * 4; ++i) asm volatile("" : "+v"(m[i]));       // no use of m[i] above the wait
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[t][4 * g + e] *= (float)m[4 * t + g][e];
+}
+
 // Decay mask evaluated in registers instead of read from a [H, S_q, S_kv] tensor.  The reference always
 // streams the tensor (reference: python/ops/retnet_interface.py:26-31) and lists "causal config" and the
 // mask stream's cost ("retnet performance issue ... mask stage 2?") as open items (README.md:102-114):
@@ -139,8 +161,9 @@ AAT_DEV void rescale_acc(f16v (&oacc)[DT], float alpha) {
 // Fold one masked score tile into the row statistics and turn it into P = S / r_ref (in place).
 // Rescales the O accumulators when the reference scale moves.
 // ACC_PIN: the O accumulators live in accumulation registers (kernels above 256 registers) and are rescaled there.
-template <int NT, int DT, bool ACC_PIN = false>
-AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) {
+// rescale(alpha): multiplies the row group's O accumulators, wherever they live.
+template <int NT, class Rescale>
+AAT_DEV void retention_step_with(f16v (&s)[NT], RetentionRow& row, Rescale&& rescale) {
   float part = 0.f;
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -152,13 +175,17 @@ AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) 
     const float r_new = fmaxf(row.big_r, 1.0f);
     const float alpha = row.r_ref * fast_rcp(r_new);
     row.r_ref = r_new;
-    rescale_acc<DT, ACC_PIN>(oacc, alpha);
+    rescale(alpha);
   }
   const float inv = fast_rcp(row.r_ref);
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int v = 0; v < 16; ++v) s[t][v] *= inv;
+}
+template <int NT, int DT, bool ACC_PIN = false>
+AAT_DEV void retention_step(f16v (&s)[NT], RetentionRow& row, f16v (&oacc)[DT]) {
+  retention_step_with<NT>(s, row, [&](float alpha) { rescale_acc<DT, ACC_PIN>(oacc, alpha); });
 }
 
 // Round 16 kv rows of P to one fp16 MFMA operand (no sum needed here).

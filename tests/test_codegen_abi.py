@@ -251,8 +251,9 @@ def test_resource_report_is_parsed_and_decides_what_the_tuner_times(tmp_path, mo
     assert not RetBwdTunner(ARCH, arrays, causal=True)._kernel_matters(usage[0]["kernel"])
     assert RetBwdTunner(ARCH, arrays, causal=True)._kernel_matters("_ZN3aat18ret_bwd_dk_from_dsILi256ELi128ELi64ELi256ELi2ELi2EEEvPKDF16_S2_PDF16_iiiiPKiii")
     attn = AttnTunner(ARCH, make_tensors("attn", 1, 2, 256, 256, 128, 128, "meta"), causal=True)
-    name = "_ZN3aat21flashattn_fwd_regfuseILi128ELi128ELi256ELi64ELi512ELi2ELi2ELi2ELb0ELb%dELb0ELb0EEEvPKDF16_"
-    assert attn._kernel_matters(name % 1) and not attn._kernel_matters(name % 0)
+    name = "_ZN3aat21flashattn_fwd_regfuseILi128ELi128ELi256ELi64ELi512ELi2ELi2ELi2ELi64ELb0ELb%dELb0ELb0ELb%dEEEvPKDF16_"
+    assert attn._kernel_matters(name % (1, 0)) and not attn._kernel_matters(name % (0, 0))
+    assert not attn._kernel_matters(name % (1, 1))            # the paired causal variant is launched only from a build that does not spill
     # every library of the shipping set carries its report, with one entry per kernel it holds
     cfg = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
     report = codegen.resource_usage(codegen.library_path(cfg))
@@ -273,8 +274,8 @@ def test_tune_skips_a_candidate_the_compiler_reports_as_spilling(tmp_path, monke
                str(bad): [{"kernel": "_Z1aILb0ELb0ELb0ELb0EEvPf", "scratch_bytes": 900}]}
     monkeypatch.setattr(codegen, "resource_usage", lambda lib: reports[lib])
     timed = []
-    monkeypatch.setattr(tuner, "profile", lambda lib: timed.append(lib) or 1.0)
-    monkeypatch.setattr(tuner, "verify", lambda lib: True)
+    monkeypatch.setattr(tuner, "profile", lambda lib, config=None: timed.append(lib) or 1.0)
+    monkeypatch.setattr(tuner, "verify", lambda lib, config=None: True)
     best = tuner.tune(log_path=str(tmp_path / "logs"), use_cache=False)
     assert best == good and timed == [str(good)] and tuner.rejected_spills == {bad: 900}
     log = (tmp_path / "logs" / "profile_result_attn_128_128.txt").read_text()
