@@ -140,22 +140,94 @@ def compile_config(config, arch, build_dir=None, timeout=None, force=False):
     with open(src, "w") as f:
         f.write(text)
     tmp = out + f".tmp{os.getpid()}_{threading.get_ident()}"     # two threads of one process may build the same library
-    try:
-        ret = subprocess.run(hipcc_command(src, tmp, arch), timeout=timeout, capture_output=True, text=True)
-    except subprocess.TimeoutExpired:
-        if os.path.exists(tmp):
+    scan = may_hold_numbered_accumulators(config)
+    workdir = None
+    command = hipcc_command(src, tmp, arch)
+    if scan:                                       # keep the compiler's assembly next to a private copy of the output
+        workdir = tmp + ".d"
+        os.makedirs(workdir, exist_ok=True)
+        tmp = os.path.join(workdir, os.path.basename(out))
+        command = hipcc_command(src, tmp, arch) + ["-save-temps=obj"]
+
+    def discard():
+        if workdir is not None:
+            shutil.rmtree(workdir, ignore_errors=True)
+        elif os.path.exists(tmp):
             os.remove(tmp)
+
+    try:
+        ret = subprocess.run(command, timeout=timeout, capture_output=True, text=True)
+    except subprocess.TimeoutExpired:
+        discard()
         return None
     if ret.returncode != 0:
         with open(out[:-3] + ".log", "w") as f:
             f.write(ret.stdout + ret.stderr)
-        if os.path.exists(tmp):
-            os.remove(tmp)
+        discard()
         return None
+    usage = parse_resource_usage(ret.stderr)
+    if scan:
+        listing = [os.path.join(workdir, f) for f in os.listdir(workdir) if f.endswith(".s") and "-hip-amdgcn" in f]
+        clashes = foreign_accumulator_use(open(listing[0]).read()) if len(listing) == 1 else {"<no device assembly found>": 1}
+        if clashes:
+            # The kernel keeps its output tile in accumulation registers it names itself and the compiler has put values
+            # of its own there as well: the library would compute garbage (or fault on a corrupted address).  A failed build.
+            with open(out[:-3] + ".log", "w") as f:
+                f.write("rejected: the compiler allocated accumulation registers in a kernel that addresses them by number\n")
+                for name, n in clashes.items():
+                    f.write(f"  {name}: {n} instructions outside the kernel's own asm statements name an accumulation register\n")
+            discard()
+            return None
     with open(usage_path(out), "w") as f:
-        json.dump(parse_resource_usage(ret.stderr), f, indent=1)
+        json.dump(usage, f, indent=1)
     os.replace(tmp, out)
+    discard()
     return out
+
+
+def may_hold_numbered_accumulators(config):
+    """Configurations whose kernels keep their output tile in accumulation registers addressed by number
+    (csrc/kernels/utils/acc_file.h): the one-wave-per-SIMD RetNet kernels.  Their builds are checked by
+    ``foreign_accumulator_use``."""
+    return getattr(config, "operation", "") in ("ret", "ret_bwd") and getattr(config, "waves_per_eu", 1) == 1
+
+
+_AGPR_OPERAND = re.compile(r"\ba\d+\b|\ba\[\d+")
+_KERNEL_LABEL = re.compile(r"^(_Z\w+):")
+
+
+NUMBERED_MARK = "aat: accumulation registers addressed by number"      # left in the assembly by acc_claim_all() (utils/acc_file.h)
+
+
+def foreign_accumulator_use(assembly):
+    """{kernel: count} for the kernels of a device assembly listing that address accumulation registers by number (they
+    carry NUMBERED_MARK) AND name such registers in instructions the compiler emitted itself (outside the #ASMSTART /
+    #ASMEND pairs).  The numbered registers are invisible to the compiler's allocation: with vector registers scarce it
+    loads operands or parks values in the same file, and the two uses overwrite each other.  Kernels without the mark
+    (ordinary MFMA code, accumulators handed to asm statements as operands) are the compiler's own business."""
+    own, foreign = {}, {}
+    kernel, in_asm = None, False
+    for line in assembly.splitlines():
+        m = _KERNEL_LABEL.match(line)
+        if m:
+            kernel, in_asm = m.group(1), False
+            continue
+        if kernel is None:
+            continue
+        if NUMBERED_MARK in line:
+            own[kernel] = 1
+        if "#ASMSTART" in line:
+            in_asm = True
+            continue
+        if "#ASMEND" in line:
+            in_asm = False
+            continue
+        text = line.split(";")[0].strip()
+        if not text or text.startswith("."):
+            continue
+        if not in_asm and _AGPR_OPERAND.search(text):
+            foreign[kernel] = foreign.get(kernel, 0) + 1
+    return {k: n for k, n in foreign.items() if own.get(k)}
 
 
 # ---- the compiler's per-kernel resource report ---------------------------------------------------------
@@ -173,7 +245,7 @@ def parse_resource_usage(text):
         m = _USAGE_LINE.search(line)
         if not m:
             continue
-        key, value = m.group(1).strip(), m.group(2)
+        key, value = m.group(1).split(":")[-1].strip(), m.group(2)      # with -save-temps the source position follows "remark:"
         if key == "Function Name":
             kernels.append({"kernel": value})
         elif kernels and key in _USAGE_FIELDS and value.lstrip("-").isdigit():

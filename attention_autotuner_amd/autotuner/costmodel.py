@@ -1,4 +1,4 @@
-"""A fitted cost model of the forward search space, used to decide which candidates are worth timing.
+"""A fitted cost model of a search space (forward kernels, RetNet backward), used to decide which candidates are worth timing.
 
 The reference exports (configuration, measured cycles) pairs for such a model and stops there
 (reference python/tests/export_costmodel_config.py:31-56; nothing in the reference reads the file back).
@@ -32,6 +32,13 @@ from . import gfx950_space
 from .configs import supported_configs
 
 FEATURES = ("matrix", "lds", "vector", "exposed", "steps", "blocks", "tail", "one")
+# ... and three more for the RetNet spaces, whose candidates differ mostly in what the first eight do not see:
+#     stream    bytes a CU pulls from L2 into LDS (K/V/mask or Y/Z tiles), at 64 bytes per cycle
+#     sync      block-wide barriers a block passes (two per step with single buffers, one with double, one more where
+#               the LDS-fused kernel exchanges row statistics)
+#     solo      matrix cycles of kernels that run one wave per SIMD (nothing to overlap with)
+RET_FEATURES = FEATURES + ("stream", "sync", "solo")
+ALL_FEATURES = RET_FEATURES
 SIMDS, CUS = 1024, 256
 
 
@@ -40,8 +47,59 @@ def _rounds(n_blocks, per_cu):
     return n_blocks / resident, math.ceil(n_blocks / resident)
 
 
-def features(cfg, shape, causal=False):
-    """The feature vector (order of FEATURES) of forward configuration ``cfg`` on ``shape`` = (B, H, Sq, Sk)."""
+def _chain_features(n_blocks, steps, rows, tile, kx, dz, nw, per_cu, wave_lds_share=1.0, barriers=2, mask_tiles=1):
+    """The per-launch quantities of one chained-contraction kernel: ``rows`` resident rows per block, streamed tiles of
+    ``tile`` rows, first contraction over ``kx`` columns, second into ``dz`` columns; every wave reads whole tiles."""
+    waves_per_simd = max(1.0, per_cu * nw / 4.0)
+    mfma_per_step = rows * tile * (kx + dz) / (32 * 32 * 16)
+    matrix = n_blocks * steps * mfma_per_step * 32.0 / SIMDS
+    lds = n_blocks * steps * nw * (tile * kx * 2 + tile * dz * 2) * wave_lds_share / 128.0 / CUS
+    vector = n_blocks * steps * nw * (rows * tile / 64.0 / nw) * 6.0 / SIMDS
+    exposed = (matrix + lds + vector) / waves_per_simd
+    frac_rounds, whole_rounds = _rounds(n_blocks, per_cu)
+    tail = (whole_rounds - frac_rounds) * steps * mfma_per_step * 32.0 / nw
+    stream = n_blocks * steps * (tile * kx * 2 + tile * dz * 2 + rows * tile * 2 * mask_tiles) / 64.0 / CUS
+    sync = steps * whole_rounds * barriers
+    solo = matrix if waves_per_simd <= 1.0 else 0.0
+    return np.array([matrix, lds, vector, exposed, steps * whole_rounds, float(whole_rounds), tail, 0.0, stream, sync, solo])
+
+
+def backward_features(cfg, shape, causal=False):
+    """The same quantities for a RetNet backward configuration, summed over the kernels one launch runs: the dV pass
+    (resident kv rows, streamed query tiles), the dQ pass (resident query rows, streamed kv tiles) and either the chained
+    dK pass or, with a stored dS, the dK kernel that reads it back (a third of a chained pass's matrix work, two waves per
+    SIMD, ``ds_rows`` kv rows per block)."""
+    b, h, sq, sk = shape
+    nw = cfg.Nthreads // 64
+    half = 0.5 if causal else 1.0                         # a causal walk visits about half the streamed tiles
+    per_cu = gfx950_space.blocks_per_cu(cfg)
+    dvb = gfx950_space.backward_dv_cols(cfg)
+    total = np.zeros(len(ALL_FEATURES))
+    bars_v = 2 if (cfg.num_stages_qk == 1 or cfg.num_stages_dv == 1) else 1
+    sds, sdq = getattr(cfg, "num_stages_ds", cfg.num_stages_qk), getattr(cfg, "num_stages_dq", cfg.num_stages_dv)
+    bars_q = 2 if (sds == 1 or sdq == 1) else 1
+    # dV: grid over kv blocks (x column slices where the output is cut), streams Sq / Bc query tiles
+    total += _chain_features(b * h * (sk // cfg.Br) * (cfg.D // dvb), half * sq / cfg.Bc + 0.5 * causal, cfg.Br, cfg.Bc, cfg.Kd, dvb, nw, per_cu, barriers=bars_v)
+    # dQ: grid over query blocks, streams Sk / Bc kv tiles
+    total += _chain_features(b * h * (sq // cfg.Br), half * sk / cfg.Bc + 0.5 * causal, cfg.Br, cfg.Bc, cfg.D, cfg.Kd, nw, per_cu, barriers=bars_q)
+    ds_rows = getattr(cfg, "ds_rows", 0)
+    if ds_rows:                                           # dK = dS^T Q only: 64-row query tiles, 2 * ds_rows threads
+        total += _chain_features(b * h * (sk // ds_rows), half * sq / 64 + 0.5 * causal, ds_rows, 64, 0, cfg.Kd, ds_rows // 32, 2, barriers=1, mask_tiles=1)
+        total[8] += b * h * sq * sk * 2 * 2 * half / 64.0 / CUS       # the dS round trip through memory (written once, read once)
+    else:
+        total += _chain_features(b * h * (sk // cfg.Br), half * sq / cfg.Bc + 0.5 * causal, cfg.Br, cfg.Bc, cfg.D, cfg.Kd, nw, per_cu, barriers=bars_q)
+    total[7] = 1.0
+    return total
+
+
+def features(cfg, shape, causal=False, names=FEATURES):
+    """The feature vector (in the order of ``names``) of configuration ``cfg`` on ``shape`` = (B, H, Sq, Sk): forward
+    kernels in ``forward_features``, the RetNet backward in ``backward_features``."""
+    full = backward_features(cfg, shape, causal) if getattr(cfg, "operation", "") == "ret_bwd" else forward_features(cfg, shape, causal)
+    return np.array([full[ALL_FEATURES.index(n)] for n in names])
+
+
+def forward_features(cfg, shape, causal=False):
     b, h, sq, sk = shape
     nw = cfg.Nthreads // 64
     splits = max(1, getattr(cfg, "kv_splits", 1))
@@ -73,21 +131,28 @@ def features(cfg, shape, causal=False):
     tail = (whole_rounds - frac_rounds) * steps * mfma_per_step * 32.0 / nw
     if getattr(cfg, "sw_pipeline", 0):
         exposed *= 0.8
-    return np.array([matrix, lds, vector, exposed, step_count, float(whole_rounds), tail, 1.0])
+    has_mask = getattr(cfg, "operation", "") == "ret"
+    stream = n_blocks * steps * (cfg.Bc * (cfg.Kd + cfg.D) * 2 + (cfg.Br * cfg.Bc * 2 if has_mask else 0)) / 64.0 / CUS
+    single = getattr(cfg, "num_stages_qk", 2) == 1 or getattr(cfg, "num_stages_v", 2) == 1
+    barriers = (2 if single else 1) + (1 if cfg.fuse_type == "shared" and max(1, cfg.warps_mma1_n) > 1 else 0) + (1 if cfg.fuse_type == "shared" else 0)
+    sync = step_count * barriers
+    solo = matrix if waves_per_simd <= 1.0 else 0.0
+    return np.array([matrix, lds, vector, exposed, step_count, float(whole_rounds), tail, 1.0, stream, sync, solo])
 
 
 class CostModel:
-    def __init__(self, weights=None, unit="ms"):
-        self.weights = np.zeros(len(FEATURES)) if weights is None else np.asarray(weights, dtype=float)
+    def __init__(self, weights=None, unit="ms", names=FEATURES):
+        self.names = tuple(names)
+        self.weights = np.zeros(len(self.names)) if weights is None else np.asarray(weights, dtype=float)
         self.unit = unit
 
     def predict(self, cfg, shape, causal=False):
-        return float(self.weights @ features(cfg, shape, causal))
+        return float(self.weights @ features(cfg, shape, causal, self.names))
 
     def fit(self, samples, ridge=1e-3):
         """``samples``: iterable of (cfg, shape, causal, measured cost).  Ridge regression on features scaled to
         unit mean, so that one weight does not dominate because its feature is counted in larger units."""
-        x = np.array([features(c, s, ca) for c, s, ca, _ in samples])
+        x = np.array([features(c, s, ca, self.names) for c, s, ca, _ in samples])
         y = np.array([t for *_, t in samples], dtype=float)
         scale = np.maximum(x.mean(axis=0), 1e-12)
         xs = x / scale
@@ -103,13 +168,13 @@ class CostModel:
         return order.index(best)
 
     def to_dict(self):
-        return {"features": list(FEATURES), "weights": [float(w) for w in self.weights], "unit": self.unit}
+        return {"features": list(self.names), "weights": [float(w) for w in self.weights], "unit": self.unit}
 
     @classmethod
     def from_dict(cls, d):
-        if list(d["features"]) != list(FEATURES):
-            raise ValueError("cost model was fitted on a different feature set")
-        return cls(d["weights"], d.get("unit", "ms"))
+        if any(n not in ALL_FEATURES for n in d["features"]) or len(d["features"]) != len(d["weights"]):
+            raise ValueError("cost model was fitted on a feature set this version does not compute")
+        return cls(d["weights"], d.get("unit", "ms"), d["features"])
 
     def save(self, path):
         with open(path, "w") as f:
@@ -152,7 +217,7 @@ def samples_from_tuning_log(path, op, dim_qk, dim_v, shape, causal=False, failed
     with open(path) as f:
         lines = [l.rstrip("\n") for l in f]
     for i in range(len(lines) - 1):
-        if not lines[i].startswith("Config(") or (i > 0 and lines[i - 1].startswith("best config")):
+        if not re.match(r"\w*Config\(", lines[i]) or (i > 0 and lines[i - 1].startswith("best config")):
             continue
         try:
             ms = float(lines[i + 1])
@@ -160,6 +225,26 @@ def samples_from_tuning_log(path, op, dim_qk, dim_v, shape, causal=False, failed
             continue
         if ms < failed:
             out.append((config_from_log_line(lines[i], op, dim_qk, dim_v), tuple(shape), bool(causal), ms))
+    return out
+
+
+def samples_from_summary(path, op, only=None):
+    """Samples of every recorded tuning run of ``op`` listed in a ``summary.jsonl`` (one JSON object per run with its
+    problem, its causal flag and the path of its per-candidate log, as ``benchmarks/tune.py`` prints them).  Log paths are
+    taken relative to the summary's directory when they do not exist as written.  ``only``: a predicate on the run record."""
+    import os
+    out = []
+    with open(path) as f:
+        runs = [json.loads(l) for l in f if l.strip()]
+    for r in runs:
+        if r.get("op") != op or (only is not None and not only(r)):
+            continue
+        log = r["log"]
+        if not os.path.exists(log):
+            log = os.path.join(os.path.dirname(os.path.abspath(path)), os.path.basename(log))
+        b, h, sq, sk, dqk, dv = r["problem"]
+        causal = bool(r.get("causal")) or "decay" in os.path.basename(log)
+        out += samples_from_tuning_log(log, op, dqk, dv, (b, h, sq, sk), causal)
     return out
 
 
@@ -185,10 +270,17 @@ def main(argv=None):
     import argparse
     from . import codegen
     ap = argparse.ArgumentParser()
-    ap.add_argument("command", choices=["fit"])
-    ap.add_argument("exports", nargs="+")
+    ap.add_argument("command", choices=["fit", "fit-logs"])
+    ap.add_argument("exports", nargs="+", help="fit: exporter JSON files; fit-logs: entries of a tuning summary.jsonl (see fit_from_summary)")
     ap.add_argument("--out", required=True)
+    ap.add_argument("--op", default=None, help="fit-logs: the operator whose runs are used")
     args = ap.parse_args(argv)
+    if args.command == "fit-logs":
+        samples = [s for path in args.exports for s in samples_from_summary(path, args.op)]
+        model = CostModel(unit="ms", names=RET_FEATURES if args.op in ("ret", "ret_bwd") else FEATURES).fit(samples)
+        model.save(args.out)
+        print(json.dumps({"samples": len(samples), "out": args.out}))
+        return 0
     samples = [s for path in args.exports for s in samples_from_export(path, codegen.MAX_SCRATCH_BYTES)]
     model = CostModel(unit="cycles").fit(samples)
     model.save(args.out)

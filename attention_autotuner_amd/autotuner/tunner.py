@@ -66,6 +66,18 @@ class _ForwardTunner(BaseTunner):
         return super().tune(*a, **kw)
 
 
+def _shipped_cost_model(arch, cache_path, name):
+    """The fitted model ``name`` next to the tuning cache, or None (no file, another platform, AAT_TUNE_PRUNE=0)."""
+    path = os.path.join(cache_path, name)
+    if not (_is_rocm(arch) and os.environ.get("AAT_TUNE_PRUNE", "1") != "0" and os.path.exists(path)):
+        return None
+    from .costmodel import CostModel
+    try:
+        return CostModel.load(path)
+    except (OSError, ValueError, KeyError):
+        return None
+
+
 class AttnTunner(_ForwardTunner):
     operation = "attn"
 
@@ -73,13 +85,7 @@ class AttnTunner(_ForwardTunner):
         super().__init__(arch, torch_array, "attention", causal=causal, softmax_scale=softmax_scale)
         # the space has a few hundred candidates: with a fitted cost model next to the tuning cache, only the
         # third it ranks best is built and timed (AAT_TUNE_PRUNE=0: time everything, as the reference does)
-        model = os.path.join(self.cache_path, "costmodel_attn.json")
-        if _is_rocm(arch) and os.environ.get("AAT_TUNE_PRUNE", "1") != "0" and os.path.exists(model):
-            from .costmodel import CostModel
-            try:
-                self.cost_model = CostModel.load(model)
-            except (OSError, ValueError, KeyError):
-                self.cost_model = None
+        self.cost_model = _shipped_cost_model(arch, self.cache_path, "costmodel_attn.json")
 
     def _ex_args(self):
         scale = self.softmax_scale
@@ -93,6 +99,7 @@ class RetTunner(_ForwardTunner):
 
     def __init__(self, arch, torch_array, causal=False, decay=False, mask_mode=None):
         super().__init__(arch, torch_array, "retnet", causal=causal or decay, decay=decay, mask_mode=mask_mode)
+        self.cost_model = _shipped_cost_model(arch, self.cache_path, "costmodel_ret.json")
 
 
 class RetBwdTunner(BaseTunner):
@@ -100,6 +107,7 @@ class RetBwdTunner(BaseTunner):
 
     def __init__(self, arch, torch_array, causal=False, decay=False, mask_mode=None):
         super().__init__(arch, torch_array, "retnet_bwd", causal=causal or decay, decay=decay, mask_mode=mask_mode)
+        self.cost_model = _shipped_cost_model(arch, self.cache_path, "costmodel_ret_bwd.json")
         if _is_rocm(arch):
             self.Br_list = list(getattr(gfx950_space, "BWD_BR_LIST", (64, 128)))
             self.Bc_list = list(getattr(gfx950_space, "BWD_BC_LIST", (32, 64, 128)))

@@ -304,18 +304,18 @@ attn_bwd_chain(const half_t* __restrict__ x1, const half_t* __restrict__ x2, con
       if constexpr (COL) read_stats(std::integral_constant<int, 0>{});
       static_for<G>([&](auto it) {
         constexpr int i = decltype(it)::value, rt = i / (NT * 4), t = (i / 4) % NT, g = i % 4;
-        f4v l2 = l2r[i % 2], dl = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (kOut2) dl = dlr[i % 2];
-        if constexpr (COL) {
+        if constexpr (COL) {                     // the next group's read goes into the other slot; wait on this slot before taking its value
           if constexpr (i + 1 < G) {
             read_stats(std::integral_constant<int, i + 1>{});
-            if constexpr (kOut2) lds_wait_younger<2>(l2, dl);
-            else lds_wait_younger<1>(l2);
+            if constexpr (kOut2) lds_wait_younger<2>(l2r[i % 2], dlr[i % 2]);
+            else lds_wait_younger<1>(l2r[i % 2]);
           } else {
-            if constexpr (kOut2) lds_wait_younger<0>(l2, dl);
-            else lds_wait_younger<0>(l2);
+            if constexpr (kOut2) lds_wait_younger<0>(l2r[i % 2], dlr[i % 2]);
+            else lds_wait_younger<0>(l2r[i % 2]);
           }
         }
+        f4v l2 = l2r[i % 2], dl = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (kOut2) dl = dlr[i % 2];
         // The score of resident row x and streamed row y = jt*BY + c + 4h (c = 32t + 8g + e, a constant) is masked
         // when kv > q + diag: COL (x is kv) x - diag - jt*BY - 4h > c, ROW (x is q) c > x + diag - jt*BY - 4h.
         const int xrow = x0 + wave * WM + rt * 32 + n;               // resident row of this lane

@@ -98,7 +98,9 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   // lives there by number, outside the compiler's allocation (utils/acc_file.h): with the tile as a C++ value the
   // variants with more than one buffer per stream -- one loop body per ring slot -- come out with the sixteen tuples
   // placed differently from body to body and hundreds of bytes of scratch traffic per tile to reconcile them.
-  constexpr bool kNumbered = WPE == 1 && RT * DT * 16 == 256;
+  // (One row group per wave only: with two the resident fragments and the score tile no longer fit 256 vector registers,
+  // the compiler would reach for the accumulation file itself, and the build would be rejected.)
+  constexpr bool kNumbered = WPE == 1 && RT == 1 && DT * 16 == 256;
   if constexpr (kNumbered) acc_claim_all();
   if constexpr (DECAY) causal = 1;
   constexpr int PF = AAT_PF;

@@ -181,12 +181,14 @@ ret_bwd_dk_from_ds(const half_t* __restrict__ q, const half_t* __restrict__ ds, 
       h8 bf;
       static_for<DT>([&](auto dt_tag) {
         constexpr int dt = decltype(dt_tag)::value;
+        // wait on the slot, take its value, refill it (a copy made before the wait could read a register whose load
+        // has not landed); the B pair is older: it has landed too
+        lds_wait_younger<2 * ((dt + PF - 1 < DT) ? PF - 1 : DT - 1 - dt)>(lo[dt % PF], hi[dt % PF]);
         h4 clo = lo[dt % PF], chi = hi[dt % PF];
         if constexpr (dt + PF < DT) {
           lo[dt % PF] = lds_read_tr_h4_async(zaddr[dt + PF], off + s * kZRow16);
           hi[dt % PF] = lds_read_tr_h4_async(zaddr[dt + PF], off + s * kZRow16 + kZRow8);
         }
-        lds_wait_younger<2 * ((dt + PF < DT) ? PF : DT - 1 - dt)>(clo, chi);      // the B pair is older: it has landed too
         if constexpr (dt == 0) {
           asm volatile("" : "+v"(blo), "+v"(bhi));
           bf = cat_h4(blo, bhi);

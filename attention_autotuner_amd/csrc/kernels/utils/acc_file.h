@@ -28,8 +28,11 @@ namespace aat {
       AAT_D10("a14"), AAT_D10("a15"), AAT_D10("a16"), AAT_D10("a17"), AAT_D10("a18"), AAT_D10("a19"), AAT_D10("a20"),  \
       AAT_D10("a21"), AAT_D10("a22"), AAT_D10("a23"), AAT_D10("a24"), "a250", "a251", "a252", "a253", "a254", "a255"
 
-// Claim all 256 accumulation registers for the kernel (call once, first thing).
-AAT_DEV void acc_claim_all() { asm volatile("" ::: AAT_AGPR_ALL); }
+// Claim all 256 accumulation registers for the kernel (call once, first thing).  The comment it leaves in the kernel's
+// assembly marks the kernel for the build's check that the compiler has kept out of the file (autotuner/codegen.py:
+// foreign_accumulator_use): without it the check takes the kernel for ordinary MFMA code, so every kernel that uses
+// the functions below must call this.
+AAT_DEV void acc_claim_all() { asm volatile("; aat: accumulation registers addressed by number" ::: AAT_AGPR_ALL); }
 
 // a[LO : LO+15] += A x B (32x32x16, fp16 operands).
 template <int LO> AAT_DEV void acc_mfma_32x32x16(const h8& a, const h8& b) {
@@ -99,9 +102,9 @@ AAT_DEV void pv_gemm_steps_numbered(h8 (&pf)[RT][NT][2], const uint32_t (&vaddr)
   static_for<S>([&](auto step_tag) {
     constexpr int step = decltype(step_tag)::value;
     constexpr int g = step / DT, dt = step % DT;
+    lds_wait_younger<2 * ((step + PF - 1 < S) ? PF - 1 : S - 1 - step)>(lo[step % PF], hi[step % PF]);   // wait, take, refill (qk_gemm_steps)
     h4 clo = lo[step % PF], chi = hi[step % PF];
     if constexpr (step + PF < S) read(step + PF, step % PF);
-    lds_wait_younger<2 * ((step + PF < S) ? PF : S - 1 - step)>(clo, chi);
     const h8 vf = cat_h4(clo, chi);
     static_for<RT>([&](auto rt_tag) {
       constexpr int rt = decltype(rt_tag)::value;

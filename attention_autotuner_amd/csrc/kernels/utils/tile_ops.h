@@ -217,9 +217,11 @@ AAT_DEV void qk_gemm_steps(f16v (&sacc)[RT][NT], const h8 (&qf)[RT][KS], const u
       }
       if constexpr (step + PF < S) ring[step % PF] = read(step + PF);
     } else {
+      // Wait on the slot itself, then take its value, then refill it: a copy of the value made before the wait (the
+      // allocator is free to split a live range with a move) would read a register whose load has not landed.
+      lds_wait_younger<(step + PF - 1 < S) ? PF - 1 : S - 1 - step>(ring[step % PF]);
       h8 cur = ring[step % PF];
       if constexpr (step + PF < S) ring[step % PF] = read(step + PF);
-      lds_wait_younger<(step + PF < S) ? PF : S - 1 - step>(cur);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         if constexpr (!VACC) sacc[rt][step / KS] = mfma_32x32x16(cur, qf[rt][step % KS], sacc[rt][step / KS]);
@@ -266,13 +268,13 @@ AAT_DEV void pv_gemm_steps_hl(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const u
   static_for<S>([&](auto step_tag) {
     constexpr int step = decltype(step_tag)::value;
     constexpr int g = step / DT, dt = step % DT;
+    lds_wait_younger_either<BLIND, 2 * ((step + PF - 1 < S) ? PF - 1 : S - 1 - step)>(lo[step % PF], hi[step % PF]);   // wait, take, refill (qk_gemm_steps)
     h4 clo = lo[step % PF], chi = hi[step % PF];
     if constexpr (step + PF < S) {
       constexpr int nx = step + PF;
       lo[step % PF] = lds_read_tr_h4_either<BLIND>(vlo[nx % DT], buf_off + (nx / DT) * kRow16);
       hi[step % PF] = lds_read_tr_h4_either<BLIND>(vhi[nx % DT], buf_off + (nx / DT) * kRow16);
     }
-    lds_wait_younger_either<BLIND, 2 * ((step + PF < S) ? PF : S - 1 - step)>(clo, chi);
     const h8 vf = cat_h4(clo, chi);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);
@@ -337,9 +339,9 @@ AAT_DEV void pv_gemm_steps(f16v (&oacc)[RT][DT], h8 (&pf)[RT][NT][2], const uint
       }
       if constexpr (step + PF < S) read(step + PF, step % PF);
     } else {
+      lds_wait_younger_either<kHand, 2 * ((step + PF - 1 < S) ? PF - 1 : S - 1 - step)>(lo[step % PF], hi[step % PF]);   // wait, take, refill (qk_gemm_steps)
       h4 clo = lo[step % PF], chi = hi[step % PF];
       if constexpr (step + PF < S) read(step + PF, step % PF);
-      lds_wait_younger_either<kHand, 2 * ((step + PF < S) ? PF : S - 1 - step)>(clo, chi);
       const h8 vf = cat_h4(clo, chi);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) oacc[rt][dt] = mfma_32x32x16(vf, pf[rt][g / 2][g % 2], oacc[rt][dt]);

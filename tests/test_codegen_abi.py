@@ -234,6 +234,11 @@ x.hip:3:1: remark:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=kernel-reso
 
 
 def test_resource_report_is_parsed_and_decides_what_the_tuner_times(tmp_path, monkeypatch):
+    # a build that keeps its temporaries prints the same remarks with the source position behind "remark:"
+    kept = codegen.parse_resource_usage("remark: a/b.h:83:0: Function Name: _Z1kv [-Rpass-analysis=kernel-resource-usage]\n"
+                                        "remark: a/b.h:83:0:     VGPRs: 42 [-Rpass-analysis=kernel-resource-usage]\n"
+                                        "remark: a/b.h:83:0:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=kernel-resource-usage]\n")
+    assert kept == [{"kernel": "_Z1kv", "vgprs": 42, "scratch_bytes": 16}]
     usage = codegen.parse_resource_usage(REMARKS)
     assert [k["scratch_bytes"] for k in usage] == [2416, 16] and usage[0]["vgprs"] == 256 and usage[0]["vgpr_spills"] == 604
     assert usage[0]["occupancy"] == 1 and usage[0]["agprs"] == 256 and usage[0]["sgprs"] == 58
@@ -280,3 +285,53 @@ def test_tune_skips_a_candidate_the_compiler_reports_as_spilling(tmp_path, monke
     assert best == good and timed == [str(good)] and tuner.rejected_spills == {bad: 900}
     log = (tmp_path / "logs" / "profile_result_attn_128_128.txt").read_text()
     assert "not timed (compiler reports 900 bytes/lane of scratch): " + str(bad) in log
+
+
+LISTING = """
+_ZN3aat15ret_fwd_regfuseILi128ELi128EEEvPKDF16_:
+	;;#ASMSTART
+	; aat: accumulation registers addressed by number
+	;;#ASMEND
+	global_load_dwordx4 a[2:5], v[6:7], off
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_f16 a[0:15], v[0:3], v[4:7], a[0:15]
+	;;#ASMEND
+	v_accvgpr_read_b32 v66, a14
+	s_endpgm
+_ZN3aat15ret_fwd_regfuseILi256ELi512EEEvPKDF16_:
+	;;#ASMSTART
+	; aat: accumulation registers addressed by number
+	;;#ASMEND
+	;;#ASMSTART
+	v_accvgpr_write_b32 a[255], 0
+	;;#ASMEND
+	v_add_f32_e32 v1, v2, v3              ; a12 in a comment is no operand
+	s_endpgm
+_ZN3aat21flashattn_fwd_regfuseILi128EEEvPKDF16_:
+	v_mfma_f32_32x32x16_f16 a[0:15], v[0:3], v[4:7], a[0:15]
+	;;#ASMSTART
+	v_accvgpr_read_b32 v5, a7
+	;;#ASMEND
+	v_accvgpr_read_b32 v1, a3
+	s_endpgm
+"""
+
+
+def test_a_build_whose_compiler_uses_the_numbered_accumulation_registers_is_rejected(tmp_path):
+    """Kernels that address accumulation registers by number (utils/acc_file.h) are only sound when the compiler keeps
+    nothing of its own in that file.  The listing check: a kernel that names such registers inside its asm statements and
+    also in compiler-emitted instructions is reported; one that does only the former, or one without the mark (ordinary
+    MFMA code, accumulators handed to asm statements as operands), is not.  And a configuration known to provoke it (two row groups per wave: the fragments no longer fit
+    the vector registers) fails to build, with the reason in its log."""
+    assert codegen.foreign_accumulator_use(LISTING) == {"_ZN3aat15ret_fwd_regfuseILi128ELi128EEEvPKDF16_": 2}
+    from attention_autotuner_amd.autotuner.configs import RetConfig
+    tight = RetConfig(256, 128, 128, 128, 128, 128, 1, 1, 1, 256, True, waves_per_eu=1).set_fuse_type("register")
+    assert codegen.may_hold_numbered_accumulators(tight)
+    assert not codegen.may_hold_numbered_accumulators(gfx950_space.default_forward_config("attn", 128, 128, ARCH))
+    assert codegen.compile_config(tight, ARCH, build_dir=str(tmp_path), force=True) is None
+    log = open(codegen.library_path(tight, str(tmp_path))[:-3] + ".log").read()
+    assert "accumulation registers" in log and "ret_fwd_regfuse" in log
+    assert not [f for f in os.listdir(os.path.dirname(codegen.library_path(tight, str(tmp_path)))) if f.endswith((".so", ".d"))]
+    # the shipped one-wave configuration of the same kernel passes the check
+    fine = gfx950_space.default_forward_config("ret", 256, 512, ARCH)
+    assert fine.waves_per_eu == 1 and fine.fuse_type == "register" and os.path.exists(codegen.library_path(fine))

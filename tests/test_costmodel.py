@@ -156,3 +156,71 @@ def test_cycle_exporter_counts_prebuilt_candidates_in_the_reference_tuple_layout
     samples = costmodel.samples_from_export(str(out))
     assert [s[1] for s in samples] == [(b, h, sq, sk)] * 4 and all(s[3] == r["cycles"] for s, r in zip(samples, records))
     assert np.isfinite(costmodel.CostModel(unit="cycles").fit(samples).weights).all()
+
+
+# ---- RetNet forward and backward spaces -----------------------------------------------------------------
+RET_RUNS = {                                              # file -> (operator, (B, H, Sq, Sk, d_qk, d_v), causal walk)
+    "ret_b4h8q2048k2048_c0_256_512.txt": ("ret", (4, 8, 2048, 2048, 256, 512), False),
+    "ret_b4h8q2048k2048_c1_256_512.txt": ("ret", (4, 8, 2048, 2048, 256, 512), True),
+    "ret_decay_b4h8q2048k2048_c1_256_512.txt": ("ret", (4, 8, 2048, 2048, 256, 512), True),
+    "ret_b4h8q2048k2048_c1_128_128.txt": ("ret", (4, 8, 2048, 2048, 128, 128), True),
+    "ret_b4h8q2048k2048_c1_256_256.txt": ("ret", (4, 8, 2048, 2048, 256, 256), True),
+    "ret_bwd_b4h8q2048k2048_c0_256_512.txt": ("ret_bwd", (4, 8, 2048, 2048, 256, 512), False),
+    "ret_bwd_b4h8q2048k2048_c1_256_512.txt": ("ret_bwd", (4, 8, 2048, 2048, 256, 512), True),
+    "ret_bwd_decay_b4h8q2048k2048_c1_256_512.txt": ("ret_bwd", (4, 8, 2048, 2048, 256, 512), True),
+    "ret_bwd_b4h8q2048k2048_c1_128_128.txt": ("ret_bwd", (4, 8, 2048, 2048, 128, 128), True),
+    "ret_bwd_b4h8q2048k2048_c1_256_256.txt": ("ret_bwd", (4, 8, 2048, 2048, 256, 256), True),
+}
+
+
+def _ret_samples(name):
+    op, (b, h, sq, sk, dqk, dv), causal = RET_RUNS[name]
+    return costmodel.samples_from_tuning_log(os.path.join(LOGS, name), op, dqk, dv, (b, h, sq, sk), causal)
+
+
+def _survives(model, runs, tuner_cls):
+    times = np.array([s[3] for s in runs])
+    pred = np.array([model.predict(*s[:3]) for s in runs])
+    keep = np.argsort(pred)[:max(tuner_cls.keep_min, int(len(runs) * tuner_cls.keep_fraction + 0.999))]
+    return times[keep].min() == times.min()
+
+
+@pytest.mark.parametrize("op", ["ret", "ret_bwd"])
+def test_retnet_models_keep_the_winner_of_head_sizes_they_have_not_seen(op):
+    """Recorded exhaustive runs of the RetNet forward and backward spaces (three head-size pairs, dense, causal and decay
+    walks; the backward with its per-pass buffer counts and the stored-dS variants).  The shipped models are the fit on
+    all of them; a model fitted WITHOUT the runs of one head-size pair must still rank that pair's measured winners
+    inside the share the tuning loop keeps."""
+    from attention_autotuner_amd.autotuner import RetBwdTunner, RetTunner
+    from attention_autotuner_amd.benchmarks.tune import make_tensors
+    cls = RetTunner if op == "ret" else RetBwdTunner
+    names = [n for n, r in RET_RUNS.items() if r[0] == op]
+    runs = {n: _ret_samples(n) for n in names}
+    assert all(len(r) >= 27 for r in runs.values())
+    if op == "ret_bwd":                                    # lines of the backward log parse back with every knob
+        some = runs["ret_bwd_b4h8q2048k2048_c1_256_512.txt"]
+        assert {c.ds_rows for c, *_ in some} == {0, 128, 256} and len({(c.num_stages_qk, c.num_stages_dv, c.num_stages_ds, c.num_stages_dq) for c, *_ in some}) > 4
+    everything = [s for r in runs.values() for s in r]
+    fitted = costmodel.CostModel(unit="ms", names=costmodel.RET_FEATURES).fit(everything)
+    tuner = cls(MI355X(), make_tensors(op, 4, 8, 2048, 2048, 256, 512, "meta"), causal=True)
+    assert tuner.cost_model is not None and tuner.cost_model.names == costmodel.RET_FEATURES
+    np.testing.assert_allclose(tuner.cost_model.weights, fitted.weights, rtol=1e-6)
+    for n in names:
+        assert _survives(tuner.cost_model, runs[n], cls), (n, tuner.cost_model.rank_of_best(runs[n]))
+    for dims in {RET_RUNS[n][1][4:] for n in names}:
+        train = [s for n in names if RET_RUNS[n][1][4:] != dims for s in runs[n]]
+        held_out = costmodel.CostModel(unit="ms", names=costmodel.RET_FEATURES).fit(train)
+        for n in names:
+            if RET_RUNS[n][1][4:] == dims:
+                assert _survives(held_out, runs[n], cls), (dims, n, held_out.rank_of_best(runs[n]))
+    # the tuner prunes with it, and AAT_TUNE_PRUNE=0 switches that off
+    cfgs = [c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)]
+    kept = tuner.prune(cfgs)
+    assert len(kept) == max(tuner.keep_min, int(len(cfgs) * tuner.keep_fraction + 0.999)) < len(cfgs)
+
+
+def test_an_attention_model_file_still_loads_and_a_foreign_feature_set_does_not(tmp_path):
+    m = costmodel.CostModel.load(os.path.join(AttnTunner(MI355X(), _meta(4, 32, 2048)).cache_path, "costmodel_attn.json"))
+    assert m.names == costmodel.FEATURES
+    with pytest.raises(ValueError):
+        costmodel.CostModel.from_dict({"features": ["matrix", "moon_phase"], "weights": [1.0, 2.0]})
