@@ -102,7 +102,7 @@ def measured_traffic(cfg, algorithmic_bytes):
 
 def cpu_baseline_retnet():
     """The oracle's fp32 torch RetNet forward (retnet_ref) and closed-form backward (retnet_bwd_ref) on the host cores at
-    BASELINE config 4's shape (B4 H8 S2048, d_qk 256, d_v 512, decay mask), every (batch, head) slice once, one batch
+    the RetNet backward shape of the reference's headline configurations (B4 H8 S2048, d_qk 256, d_v 512, decay mask), every (batch, head) slice once, one batch
     (8 heads) at a time."""
     import torch
     from oracle import ref_op
