@@ -27,6 +27,9 @@ RUNS_WITH_UNITS = {
     "attn_b4h32q2048k2048_c0_128_128_units.txt": ((4, 32, 2048, 2048), False),
     "attn_b4h32q2048k2048_c1_128_128_units.txt": ((4, 32, 2048, 2048), True),
     "attn_b1h32q256k16384_c0_128_128_units.txt": ((1, 32, 256, 16384), False),
+    # searched in full once more after the operand rings changed their wait order: the causal winner moved to 512-row blocks
+    "attn_b4h32q2048k2048_c0_128_128_units2.txt": ((4, 32, 2048, 2048), False),
+    "attn_b4h32q2048k2048_c1_128_128_units2.txt": ((4, 32, 2048, 2048), True),
 }
 EXPORTS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "costmodel_export")
 
