@@ -104,7 +104,28 @@ def prune_stale(build_dir=None):
     return removed
 
 
+def prune_candidates(extra=(), build_dir=None):
+    """Delete every library that is not in the shipping set (+ ``extra``): what a tuning run over a whole search space
+    leaves behind.  Returns the number of files removed."""
+    root = build_dir or codegen.DEFAULT_BUILD_DIR
+    keep = {os.path.basename(codegen.library_path(c, build_dir))[:-3] for c in shipping_set(extra=extra)}
+    removed = 0
+    for op in sorted(os.listdir(root)) if os.path.isdir(root) else []:
+        if op not in codegen.SOURCE_DIRS or op == "ret_recurrent":
+            continue
+        for dirpath, _, files in os.walk(os.path.join(root, op)):
+            for fn in files:
+                stem = fn[:-len(".usage.json")] if fn.endswith(".usage.json") else os.path.splitext(fn)[0]
+                if fn.endswith((".so", ".hip", ".log", ".usage.json")) and stem not in keep:
+                    os.remove(os.path.join(dirpath, fn))
+                    removed += 1
+    return removed
+
+
 if __name__ == "__main__":
     if "--prune" in sys.argv:
         print("removed", prune_stale(), "stale files")
+    if "--prune-candidates" in sys.argv:          # keep the shipping set and the parity suite's variants only
+        from . import prebuilt_extra
+        print("removed", prune_candidates(extra=prebuilt_extra.parity_configs()), "files of libraries outside the shipping set")
     build_all(force="--force" in sys.argv)

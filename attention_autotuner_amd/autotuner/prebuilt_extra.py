@@ -40,10 +40,24 @@ STANDALONE_BENCH_TILES = [(64, 128, 64, 256, 2), (64, 128, 32, 256, 2), (64, 64,
                           (128, 256, 64, 512, 2), (128, 128, 64, 256, 3), (128, 128, 32, 256, 3)]
 
 
+def persistent_graph_config():
+    """A 256-row, 512-thread attention configuration with one row group per wave: takes the persistent-block kernel on
+    short rows (the graph-capture test of that kernel runs it)."""
+    return AttnConfig(256, 128, 128, 128, 128, 128, 2, 2, 512, True, waves_per_eu=2).set_fuse_type("register")
+
+
 def ret_register_wide():
     """The register-fused RetNet forward at d_qk 256, d_v 512 (the reference has this variant,
     csrc/kernels/retnet/regfuse/regfuse.h:267-340): 256 output accumulators per lane."""
     return RetConfig(128, 64, 256, 512, 256, 64, 1, 1, 1, 256, True, waves_per_eu=1).set_fuse_type("register")
+
+
+def ret_register_wide_buffered():
+    """The same kernel with a second buffer per stream: two K / mask buffers next to one V buffer on 64-row tiles, and every
+    stream double-buffered on 32-row tiles (one barrier per tile).  The run-time buffer parity and the copies threaded
+    between the matrix steps take other paths here than in the single-buffer build."""
+    return [RetConfig(128, 64, 256, 512, 256, 64, 2, 2, 1, 256, True, waves_per_eu=1).set_fuse_type("register"),
+            RetConfig(128, 32, 256, 512, 256, 32, 2, 2, 2, 256, True, waves_per_eu=1).set_fuse_type("register")]
 
 
 def ret_shared_wide_one_wave():
@@ -82,7 +96,9 @@ def parity_configs(arch=None):
             cfg.fuse_type = fuse
             if gfx950_space.forward_valid(cfg, arch):
                 out.append(cfg)
+    out.append(persistent_graph_config())
     out.append(ret_register_wide())
+    out += ret_register_wide_buffered()
     out.append(ret_shared_wide_one_wave())
     for t in RET_BWD_STORED_DS:
         out += [ret_bwd_stored_ds_config(*t), ret_bwd_stored_ds_config(*t[:5], 0)]      # and the same passes without it

@@ -330,7 +330,7 @@ def test_forward_replays_from_a_captured_graph():
 
 def test_persistent_forward_replays_from_a_captured_graph():
     """The same for a launch that takes the persistent-block kernel (more row blocks than the chip holds)."""
-    cfg = AttnConfig(256, 128, 128, 128, 128, 128, 2, 2, 512, True, waves_per_eu=2).set_fuse_type("register")
+    cfg = parity_matrix.persistent_graph_config()
     assert _persistent_ok(256, 128, 512, 2, 2, 2, 128, 128)
     q, k, v = (t.cuda() for t in _inputs(2, 130, 512, 256, 128, 128, seed=31))
     rt = Runtime(ARCH, cfg)

@@ -161,13 +161,15 @@ def test_non_square_and_every_prebuilt_variant():
     assert ran >= 4
 
 
-@pytest.mark.parametrize("which", ["register", "shared"])
+@pytest.mark.parametrize("which", ["register", "register-two-k-buffers", "register-all-double-buffered", "shared"])
 def test_one_wave_forward_with_256_accumulators_at_dqk256_dv512(which):
     """The register-fused kernel (and the LDS-fused one with four waves) holds a 32 x 512 fp32 output block per wave: all
     256 accumulation registers of a wave that has its SIMD to itself, rescaled in place when the lazy normaliser moves
     (the sums of |S| pass 256 within the first tiles here).  It is built without a byte of scratch and must be right
     for every way of handing over the mask."""
-    cfg = parity_matrix.ret_register_wide() if which == "register" else parity_matrix.ret_shared_wide_one_wave()
+    cfg = {"register": parity_matrix.ret_register_wide, "shared": parity_matrix.ret_shared_wide_one_wave,
+           "register-two-k-buffers": lambda: parity_matrix.ret_register_wide_buffered()[0],
+           "register-all-double-buffered": lambda: parity_matrix.ret_register_wide_buffered()[1]}[which]()
     assert gfx950_space.forward_valid(cfg, ARCH) and os.path.exists(codegen.library_path(cfg))
     report = [k for k in codegen.resource_usage(codegen.library_path(cfg)) if "ret_fwd_" in k["kernel"]]
     assert len(report) == 2 and all(k["scratch_bytes"] == 0 and k["agprs"] == 256 for k in report), report
