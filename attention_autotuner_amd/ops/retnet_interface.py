@@ -103,8 +103,9 @@ class RetNetAttn(torch.autograd.Function):
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)
         # The reference's kernel accumulates dQ into this fp32 scratch with atomics; the kernels here never
-        # touch it (dQ is produced directly), so a token buffer stands in for the [B,H,S_q,d_qk] tensor.
-        dq_accum = torch.zeros(1, device=q.device, dtype=torch.float32)
+        # touch it (dQ is produced directly), so a token buffer stands in for the [B,H,S_q,d_qk] tensor -- uninitialised:
+        # zeroing it would put a fill kernel between the forward's and the backward's launches for nothing.
+        dq_accum = torch.empty(1, device=q.device, dtype=torch.float32)
         arrays = [q, k, v, mask, do, r, dq, dk, dv, dq_accum]
         tuner = RetBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal is None or bool(ctx.causal),
                              mask_mode="scan" if ctx.mask_scan is not None else None)
