@@ -6,6 +6,7 @@ python/tests/attntuner_demo.py:186-192 and python/tests/test_retbwdtunner.py:88-
     python -m attention_autotuner_amd.benchmarks.tune ret_bwd B H Sq Sk dqk dv [--causal]
     python -m attention_autotuner_amd.benchmarks.tune attn_bwd B H Sq Sk dqk dv [--causal]
     python -m attention_autotuner_amd.benchmarks.tune ret|ret_bwd ... --decay      (decay mask built in registers)
+    python -m attention_autotuner_amd.benchmarks.tune ... --input-path DIR       (q.pt, k.pt, v.pt, mask.pt, do.pt instead of synthetic tensors)
 
 Writes the best configuration into the tuning cache, the per-candidate log next to it, and prints a
 one-line JSON summary.  ``--compile-only`` builds every candidate library (no GPU needed) so that a
@@ -63,6 +64,31 @@ def make_tensors(op, b, h, sq, sk, dqk, dv, device, seed=0):
     return [q, k, v, mask, do, r, dq, dk, dv_, acc]
 
 
+def load_inputs(arrays, op, input_path, device):
+    """Replace the synthetic q, k, v (and the RetNet mask, and dO where there is one) by tensors stored under ``input_path``
+    as q.pt, k.pt, v.pt, mask.pt, do.pt -- the layout of the reference's tuner driver
+    (reference python/tests/attntuner_demo.py:38-43: a singleton dimension 1 is dropped, the leading [B, H, S, d] corner is
+    used).  Files are read with ``weights_only=True``: plain tensors only, nothing in them is executed.  A file that is
+    absent keeps the synthetic tensor."""
+    def corner(name, like):
+        path = os.path.join(input_path, name)
+        if not os.path.exists(path):
+            return like
+        t = torch.load(path, map_location="cpu", weights_only=True)
+        if t.dim() == like.dim() + 1 and t.shape[1] == 1:
+            t = t.squeeze(1)
+        if t.dim() != like.dim() or any(a < b for a, b in zip(t.shape, like.shape)):
+            raise ValueError(f"{path}: shape {tuple(t.shape)} does not cover the problem's {tuple(like.shape)}")
+        t = t[tuple(slice(0, n) for n in like.shape)].to(like.dtype).contiguous()
+        return t.to(device) if device != "meta" else like
+    arrays[0], arrays[1], arrays[2] = corner("q.pt", arrays[0]), corner("k.pt", arrays[1]), corner("v.pt", arrays[2])
+    if op in ("ret", "ret_bwd"):
+        arrays[3] = corner("mask.pt", arrays[3])
+    if op in ("ret_bwd", "attn_bwd"):
+        arrays[4] = corner("do.pt", arrays[4])
+    return arrays
+
+
 def flops(op, b, h, sq, sk, dqk, dv, causal):
     f = 2.0 * b * h * sq * sk * ((dqk + dv) if op in ("attn", "ret") else (3 * dqk + 2 * dv))
     return f / 2 if (causal and op in ("attn", "attn_bwd")) else f      # RetNet rates are quoted on the dense count
@@ -78,12 +104,15 @@ def main(argv=None):
     ap.add_argument("--log-dir", default=DEFAULT_LOG_DIR)
     ap.add_argument("--cache-dir", default=None, help="where the best configuration is recorded (default: the package's tuning cache)")
     ap.add_argument("--cost-model", default=None, help="a fitted cost model (JSON): only the candidates it ranks best are built and timed")
+    ap.add_argument("--input-path", default="", help="directory with q.pt, k.pt, v.pt (mask.pt, do.pt): tune on these tensors instead of synthetic ones")
     args = ap.parse_args(argv)
     b, h, sq, sk, dqk, dv = args.dims
     arch = MI355X()
     cls = {"attn": AttnTunner, "ret": RetTunner, "ret_bwd": RetBwdTunner, "attn_bwd": AttnBwdTunner}[args.op]
     device = "meta" if args.compile_only else "cuda"
     arrays = make_tensors(args.op, b, h, sq, sk, dqk, dv, device)
+    if args.input_path:
+        arrays = load_inputs(arrays, args.op, args.input_path, device)
     if args.decay:
         if args.op not in ("ret", "ret_bwd"):
             ap.error("--decay applies to ret and ret_bwd")
