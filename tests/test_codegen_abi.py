@@ -335,3 +335,20 @@ def test_a_build_whose_compiler_uses_the_numbered_accumulation_registers_is_reje
     # the shipped one-wave configuration of the same kernel passes the check
     fine = gfx950_space.default_forward_config("ret", 256, 512, ARCH)
     assert fine.waves_per_eu == 1 and fine.fuse_type == "register" and os.path.exists(codegen.library_path(fine))
+
+
+def test_no_cached_winner_keeps_its_working_set_in_scratch():
+    """Every configuration in the shipped tuning cache is built, carries the compiler's report, and none of the kernels a
+    launch of it can take keeps more than the tolerated few dwords in scratch memory.  (The paired causal variant of the
+    attention forward is the one exception the wrapper handles itself: it is only launched from a build in which the
+    runtime reports no scratch for it.)"""
+    from attention_autotuner_amd.autotuner import prebuilt
+    cached = prebuilt.cached_configs()
+    assert len(cached) >= 18
+    for cfg in cached:
+        usage = codegen.resource_usage(codegen.library_path(cfg))
+        assert usage, cfg
+        def launched(name):
+            flags = codegen.template_bools(name)
+            return not ("flashattn_fwd_regfuse" in name and len(flags) == 5 and flags[4])        # <..., PIPE, CAUSAL, SPLIT, PERSIST, PAIR>
+        assert codegen.spilling_kernels(usage, launched) == [], (str(cfg), codegen.spilling_kernels(usage, launched))
