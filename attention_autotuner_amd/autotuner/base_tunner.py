@@ -15,8 +15,10 @@ an on-disk cache first -- with these deliberate changes:
 """
 import ctypes
 import json
+import math
 import os
 import pprint
+import re
 import time
 
 import torch
@@ -192,6 +194,45 @@ class BaseTunner:
                 continue                                  # missing or corrupt cache file: fall through
             if self._fits_problem(cfg):
                 _memo[self._memo_key()] = cfg
+                return cfg
+        return None
+
+    nearest_limit = 12.0       # e.g. one length and the row count a factor 16 apart
+
+    def nearest_cached(self):
+        """The tuned configuration of the closest problem this cache holds for the same operator, head sizes and mask
+        walk whose tiles also divide this problem's lengths, or None.  For callers that do not want a tuning run on a
+        miss: the reference keys its cache by the two head sizes alone (python/autotuner/base_tunner.py:190-208), i.e. it always launches
+        whatever was tuned first; here the entry of the nearest lengths and block count stands in, and only then the
+        built-in default.  Distance in octaves: lengths count twice (they decide tile sizes and the kv split), the number
+        of rows in the launch once (it decides how many blocks a CU gets); an entry more than ``nearest_limit`` away says
+        nothing about this problem."""
+        s = self.problem_shape
+        stem = os.path.basename(self._cache_file()).split("_b%d" % s["B"])[0]
+        pat = re.compile(re.escape(stem) + r"_b(\d+)h(\d+)q(\d+)k(\d+)_c%d\.json$" % int(self.causal))
+        try:
+            names = sorted(os.listdir(self.cache_path))
+        except OSError:
+            return None
+        found = []
+        for name in names:
+            m = pat.match(name)
+            if not m:
+                continue
+            b, h, sq, sk = (int(x) for x in m.groups())
+            far = 2 * abs(math.log2(sq / s["Sq"])) + 2 * abs(math.log2(sk / s["Sk"])) + \
+                abs(math.log2((b * h * sq) / (s["B"] * s["H"] * s["Sq"])))
+            if far <= self.nearest_limit:
+                found.append((far, name))
+        for _, name in sorted(found):
+            try:
+                with open(os.path.join(self.cache_path, name)) as f:
+                    dd = json.load(f)
+                cfg = supported_configs[dd["operation"]].from_dict(dd)
+            except (OSError, ValueError, KeyError):
+                continue
+            if self._fits_problem(cfg):
+                _memo[self._memo_key()] = cfg             # this process keeps launching it for this problem
                 return cfg
         return None
 

@@ -1,7 +1,7 @@
 """End-to-end RetNet benchmark through the public operator (forward and forward+backward), against
 the same math in plain PyTorch on the GPU (counterpart of reference python/benchmarks/bench_retnet.py:32-116).
 
-    python -m attention_autotuner_amd.benchmarks.bench_retnet [--dims 64 128 256] [--dv 512]
+    python -m attention_autotuner_amd.benchmarks.bench_retnet [--dims 64 128 192 256] [--dv 512]
 """
 import argparse
 
@@ -47,7 +47,7 @@ def run(batch, heads, seq_q, seq_k, dim_qk, dim_v, arch, causal):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--dims", type=int, nargs="*", default=[64, 128, 256])
+    ap.add_argument("--dims", type=int, nargs="*", default=[64, 128, 192, 256])
     ap.add_argument("--dv", type=int, default=None, help="value head size (default: same as d_qk)")
     ap.add_argument("--shape", type=int, nargs=4, default=[4, 8, 2048, 2048], metavar=("B", "H", "Sq", "Sk"))
     ap.add_argument("--causal", action="store_true", help="promise a lower-triangular mask so tiles above the diagonal are skipped")

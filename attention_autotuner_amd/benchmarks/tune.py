@@ -9,8 +9,9 @@ python/tests/attntuner_demo.py:186-192 and python/tests/test_retbwdtunner.py:88-
     python -m attention_autotuner_amd.benchmarks.tune ... --input-path DIR       (q.pt, k.pt, v.pt, mask.pt, do.pt instead of synthetic tensors)
 
 Writes the best configuration into the tuning cache, the per-candidate log next to it, and prints a
-one-line JSON summary.  ``--compile-only`` builds every candidate library (no GPU needed) so that a
-later run on a machine without spare CPU time only has to time them.
+one-line JSON summary.  ``--compile-only`` builds the candidate libraries a tuning run would time (no GPU
+needed; all of them under AAT_TUNE_PRUNE=0) so that a later run on a machine without spare CPU time only
+has to time them.
 """
 import argparse
 import json
@@ -129,7 +130,7 @@ def main(argv=None):
         from ..autotuner.costmodel import CostModel
         tuner.cost_model = CostModel.load(args.cost_model)
     if args.compile_only:
-        cfgs = [c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)]
+        cfgs = tuner.prune([c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)])   # what a tuning run would time
         t0 = time.time()
         libs = codegen.compile_parallel(cfgs, arch, timeout=300)
         print(json.dumps({"op": args.op, "candidates": len(cfgs), "built": sum(l is not None for l in libs),

@@ -352,3 +352,36 @@ def test_no_cached_winner_keeps_its_working_set_in_scratch():
             flags = codegen.template_bools(name)
             return not ("flashattn_fwd_regfuse" in name and len(flags) == 5 and flags[4])        # <..., PIPE, CAUSAL, SPLIT, PERSIST, PAIR>
         assert codegen.spilling_kernels(usage, launched) == [], (str(cfg), codegen.spilling_kernels(usage, launched))
+
+
+def test_without_tuning_a_miss_launches_the_entry_of_the_nearest_problem(tmp_path, monkeypatch):
+    """AAT_TUNE_ON_MISS=0: same operator, head sizes and mask walk; nearest lengths first; tiles must divide the problem."""
+    from attention_autotuner_amd.ops import _resolve
+    base_tunner._memo.clear()
+    near = AttnConfig(Br=128, Bc=64, Kd=128, D=128, Nthreads=256)
+    far = AttnConfig(Br=256, Bc=128, Kd=128, D=128, Nthreads=256)
+    other_walk = AttnConfig(Br=64, Bc=64, Kd=128, D=128, Nthreads=128)
+
+    def entry(name, cfg):
+        with open(tmp_path / name, "w") as f:
+            json.dump(cfg.to_dict(), f)
+    entry("best_config_attention_MI355X_128_128_b4h32q2048k2048_c0.json", near)
+    entry("best_config_attention_MI355X_128_128_b1h32q256k16384_c0.json", far)
+    entry("best_config_attention_MI355X_128_128_b4h32q1024k1024_c1.json", other_walk)
+    entry("best_config_attention_MI355X_64_64_b4h32q1024k1024_c0.json", other_walk)
+    entry("best_config_attention_bwd_MI355X_128_128_b4h32q1024k1024_c0.json", other_walk)
+    monkeypatch.setenv("AAT_TUNE_ON_MISS", "0")
+    default = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
+
+    def resolved(**kw):
+        t = AttnTunner(ARCH, _meta(**kw), causal=False)
+        t.cache_path = str(tmp_path)
+        assert t.check_cache() is None
+        return _resolve.resolve(t, lambda: default), t
+
+    cfg, t = resolved(sq=1024, sk=1024)
+    assert cfg == near and t.check_cache() == near        # and the process remembers it for this problem
+    assert resolved(sq=256, sk=8192)[0] == far
+    assert resolved(sq=384, sk=8192)[0] == near           # 256-row blocks do not divide 384 rows: the next nearest
+    assert resolved(sq=64, sk=2048)[0] == default         # the one entry within reach does not fit: the built-in default
+    base_tunner._memo.clear()
