@@ -31,7 +31,8 @@ _PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)),
 DEFAULT_CACHE_DIR = os.environ.get("AAT_CACHE_DIR", os.path.join(_PKG, "cache"))
 FAILED = 1e8                          # latency recorded for a configuration that errored at run time
 
-_memo = {}                            # in-process memo of resolved best configs
+_memo = {}                            # in-process memo of resolved best configs (and of the operators' launch plans)
+_UNSET = object()
 
 
 class CompileResult:
@@ -61,6 +62,7 @@ class BaseTunner:
         self.Br_list = [32, 64, 128, 256]
         self.Bc_list = [32, 64, 128, 256]
         self.cache_path = DEFAULT_CACHE_DIR
+        self.cost_model_dir = self.cache_path     # a caller that records its results elsewhere still prunes with the shipped model
         self.build_dir = None
         self.verbose = os.environ.get("AAT_VERBOSE", "0") == "1"
         q, k, v = torch_array[0], torch_array[1], torch_array[2]
@@ -248,7 +250,25 @@ class BaseTunner:
         several variants: causal or not, decay mask or mask tensor)."""
         return True
 
-    cost_model = None          # a fitted costmodel.CostModel: tune() then times only its best-ranked candidates
+    # A fitted costmodel.CostModel: tune() then times only its best-ranked candidates.  Subclasses name a model file
+    # next to the tuning cache; it is read when first asked for, not when the tuner is built: an operator builds a
+    # tuner on every call of a problem it has not launched before, and only a tuning run needs the model.
+    cost_model_file = None
+    _cost_model = _UNSET
+
+    @property
+    def cost_model(self):
+        if self._cost_model is _UNSET:
+            self._cost_model = self._shipped_cost_model()
+        return self._cost_model
+
+    @cost_model.setter
+    def cost_model(self, model):
+        self._cost_model = model
+
+    def _shipped_cost_model(self):
+        return None
+
     keep_fraction = 0.35       # ... this share of them (at least keep_min)
     keep_min = 8
 

@@ -55,6 +55,9 @@ class Runtime:
         self.config = config
         self.tmp_dir = tmp_dir
         self.libname = libname
+        self._lib = None                  # the loaded library and the workspace each problem shape needs, kept between calls
+        self._need = {}
+        self._asks = {}
         if self.libname is None:
             self.libname = self.compile()
         if self.libname is None:
@@ -70,7 +73,12 @@ class Runtime:
         return os.path.join(self.tmp_dir or codegen.DEFAULT_BUILD_DIR, self.libname)
 
     def workspace_size(self, B, H, Sq, Sk):
-        return int(library.load(self._path(), self.config.operation).workspace_size(B, H, Sq, Sk))
+        size = self._asks.get((B, H, Sq, Sk))
+        if size is None:
+            if self._lib is None:
+                self._lib = library.load(self._path(), self.config.operation)
+            size = self._asks[(B, H, Sq, Sk)] = int(self._lib.workspace_size(B, H, Sq, Sk))
+        return size
 
     def apply(self, torch_array, device=None, softmax_scale=None, causal=False, workspace=None, lse=None, decay=False):
         """``lse`` (attention forward only): fp32 [B,H,S_q] tensor that receives the log-sum-exp of every row.
@@ -79,22 +87,33 @@ class Runtime:
         q, k = torch_array[0], torch_array[1]
         if not q.is_cuda:
             raise KernelLaunchError("kernel libraries run on the GPU only; got CPU tensors")
-        B, H, Sq, Sk = int(q.shape[0]), int(q.shape[1]), int(q.shape[2]), int(k.shape[2])
+        B, H, Sq, Sk = q.shape[0], q.shape[1], q.shape[2], k.shape[2]
         op = self.config.operation
-        lib = library.load(self._path(), op)
-        need = _wanted(self.config, int(lib.workspace_size(B, H, Sq, Sk)), B, H, Sq, Sk)
+        lib = self._lib
+        if lib is None:
+            lib = self._lib = library.load(self._path(), op)
+        need = self._need.get((B, H, Sq, Sk))               # a property of the library and the problem: asked once
+        if need is None:
+            need = self._need[(B, H, Sq, Sk)] = _wanted(self.config, int(lib.workspace_size(B, H, Sq, Sk)), B, H, Sq, Sk)
         if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
             workspace = _grown(workspace, need, q.device, keep=causal == "scanned")
-        ws_ptr = ctypes.c_void_p(workspace.data_ptr() if workspace is not None else 0)
-        ws_bytes = ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0)
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
         if op in library.SCALED_OPS:
             scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(q.shape[-1])
-            extra = [ctypes.c_float(scale), ctypes.c_int(int(bool(causal)))]
+            extra = (scale, int(bool(causal)))
         else:
-            extra = [ctypes.c_int(mask_mode(causal))]
-        with torch.cuda.device(q.device):
-            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-            ptrs = [ctypes.c_void_p(t.data_ptr()) for t in torch_array]
+            extra = (mask_mode(causal),)
+        # the prototypes are set (library.py), so plain integers convert; the launch goes to the stream that is current
+        # on the tensors' device, with that device current
+        index = q.device.index
+        other = index != torch.cuda.current_device()
+        if other:
+            previous = torch.cuda.current_device()
+            torch.cuda.set_device(index)
+        try:
+            stream = torch._C._cuda_getCurrentRawStream(index)
+            ptrs = [t.data_ptr() for t in torch_array]
             if decay:
                 if op not in library.DECAY_OPS:
                     raise KernelLaunchError("only the RetNet operators have a decay-mask variant")
@@ -102,9 +121,12 @@ class Runtime:
             elif lse is not None:
                 if op != "attn":
                     raise KernelLaunchError("only the attention forward writes a log-sum-exp")
-                rc = lib.kernel_entry_lse(*ptrs, ctypes.c_void_p(lse.data_ptr()), B, H, Sq, Sk, *extra, ws_ptr, ws_bytes, stream)
+                rc = lib.kernel_entry_lse(*ptrs, lse.data_ptr(), B, H, Sq, Sk, *extra, ws_ptr, ws_bytes, stream)
             else:
                 rc = lib.kernel_entry_ex(*ptrs, B, H, Sq, Sk, *extra, ws_ptr, ws_bytes, stream)
+        finally:
+            if other:
+                torch.cuda.set_device(previous)
         if rc != 0:
             raise KernelLaunchError(f"{op}:{self.config} failed with code {rc}: {_ERRORS.get(rc, 'HIP error')}")
         return rc

@@ -66,10 +66,13 @@ class _ForwardTunner(BaseTunner):
         return super().tune(*a, **kw)
 
 
-def _shipped_cost_model(arch, cache_path, name):
-    """The fitted model ``name`` next to the tuning cache, or None (no file, another platform, AAT_TUNE_PRUNE=0)."""
-    path = os.path.join(cache_path, name)
-    if not (_is_rocm(arch) and os.environ.get("AAT_TUNE_PRUNE", "1") != "0" and os.path.exists(path)):
+def _shipped_cost_model(self):
+    """The fitted model ``cost_model_file`` next to the tuning cache, or None (no file, another platform,
+    AAT_TUNE_PRUNE=0)."""
+    if self.cost_model_file is None:
+        return None
+    path = os.path.join(self.cost_model_dir, self.cost_model_file)
+    if not (_is_rocm(self.arch) and os.environ.get("AAT_TUNE_PRUNE", "1") != "0" and os.path.exists(path)):
         return None
     from .costmodel import CostModel
     try:
@@ -80,12 +83,13 @@ def _shipped_cost_model(arch, cache_path, name):
 
 class AttnTunner(_ForwardTunner):
     operation = "attn"
+    # the space has a few hundred candidates: with a fitted cost model next to the tuning cache, only the
+    # third it ranks best is built and timed (AAT_TUNE_PRUNE=0: time everything, as the reference does)
+    cost_model_file = "costmodel_attn.json"
+    _shipped_cost_model = _shipped_cost_model
 
     def __init__(self, arch, torch_array, causal=False, softmax_scale=None):
         super().__init__(arch, torch_array, "attention", causal=causal, softmax_scale=softmax_scale)
-        # the space has a few hundred candidates: with a fitted cost model next to the tuning cache, only the
-        # third it ranks best is built and timed (AAT_TUNE_PRUNE=0: time everything, as the reference does)
-        self.cost_model = _shipped_cost_model(arch, self.cache_path, "costmodel_attn.json")
 
     def _ex_args(self):
         scale = self.softmax_scale
@@ -96,18 +100,20 @@ class AttnTunner(_ForwardTunner):
 
 class RetTunner(_ForwardTunner):
     operation = "ret"
+    cost_model_file = "costmodel_ret.json"
+    _shipped_cost_model = _shipped_cost_model
 
     def __init__(self, arch, torch_array, causal=False, decay=False, mask_mode=None):
         super().__init__(arch, torch_array, "retnet", causal=causal or decay, decay=decay, mask_mode=mask_mode)
-        self.cost_model = _shipped_cost_model(arch, self.cache_path, "costmodel_ret.json")
 
 
 class RetBwdTunner(BaseTunner):
     operation = "ret_bwd"
+    cost_model_file = "costmodel_ret_bwd.json"
+    _shipped_cost_model = _shipped_cost_model
 
     def __init__(self, arch, torch_array, causal=False, decay=False, mask_mode=None):
         super().__init__(arch, torch_array, "retnet_bwd", causal=causal or decay, decay=decay, mask_mode=mask_mode)
-        self.cost_model = _shipped_cost_model(arch, self.cache_path, "costmodel_ret_bwd.json")
         if _is_rocm(arch):
             self.Br_list = list(getattr(gfx950_space, "BWD_BR_LIST", (64, 128)))
             self.Bc_list = list(getattr(gfx950_space, "BWD_BC_LIST", (32, 64, 128)))

@@ -1,6 +1,9 @@
 """Shared by the two operator front ends: pick the configuration to launch."""
 import os
 
+from ..autotuner import base_tunner
+from ..autotuner.runtime import Runtime
+
 _PKG = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
 DEFAULT_LOG_DIR = os.environ.get("AAT_LOG_DIR", os.path.join(_PKG, "logs"))
 
@@ -19,3 +22,18 @@ def resolve(tuner, default_factory):
     if tune_on_miss():
         return tuner.tune(log_path=DEFAULT_LOG_DIR)
     return tuner.nearest_cached() or default_factory()
+
+
+def planned(key, make_tuner, default_factory):
+    """``(configuration, Runtime)`` for the problem ``key`` (operator, shapes, mask walk): resolved through a tuner the
+    first time this process meets the problem and kept in the tuners' own memo, so that every later call costs one
+    dictionary lookup instead of a tuner, a cache-file name and a library path (the reference reads its JSON cache,
+    python/autotuner/base_tunner.py:197-206, and opens the library, python/autotuner/runtime.py:74-82, on every call;
+    its README.md:113 lists "the performance of python interface?" as open)."""
+    k = ("plan", base_tunner.DEFAULT_CACHE_DIR, tune_on_miss()) + key
+    plan = base_tunner._memo.get(k)
+    if plan is None:
+        tuner = make_tuner()
+        cc = resolve(tuner, default_factory)
+        plan = base_tunner._memo[k] = (cc, Runtime(tuner.arch, cc))
+    return plan

@@ -14,9 +14,8 @@ import torch
 
 from ..arch import Arch
 from ..autotuner import gfx950_space
-from ..autotuner.runtime import Runtime
 from ..autotuner.tunner import AttnBwdTunner, AttnTunner
-from ._resolve import resolve
+from ._resolve import planned
 
 REFERENCE_SOFTMAX_SCALE = 0.125
 
@@ -41,11 +40,13 @@ class MultiHeadAttnFunc(torch.autograd.Function):
             softmax_scale = 1.0 / math.sqrt(key_dim)
 
         o = torch.empty(batch_size, nheads, seqlen_q, head_dim, device=q.device, dtype=q.dtype)
-        tuner = AttnTunner(arch=device_type, torch_array=[q, k, v, o], causal=causal, softmax_scale=softmax_scale)
-        cc = resolve(tuner, lambda: gfx950_space.default_forward_config("attn", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+        causal = bool(causal)
+        _, rt = planned(("attn", device_type.name, batch_size, nheads, seqlen_q, seqlen_k, key_dim, head_dim, causal),
+                        lambda: AttnTunner(arch=device_type, torch_array=[q, k, v, o], causal=causal, softmax_scale=softmax_scale),
+                        lambda: gfx950_space.default_forward_config("attn", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
         needs_grad = any(ctx.needs_input_grad[:3])
         lse = torch.empty(batch_size, nheads, seqlen_q, device=q.device, dtype=torch.float32) if needs_grad else None
-        Runtime(device_type, cc).apply([q, k, v, o], softmax_scale=softmax_scale, causal=causal, lse=lse)
+        rt.apply([q, k, v, o], softmax_scale=softmax_scale, causal=causal, lse=lse)
         if needs_grad:
             ctx.save_for_backward(q, k, v, o, lse)
         ctx.device_type = device_type
@@ -63,12 +64,13 @@ class MultiHeadAttnFunc(torch.autograd.Function):
         assert do.dtype == torch.float16 and do.shape == o.shape
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         arrays = [q, k, v, o, do, lse, dq, dk, dv]
-        tuner = AttnBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal, softmax_scale=ctx.softmax_scale)
         try:
-            cc = resolve(tuner, lambda: gfx950_space.default_attn_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+            _, rt = planned(("attn_bwd", device_type.name, q.shape[0], q.shape[1], seqlen_q, seqlen_k, key_dim, head_dim, ctx.causal),
+                            lambda: AttnBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal, softmax_scale=ctx.softmax_scale),
+                            lambda: gfx950_space.default_attn_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
         except gfx950_space.NoValidConfigError as e:      # e.g. d_v = 512: dK and dV do not fit one wave's registers
             raise NotImplementedError(f"attention backward: {e}") from e
-        Runtime(device_type, cc).apply(arrays, softmax_scale=ctx.softmax_scale, causal=ctx.causal)
+        rt.apply(arrays, softmax_scale=ctx.softmax_scale, causal=ctx.causal)
         return dq, dk, dv, None, None, None
 
 

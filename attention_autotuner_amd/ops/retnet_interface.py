@@ -25,7 +25,7 @@ from ..arch import Arch
 from ..autotuner import gfx950_space
 from ..autotuner.runtime import Runtime
 from ..autotuner.tunner import RetTunner, RetBwdTunner
-from ._resolve import resolve
+from ._resolve import planned
 
 
 def retnet_mask_scan(mask, device_type: Arch):
@@ -70,10 +70,10 @@ class RetNetAttn(torch.autograd.Function):
         if reused is not None:
             causal = None
         # ... but a tuning run on a cache miss times and verifies its candidates in the mode launched here, on this mask
-        tuner = RetTunner(arch=device_type, torch_array=arrays, causal=causal is None or bool(causal),
-                          mask_mode="scan" if causal is None else None)
-        cc = resolve(tuner, lambda: gfx950_space.default_forward_config("ret", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        rt = Runtime(device_type, cc)
+        walk, mode = causal is None or bool(causal), "scan" if causal is None else None
+        _, rt = planned(("ret", device_type.name, batch_size, nheads, seqlen_q, seqlen_k, key_dim, head_dim, walk, mode),
+                        lambda: RetTunner(arch=device_type, torch_array=arrays, causal=walk, mask_mode=mode),
+                        lambda: gfx950_space.default_forward_config("ret", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
         scan = None
         if reused is not None:
             scan = reused
@@ -107,13 +107,14 @@ class RetNetAttn(torch.autograd.Function):
         # zeroing it would put a fill kernel between the forward's and the backward's launches for nothing.
         dq_accum = torch.empty(1, device=q.device, dtype=torch.float32)
         arrays = [q, k, v, mask, do, r, dq, dk, dv, dq_accum]
-        tuner = RetBwdTunner(arch=device_type, torch_array=arrays, causal=ctx.causal is None or bool(ctx.causal),
-                             mask_mode="scan" if ctx.mask_scan is not None else None)
-        cc = resolve(tuner, lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+        walk, mode = ctx.causal is None or bool(ctx.causal), "scan" if ctx.mask_scan is not None else None
+        _, rt = planned(("ret_bwd", device_type.name, batch_size, nheads, seqlen_q, seqlen_k, key_dim, head_dim, walk, mode),
+                        lambda: RetBwdTunner(arch=device_type, torch_array=arrays, causal=walk, mask_mode=mode),
+                        lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
         if ctx.mask_scan is not None:
-            Runtime(device_type, cc).apply(arrays, causal="scanned", workspace=ctx.mask_scan)
+            rt.apply(arrays, causal="scanned", workspace=ctx.mask_scan)
         else:
-            Runtime(device_type, cc).apply(arrays, causal=bool(ctx.causal))
+            rt.apply(arrays, causal=bool(ctx.causal))
         return dq, dk, dv, None, None, None
 
 
@@ -155,9 +156,10 @@ class RetNetDecayAttn(torch.autograd.Function):
         o = torch.empty(batch_size, nheads, seqlen_q, head_dim, device=q.device, dtype=torch.float16)
         r = torch.empty(batch_size, nheads, seqlen_q, device=q.device, dtype=torch.float32)
         arrays = [q, k, v, lg, o, r]
-        tuner = RetTunner(arch=device_type, torch_array=arrays, decay=True)
-        cc = resolve(tuner, lambda: gfx950_space.default_forward_config("ret", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        Runtime(device_type, cc).apply(arrays, decay=True)
+        _, rt = planned(("ret_decay", device_type.name, batch_size, nheads, seqlen_q, seqlen_k, key_dim, head_dim),
+                        lambda: RetTunner(arch=device_type, torch_array=arrays, decay=True),
+                        lambda: gfx950_space.default_forward_config("ret", key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+        rt.apply(arrays, decay=True)
         ctx.save_for_backward(q, k, v, lg, r)
         ctx.device_type = device_type
         return o
@@ -171,9 +173,10 @@ class RetNetDecayAttn(torch.autograd.Function):
         do = do.contiguous()
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         arrays = [q, k, v, lg, do, r, dq, dk, dv]
-        tuner = RetBwdTunner(arch=device_type, torch_array=arrays, decay=True)
-        cc = resolve(tuner, lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
-        Runtime(device_type, cc).apply(arrays, decay=True)
+        _, rt = planned(("ret_bwd_decay", device_type.name, q.shape[0], q.shape[1], seqlen_q, seqlen_k, key_dim, head_dim),
+                        lambda: RetBwdTunner(arch=device_type, torch_array=arrays, decay=True),
+                        lambda: gfx950_space.default_backward_config(key_dim, head_dim, device_type, seqlen_q, seqlen_k))
+        rt.apply(arrays, decay=True)
         return dq, dk, dv, None, None
 
 

@@ -342,16 +342,28 @@ def test_no_cached_winner_keeps_its_working_set_in_scratch():
     launch of it can take keeps more than the tolerated few dwords in scratch memory.  (The paired causal variant of the
     attention forward is the one exception the wrapper handles itself: it is only launched from a build in which the
     runtime reports no scratch for it.)"""
-    from attention_autotuner_amd.autotuner import prebuilt
-    cached = prebuilt.cached_configs()
-    assert len(cached) >= 18
-    for cfg in cached:
+    import glob
+    from attention_autotuner_amd.autotuner.configs import supported_configs
+    entries = sorted(glob.glob(os.path.join(base_tunner.DEFAULT_CACHE_DIR, "best_config_*.json")))
+    assert len(entries) >= 18
+    for path in entries:
+        with open(path) as f:
+            dd = json.load(f)
+        cfg = supported_configs[dd["operation"]].from_dict(dd)
+        decay = "_decay_" in os.path.basename(path)           # the entry of a decay-mask problem launches the DECAY kernels
         usage = codegen.resource_usage(codegen.library_path(cfg))
         assert usage, cfg
+
         def launched(name):
             flags = codegen.template_bools(name)
-            return not ("flashattn_fwd_regfuse" in name and len(flags) == 5 and flags[4])        # <..., PIPE, CAUSAL, SPLIT, PERSIST, PAIR>
-        assert codegen.spilling_kernels(usage, launched) == [], (str(cfg), codegen.spilling_kernels(usage, launched))
+            if "flashattn_fwd_regfuse" in name and len(flags) == 5:          # <..., PIPE, CAUSAL, SPLIT, PERSIST, PAIR>
+                return not flags[4]
+            if "ret_fwd" in name and flags:                                  # <..., DECAY>
+                return flags[-1] == decay
+            if "ret_bwd_chain" in name and len(flags) == 2:                  # <..., PASS, WPE, DECAY, DS_OUT>
+                return flags[0] == decay
+            return True
+        assert codegen.spilling_kernels(usage, launched) == [], (os.path.basename(path), codegen.spilling_kernels(usage, launched))
 
 
 def test_without_tuning_a_miss_launches_the_entry_of_the_nearest_problem(tmp_path, monkeypatch):
