@@ -1,6 +1,8 @@
 """Shared by the two operator front ends: pick the configuration to launch."""
 import os
 
+import torch
+
 from ..autotuner import base_tunner
 from ..autotuner.runtime import Runtime
 
@@ -37,3 +39,16 @@ def planned(key, make_tuner, default_factory):
         cc = resolve(tuner, default_factory)
         plan = base_tunner._memo[k] = (cc, Runtime(tuner.arch, cc))
     return plan
+
+
+class NoGraph:
+    """Stands in for the autograd context when no input of a call requires a gradient: the operators then run their
+    forward directly (an inference call skips the ~15 us a ``torch.autograd.Function.apply`` costs on the host)."""
+    needs_input_grad = (False,) * 8
+
+    def save_for_backward(self, *tensors):
+        pass
+
+
+def wants_graph(*tensors):
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)

@@ -15,7 +15,7 @@ import torch
 from ..arch import Arch
 from ..autotuner import gfx950_space
 from ..autotuner.tunner import AttnBwdTunner, AttnTunner
-from ._resolve import planned
+from ._resolve import NoGraph, planned, wants_graph
 
 REFERENCE_SOFTMAX_SCALE = 0.125
 
@@ -74,4 +74,9 @@ class MultiHeadAttnFunc(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
-flash_attn_func = MultiHeadAttnFunc.apply
+def flash_attn_func(q, k, v, device_type: Arch, causal=False, softmax_scale=None):
+    """``MultiHeadAttnFunc.apply`` (the reference's ``flash_attn_func``, python/ops/attention_interface.py:60) when a
+    gradient may be asked for; the same forward without the autograd machinery otherwise."""
+    if wants_graph(q, k, v):
+        return MultiHeadAttnFunc.apply(q, k, v, device_type, causal, softmax_scale)
+    return MultiHeadAttnFunc.forward(NoGraph(), q, k, v, device_type, causal, softmax_scale)

@@ -25,7 +25,7 @@ from ..arch import Arch
 from ..autotuner import gfx950_space
 from ..autotuner.runtime import Runtime
 from ..autotuner.tunner import RetTunner, RetBwdTunner
-from ._resolve import planned
+from ._resolve import NoGraph, planned, wants_graph
 
 
 def retnet_mask_scan(mask, device_type: Arch):
@@ -180,5 +180,15 @@ class RetNetDecayAttn(torch.autograd.Function):
         return dq, dk, dv, None, None
 
 
-RetNetAttnFunc = RetNetAttn.apply
-RetNetDecayAttnFunc = RetNetDecayAttn.apply
+def RetNetAttnFunc(q, k, v, mask, device_type: Arch, causal=None):
+    """``RetNetAttn.apply`` (the reference's ``RetNetAttnFunc``, python/ops/retnet_interface.py:57) when a gradient may
+    be asked for; the same forward without the autograd machinery otherwise."""
+    if wants_graph(q, k, v):
+        return RetNetAttn.apply(q, k, v, mask, device_type, causal)
+    return RetNetAttn.forward(NoGraph(), q, k, v, mask, device_type, causal)
+
+
+def RetNetDecayAttnFunc(q, k, v, gamma, device_type: Arch):
+    if wants_graph(q, k, v):
+        return RetNetDecayAttn.apply(q, k, v, gamma, device_type)
+    return RetNetDecayAttn.forward(NoGraph(), q, k, v, gamma, device_type)

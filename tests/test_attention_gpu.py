@@ -350,3 +350,25 @@ def test_persistent_forward_replays_from_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(o, eager)
         assert _err(o, ref_op.attention_ref(q2, k2, v2, None, False)) <= TOL
+
+
+def test_calls_without_a_gradient_skip_autograd_and_repeated_calls_keep_one_plan():
+    """``flash_attn_func`` on inputs that need no gradient runs the forward directly; with a gradient it goes through
+    ``MultiHeadAttnFunc.apply``.  Same bits either way, and the (configuration, runtime) pair of a problem is resolved
+    once per process."""
+    from attention_autotuner_amd.autotuner import base_tunner
+    q, k, v = (t.cuda() for t in _inputs(2, 4, 512, 512, 128, 128, seed=41))
+    o0 = aat.flash_attn_func(q, k, v, ARCH, True)
+    keys = [key for key in base_tunner._memo if key[0] == "plan" and key[3] == "attn" and key[5:] == (2, 4, 512, 512, 128, 128, True)]
+    assert len(keys) == 1
+    plan = base_tunner._memo[keys[0]]
+    qg = q.clone().requires_grad_(True)
+    o1 = aat.flash_attn_func(qg, k, v, ARCH, True)
+    assert o1.requires_grad and o1.grad_fn is not None and not o0.requires_grad
+    with torch.no_grad():
+        o2 = aat.flash_attn_func(qg, k, v, ARCH, True)
+    assert not o2.requires_grad and torch.equal(o0, o1) and torch.equal(o0, o2)
+    assert base_tunner._memo[keys[0]] is plan
+    o1.backward(torch.ones_like(o1))
+    assert qg.grad is not None and bool(torch.isfinite(qg.grad).all())
+    assert _err(o0, ref_op.attention_ref(*(t.cpu() for t in (q, k, v)), None, True)) <= TOL
