@@ -161,11 +161,13 @@ int kernel_entry_ex(aat_half* q, aat_half* k, aat_half* v, aat_half* o, aat_half
  * retnet_recurrent_workspace_size() bytes of workspace hold the per-(head, chunk) decay factors and, for
  * more than 128 key dims (contracted in passes of 128 whose outputs add), a second output-sized buffer;
  * workspace_size(B, H, l, l) is the same figure for up to 128 key dims.  The
- * reference-signature entry point has no workspace argument: it is the one exception to "nothing is
- * allocated by the callee" -- it keeps one buffer per device, grown on demand, until the process ends,
- * launches on the null stream and reports errors on stderr.  Every call on a device uses that one buffer:
- * calls that overlap on one GPU (other streams, other threads) race; such callers take the _ex entry point
- * with a workspace of their own. */
+ * reference-signature entry point has no workspace argument: up to 128 key dims and
+ * AAT_RECURRENT_NOALLOC_MAX_RECORDS (head, chunk) pairs (the reference benchmark's shape among them) it keeps
+ * the factors in the static array of retnet_recurrent_fwd_noalloc below and allocates nothing; beyond that it
+ * is the one exception to "nothing is allocated by the callee" -- one buffer per device, grown on demand, kept
+ * until the process ends.  It launches on the null stream and reports errors on stderr.  Every call on a
+ * device uses that device's one array or buffer: calls that overlap on one GPU (other streams, other
+ * threads) race; such callers take the _ex entry point with a workspace of their own. */
 void retnet_recurrent_fwd(void* d_q, void* d_k, void* d_v, void* d_decay, void* d_out, int batch, int heads,
                           int kdim, int vdim, int l, int block_kdim);
 size_t retnet_recurrent_workspace_size(int batch, int heads, int kdim, int vdim, int l, int block_kdim);

@@ -89,12 +89,22 @@ def test_reference_signature_entry_point_and_error_codes():
     torch.cuda.synchronize()
     out_ex = aat.retnet_recurrent_fwd(q, k, v, decay)
     assert torch.equal(out_ref_sig, out_ex)
-    # a second, larger call makes the cached workspace grow
+    # a second, larger call: still within what the library's static array holds, so nothing is allocated
     q2, k2, v2, decay2 = [t.cuda() for t in _inputs(5, 1, 4, 64, 64, 256, 0.7, 1.0)]
     out2 = torch.zeros_like(v2)
+    want2 = aat.retnet_recurrent_fwd(q2, k2, v2, decay2)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
     lib.retnet_recurrent_fwd(ptr(q2), ptr(k2), ptr(v2), ptr(decay2), ptr(out2), 1, 4, 64, 64, 256, 64)
     torch.cuda.synchronize()
-    assert torch.equal(out2, aat.retnet_recurrent_fwd(q2, k2, v2, decay2))
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(out2, want2)
+    # more than 128 key dims per pass need a second output-sized buffer: the entry point allocates one and keeps it
+    q3, k3, v3, decay3 = [t.cuda() for t in _inputs(6, 1, 2, 256, 64, 128, 0.7, 1.0)]
+    out3 = torch.zeros_like(v3)
+    lib.retnet_recurrent_fwd(ptr(q3), ptr(k3), ptr(v3), ptr(decay3), ptr(out3), 1, 2, 256, 64, 128, 256)
+    torch.cuda.synchronize()
+    assert torch.equal(out3, aat.retnet_recurrent_fwd(q3, k3, v3, decay3, block_kdim=256))
 
     need = lib.workspace_size(b, h, seqlen, seqlen)
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
