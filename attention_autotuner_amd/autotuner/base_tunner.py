@@ -242,6 +242,8 @@ class BaseTunner:
         os.makedirs(self.cache_path, exist_ok=True)
         with open(self._cache_file(), "w") as f:
             json.dump(config.to_dict(), f)
+        for key in [k for k in _memo if k[0] == "plan"]:      # launch plans the operators resolved before this entry existed
+            del _memo[key]
         _memo[self._memo_key()] = config
 
     # ---- what is not worth timing ----------------------------------------------------------------------

@@ -397,3 +397,26 @@ def test_without_tuning_a_miss_launches_the_entry_of_the_nearest_problem(tmp_pat
     assert resolved(sq=384, sk=8192)[0] == near           # 256-row blocks do not divide 384 rows: the next nearest
     assert resolved(sq=64, sk=2048)[0] == default         # the one entry within reach does not fit: the built-in default
     base_tunner._memo.clear()
+
+
+def test_an_operator_resolves_a_problem_once_and_again_after_a_tuning_result_is_written(tmp_path, monkeypatch):
+    from attention_autotuner_amd.ops import _resolve
+    base_tunner._memo.clear()
+    monkeypatch.setattr(_resolve, "Runtime", lambda arch, cc: ("runtime of", cc))      # no library is built or loaded here
+    monkeypatch.setenv("AAT_TUNE_ON_MISS", "0")
+    default = gfx950_space.default_forward_config("attn", 128, 128, ARCH)
+    tuned = AttnConfig(Br=128, Bc=64, Kd=128, D=128, Nthreads=256)
+    built = []
+
+    def make():
+        t = AttnTunner(ARCH, _meta(), causal=False)
+        t.cache_path = str(tmp_path)
+        built.append(t)
+        return t
+    key = ("attn", ARCH.name, 4, 32, 2048, 2048, 128, 128, False)
+    cc, rt = _resolve.planned(key, make, lambda: default)
+    assert cc == default and rt == ("runtime of", default) and len(built) == 1
+    assert _resolve.planned(key, make, lambda: default)[0] is cc and len(built) == 1      # one dictionary lookup, no tuner
+    built[0]._write_cache(tuned)
+    assert _resolve.planned(key, make, lambda: default)[0] == tuned and len(built) == 2
+    base_tunner._memo.clear()
