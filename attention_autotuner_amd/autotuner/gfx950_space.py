@@ -407,7 +407,7 @@ def attn_backward_valid(cfg, arch):
     if nw > 4 * cfg.waves_per_eu or cfg.num_stages_qk not in (2, 3):
         return False
     for cols in (cfg.Kd, cfg.D):
-        if cols % 64 or (cols // 8 != 8 and (cols // 8) % 16):     # the dual swizzle covers 64-wide and multiples of 128
+        if cols % 64:                                              # the dual swizzle covers every multiple of 64
             return False
         if (cfg.Bc * cols // 8) % cfg.Nthreads:
             return False

@@ -71,19 +71,24 @@ struct AttnBwdChain {
   static constexpr int kSmemBytes = kMainBytes > kEpiBytes ? kMainBytes : kEpiBytes;
 };
 
-// delta[row] = sum_d dO[row][d] * O[row][d], lse2[row] = lse[row] * log2(e); one wave per 64/(D/8) rows.
+// delta[row] = sum_d dO[row][d] * O[row][d], lse2[row] = lse[row] * log2(e); a power-of-two group of lanes per row.
+template <int D> constexpr int attn_bwd_prepare_lanes_per_row() {
+  return D / 8 <= 8 ? 8 : D / 8 <= 16 ? 16 : D / 8 <= 32 ? 32 : 64;
+}
+template <int D> constexpr int attn_bwd_prepare_rows_per_block() { return 4 * (64 / attn_bwd_prepare_lanes_per_row<D>()); }
 template <int D>
 __global__ void __launch_bounds__(256) attn_bwd_prepare(const half_t* __restrict__ o, const half_t* __restrict__ dO,
                                                         const float* __restrict__ lse, float* __restrict__ lse2,
                                                         float* __restrict__ delta, int rows) {
-  constexpr int kLanesPerRow = D / 8;                   // 16-byte chunks per row: 8, 16, 32 or 64
-  static_assert(64 % kLanesPerRow == 0, "row width");
+  constexpr int kChunks = D / 8;                        // 16-byte chunks per row: 8, 16, 24, 32 or 64
+  constexpr int kLanesPerRow = attn_bwd_prepare_lanes_per_row<D>();   // lanes beyond the row's chunks idle
+  static_assert(kChunks <= 64, "row width");
   constexpr int kRowsPerWave = 64 / kLanesPerRow;
   const int lane = threadIdx.x & 63;
   const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6;
   const int row = wave * kRowsPerWave + lane / kLanesPerRow;
   float s = 0.f;
-  if (row < rows) {
+  if (row < rows && lane % kLanesPerRow < kChunks) {
     const size_t off = (size_t)row * D + (lane % kLanesPerRow) * 8;
     const h8 a = *reinterpret_cast<const h8*>(o + off);
     const h8 b = *reinterpret_cast<const h8*>(dO + off);

@@ -63,7 +63,7 @@ hipError_t launch(aat_half* q, aat_half* k, aat_half* v, aat_half* o, aat_half* 
   const int rows = B * H * Seq_q;
   float* lse2 = static_cast<float*>(workspace);
   float* delta = lse2 + rows;
-  constexpr int rows_per_block = 4 * (64 / (D / 8));
+  constexpr int rows_per_block = aat::attn_bwd_prepare_rows_per_block<D>();
   aat::attn_bwd_prepare<D><<<dim3((rows + rows_per_block - 1) / rows_per_block), dim3(256), 0, stream>>>(O, G, lse, lse2, delta, rows);
   const float c2 = softmax_scale * 1.4426950408889634f;
 #if AAT_COL_SPLIT

@@ -108,9 +108,12 @@ template <int NC> AAT_DEV constexpr int swz_both(int row, int c) {
   if constexpr (NC % 16 == 0) {
     return c ^ ((row & 15) ^ ((row & 3) << 2));                      // (b3^b1, b2^b0, b1, b0)
   } else {
-    static_assert(NC == 8, "tiles read both ways are 64 or a multiple of 128 halfs wide");
+    // an odd number of 128-byte halves per row (64, 192, 320 ... halfs): consecutive rows start on alternating halves
+    // of a 256-byte line, so the row's lowest bit already separates them and the XOR term, which stays inside a group
+    // of 8 chunks, is a bijection of the other three
+    static_assert(NC % 16 == 8, "tiles read both ways are a multiple of 64 halfs wide");
     const int b1 = (row >> 1) & 1, b2 = (row >> 2) & 1, b3 = (row >> 3) & 1;
-    return c ^ (((b3 ^ b1) << 2) | (b2 << 1) | b1);                  // two rows share a 256-byte line
+    return c ^ (((b3 ^ b1) << 2) | (b2 << 1) | b1);
   }
 }
 
@@ -157,8 +160,10 @@ static_assert(transposing_phase_conflict_free<8, Swz::Rows4>() && transposing_ph
               "transposing reads of 64..512-wide tiles are conflict-free");
 static_assert(b128_phase_conflict_free<8, Swz::Both>() && transposing_phase_conflict_free<8, Swz::Both>() &&
               b128_phase_conflict_free<16, Swz::Both>() && transposing_phase_conflict_free<16, Swz::Both>() &&
-              b128_phase_conflict_free<32, Swz::Both>() && transposing_phase_conflict_free<32, Swz::Both>(),
-              "tiles read both ways (64/128/256 wide) are conflict-free for both access patterns");
+              b128_phase_conflict_free<24, Swz::Both>() && transposing_phase_conflict_free<24, Swz::Both>() &&
+              b128_phase_conflict_free<32, Swz::Both>() && transposing_phase_conflict_free<32, Swz::Both>() &&
+              b128_phase_conflict_free<64, Swz::Both>() && transposing_phase_conflict_free<64, Swz::Both>(),
+              "tiles read both ways (64/128/192/256/512 wide) are conflict-free for both access patterns");
 
 constexpr int cgcd(int a, int b) { return b == 0 ? a : cgcd(b, a % b); }
 

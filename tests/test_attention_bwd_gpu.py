@@ -148,11 +148,18 @@ def test_abi_error_paths_and_stream():
     assert rc == 0 and torch.isfinite(dq.float()).all()
 
 
-def test_unsupported_head_sizes_say_so():
-    """192-wide rows have no dual swizzle (64 or multiples of 128): the forward runs, the backward says so."""
-    q, k, v, do = _inputs(1, 1, 128, 128, 192, 192, seed=9)
+def test_a_problem_without_a_backward_configuration_says_so(monkeypatch):
+    """The forward runs; the backward reports what the search space cannot cover as NotImplementedError."""
+    from attention_autotuner_amd.autotuner import base_tunner, gfx950_space
+
+    def none_fits(*a, **kw):
+        raise gfx950_space.NoValidConfigError("no default attn_bwd configuration fits")
+    q, k, v, do = _inputs(1, 1, 128, 128, 64, 64, seed=9)
     qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
     o = aat.flash_attn_func(qc, kc, vc, ARCH)
+    monkeypatch.setattr(gfx950_space, "default_attn_backward_config", none_fits)
+    for key in [key for key in base_tunner._memo if key[0] == "plan" and key[3] == "attn_bwd"]:
+        del base_tunner._memo[key]
     with pytest.raises(NotImplementedError):
         o.backward(do.cuda())
 
