@@ -162,8 +162,11 @@ static_assert(b128_phase_conflict_free<8, Swz::Both>() && transposing_phase_conf
               b128_phase_conflict_free<16, Swz::Both>() && transposing_phase_conflict_free<16, Swz::Both>() &&
               b128_phase_conflict_free<24, Swz::Both>() && transposing_phase_conflict_free<24, Swz::Both>() &&
               b128_phase_conflict_free<32, Swz::Both>() && transposing_phase_conflict_free<32, Swz::Both>() &&
+              b128_phase_conflict_free<40, Swz::Both>() && transposing_phase_conflict_free<40, Swz::Both>() &&
+              b128_phase_conflict_free<48, Swz::Both>() && transposing_phase_conflict_free<48, Swz::Both>() &&
+              b128_phase_conflict_free<56, Swz::Both>() && transposing_phase_conflict_free<56, Swz::Both>() &&
               b128_phase_conflict_free<64, Swz::Both>() && transposing_phase_conflict_free<64, Swz::Both>(),
-              "tiles read both ways (64/128/192/256/512 wide) are conflict-free for both access patterns");
+              "tiles read both ways (every multiple of 64 halfs up to 512) are conflict-free for both access patterns");
 
 constexpr int cgcd(int a, int b) { return b == 0 ? a : cgcd(b, a % b); }
 
