@@ -17,10 +17,10 @@ from .configs import supported_configs
 
 # (operator, d_qk, d_v) pairs whose default configuration is always built
 DEFAULT_PROBLEMS = [
-    ("attn", 64, 64), ("attn", 128, 128), ("attn", 256, 256), ("attn", 192, 192), ("attn", 256, 128), ("attn", 64, 128), ("attn", 128, 64),
+    ("attn", 64, 64), ("attn", 128, 128), ("attn", 256, 256), ("attn", 192, 192), ("attn", 256, 128), ("attn", 64, 128), ("attn", 128, 64), ("attn", 128, 192), ("attn", 192, 64),
     ("attn", 256, 512),
     ("ret", 64, 64), ("ret", 128, 128), ("ret", 192, 192), ("ret", 256, 256), ("ret", 64, 128), ("ret", 256, 512),
-    ("attn_bwd", 64, 64), ("attn_bwd", 128, 128), ("attn_bwd", 64, 128), ("attn_bwd", 128, 64), ("attn_bwd", 192, 192), ("attn_bwd", 256, 128),
+    ("attn_bwd", 64, 64), ("attn_bwd", 128, 128), ("attn_bwd", 64, 128), ("attn_bwd", 128, 64), ("attn_bwd", 192, 192), ("attn_bwd", 128, 192), ("attn_bwd", 192, 64), ("attn_bwd", 256, 128),
     ("attn_bwd", 256, 256), ("attn_bwd", 256, 512),
 ]
 

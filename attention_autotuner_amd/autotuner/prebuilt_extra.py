@@ -23,7 +23,7 @@ def unit_config(br, bc, unit, nt, wpe, dqk, dv):
 SHARED_TILES = [(128, 64, 256, 2, 2, 1, 4, 2), (64, 64, 256, 1, 1, 2, 4, 2), (64, 64, 256, 2, 1, 2, 2, 2), (64, 64, 256, 1, 1, 2, 4, 1)]
 SHARED_DIMS = [(64, 64), (128, 128), (256, 512)]
 # attention backward: head-size pairs run at their defaults, and (Br, Bc, Nthreads, buffers) variants at 128/128
-ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (192, 192), (256, 128), (256, 256), (256, 512)]
+ATTN_BWD_DIMS = [(64, 64), (128, 128), (64, 128), (128, 64), (192, 192), (128, 192), (192, 64), (256, 128), (256, 256), (256, 512)]
 ATTN_BWD_TILES = [(64, 32, 128, 2), (64, 64, 128, 2), (128, 64, 256, 3), (128, 32, 256, 2)]
 # ... and with one column kernel per output: (Br, Bc, Nthreads, buffers, row waves/SIMD, row Bc, dV waves/SIMD, dK waves/SIMD)
 ATTN_BWD_SPLIT_TILES = [(128, 32, 256, 2, 2, 32, 2, 2), (128, 64, 256, 2, 2, 32, 2, 1), (128, 32, 256, 3, 2, 32, 3, 2),
