@@ -98,3 +98,19 @@ def test_random_problems_match_the_oracle(seed):
                 print(f"   {name}: {small:.3e} under the literal rule vs the fp16-operand form; |err| / (ulp/2 + 2^-11 T) vs the exact form = {ratio:.2f}")
             assert ok, (what, name, small, large)
     assert held_to_terms <= 4, held_to_terms                   # a thin set: most problems meet the literal rule everywhere
+
+
+def test_long_rows_s8192_causal_forward_and_backward():
+    """B1 H4 S8192 d128, causal: 64 kv tiles per row block and the configurations tuned for long rows; one head against the oracle."""
+    g = torch.Generator().manual_seed(5)
+    q, k, v, do = (torch.randn(1, 4, 8192, 128, generator=g).half() for _ in range(4))
+    qc, kc, vc = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = aat.flash_attn_func(qc, kc, vc, ARCH, True)
+    o.backward(do.cuda())
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(o).all()) and all(bool(torch.isfinite(t.grad).all()) for t in (qc, kc, vc))
+    sl = (slice(0, 1), slice(3, 4))
+    tolerance.assert_close(o[sl], ref_op.attention_ref(q[sl], k[sl], v[sl], None, True), "S8192 causal o")
+    as_kernel = ref_op.attention_bwd_ref(q[sl], k[sl], v[sl], do[sl], None, True, o=o[sl].detach().cpu(), operand_dtype=torch.float16)
+    for name, got, want in zip(("dq", "dk", "dv"), (qc.grad[sl], kc.grad[sl], vc.grad[sl]), as_kernel):
+        tolerance.assert_close(got, want, f"S8192 causal {name}")
