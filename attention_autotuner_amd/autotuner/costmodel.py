@@ -92,10 +92,36 @@ def backward_features(cfg, shape, causal=False):
     return total
 
 
+def attn_backward_features(cfg, shape, causal=False):
+    """The same quantities for an attention backward configuration, summed over its kernels: the column kernel (``Br`` kv
+    rows resident, query tiles of ``Bc`` rows streamed; S, dP, dV and dK: contractions over d_qk + d_v and into
+    d_v + d_qk columns) -- or, with ``col_split``, one column kernel for dV (S and dV) and one for dK (S, dP and dK), each
+    at its own waves per SIMD -- and the row kernel (``Br`` query rows resident, kv tiles of ``row_Bc`` rows; S, dP, dQ)."""
+    b, h, sq, sk = shape
+    nw = cfg.Nthreads // 64
+    half = 0.5 if causal else 1.0
+
+    def per_cu(wpe):
+        return max(1, wpe * 4 // nw)
+    total = np.zeros(len(ALL_FEATURES))
+    col_blocks, col_steps = b * h * (sk // cfg.Br), half * sq / cfg.Bc + 0.5 * causal
+    if getattr(cfg, "col_split", 0):
+        total += _chain_features(col_blocks, col_steps, cfg.Br, cfg.Bc, cfg.Kd, cfg.D, nw, per_cu(cfg.dv_waves_per_eu), barriers=1, mask_tiles=0)
+        total += _chain_features(col_blocks, col_steps, cfg.Br, cfg.Bc, cfg.Kd + cfg.D, cfg.Kd, nw, per_cu(cfg.dk_waves_per_eu), barriers=1, mask_tiles=0)
+    else:
+        total += _chain_features(col_blocks, col_steps, cfg.Br, cfg.Bc, cfg.Kd + cfg.D, cfg.D + cfg.Kd, nw, per_cu(cfg.waves_per_eu), barriers=1, mask_tiles=0)
+    row_bc = getattr(cfg, "row_Bc", cfg.Bc)
+    row_wpe = getattr(cfg, "row_waves_per_eu", cfg.waves_per_eu)
+    total += _chain_features(b * h * (sq // cfg.Br), half * sk / row_bc + 0.5 * causal, cfg.Br, row_bc, cfg.Kd + cfg.D, cfg.Kd, nw, per_cu(row_wpe), barriers=1, mask_tiles=0)
+    total[7] = 1.0
+    return total
+
+
 def features(cfg, shape, causal=False, names=FEATURES):
     """The feature vector (in the order of ``names``) of configuration ``cfg`` on ``shape`` = (B, H, Sq, Sk): forward
-    kernels in ``forward_features``, the RetNet backward in ``backward_features``."""
-    full = backward_features(cfg, shape, causal) if getattr(cfg, "operation", "") == "ret_bwd" else forward_features(cfg, shape, causal)
+    kernels in ``forward_features``, the backward operators in ``backward_features`` / ``attn_backward_features``."""
+    op = getattr(cfg, "operation", "")
+    full = (backward_features if op == "ret_bwd" else attn_backward_features if op == "attn_bwd" else forward_features)(cfg, shape, causal)
     return np.array([full[ALL_FEATURES.index(n)] for n in names])
 
 
@@ -277,7 +303,7 @@ def main(argv=None):
     args = ap.parse_args(argv)
     if args.command == "fit-logs":
         samples = [s for path in args.exports for s in samples_from_summary(path, args.op)]
-        model = CostModel(unit="ms", names=RET_FEATURES if args.op in ("ret", "ret_bwd") else FEATURES).fit(samples)
+        model = CostModel(unit="ms", names=RET_FEATURES if args.op in ("ret", "ret_bwd", "attn_bwd") else FEATURES).fit(samples)
         model.save(args.out)
         print(json.dumps({"samples": len(samples), "out": args.out}))
         return 0

@@ -143,6 +143,8 @@ class AttnBwdTunner(BaseTunner):
     python/ops/attention_interface.py:37-58 leaves the operator empty).  ``torch_array`` is
     [q, k, v, o, dO, lse, dq, dk, dv]."""
     operation = "attn_bwd"
+    cost_model_file = "costmodel_attn_bwd.json"
+    _shipped_cost_model = _shipped_cost_model
 
     def __init__(self, arch, torch_array, causal=False, softmax_scale=None):
         super().__init__(arch, torch_array, "attention_bwd", causal=causal, softmax_scale=softmax_scale)

@@ -222,6 +222,45 @@ def test_retnet_models_keep_the_winner_of_head_sizes_they_have_not_seen(op):
     assert len(kept) == max(tuner.keep_min, int(len(cfgs) * tuner.keep_fraction + 0.999)) < len(cfgs)
 
 
+ATTN_BWD_RUNS = {                                         # file -> ((B, H, Sq, Sk, d_qk, d_v), causal)
+    "attn_bwd_b4h32q2048k2048_c0_128_128.txt": ((4, 32, 2048, 2048, 128, 128), False),
+    "attn_bwd_b4h32q2048k2048_c1_128_128.txt": ((4, 32, 2048, 2048, 128, 128), True),
+    "attn_bwd_b8h32q1024k1024_c1_128_128.txt": ((8, 32, 1024, 1024, 128, 128), True),
+    "attn_bwd_b4h8q2048k2048_c0_64_64.txt": ((4, 8, 2048, 2048, 64, 64), False),
+    "attn_bwd_b4h32q2048k2048_c1_64_64.txt": ((4, 32, 2048, 2048, 64, 64), True),
+    "attn_bwd_b4h8q2048k2048_c1_192_192.txt": ((4, 8, 2048, 2048, 192, 192), True),
+    "attn_bwd_b4h8q2048k2048_c0_256_256.txt": ((4, 8, 2048, 2048, 256, 256), False),
+}
+
+
+def test_attention_backward_model_keeps_the_winner_of_head_sizes_it_has_not_seen():
+    """Seven recorded exhaustive runs of the attention backward space (four head sizes, three problem shapes, both walks;
+    the row kernel's own occupancy and tile height and the one-kernel-per-output variants among the candidates).  The
+    shipped model is the fit on all of them; fitted without one head size it still ranks that size's winners inside the
+    share the tuning loop keeps."""
+    from attention_autotuner_amd.autotuner.tunner import AttnBwdTunner
+    from attention_autotuner_amd.benchmarks.tune import make_tensors
+    runs = {n: costmodel.samples_from_tuning_log(os.path.join(LOGS, n), "attn_bwd", p[4], p[5], p[:4], c) for n, (p, c) in ATTN_BWD_RUNS.items()}
+    assert [len(runs[n]) for n in ATTN_BWD_RUNS] == [50, 50, 50, 118, 118, 15, 6]
+    some = runs["attn_bwd_b4h32q2048k2048_c0_128_128.txt"]       # the log lines parse back with every knob
+    assert {c.col_split for c, *_ in some} == {0, 1} and {c.row_waves_per_eu for c, *_ in some} == {1, 2} and {c.row_Bc for c, *_ in some} == {32, 64}
+    fitted = costmodel.CostModel(unit="ms", names=costmodel.RET_FEATURES).fit([s for r in runs.values() for s in r])
+    tuner = AttnBwdTunner(MI355X(), make_tensors("attn_bwd", 4, 32, 2048, 2048, 128, 128, "meta"), causal=True)
+    assert tuner.cost_model is not None and tuner.cost_model.names == costmodel.RET_FEATURES
+    np.testing.assert_allclose(tuner.cost_model.weights, fitted.weights, rtol=1e-6)
+    for n in runs:
+        assert _survives(tuner.cost_model, runs[n], AttnBwdTunner), (n, tuner.cost_model.rank_of_best(runs[n]))
+    for dims in {p[4:] for p, _ in ATTN_BWD_RUNS.values()}:
+        train = [s for n, (p, _) in ATTN_BWD_RUNS.items() if p[4:] != dims for s in runs[n]]
+        held_out = costmodel.CostModel(unit="ms", names=costmodel.RET_FEATURES).fit(train)
+        for n, (p, _) in ATTN_BWD_RUNS.items():
+            if p[4:] == dims:
+                assert _survives(held_out, runs[n], AttnBwdTunner), (dims, n, held_out.rank_of_best(runs[n]))
+    cfgs = [c for c in tuner.get_tuned_configs() if tuner._fits_problem(c)]
+    kept = tuner.prune(cfgs)
+    assert len(kept) == max(tuner.keep_min, int(len(cfgs) * tuner.keep_fraction + 0.999)) < len(cfgs)
+
+
 def test_an_attention_model_file_still_loads_and_a_foreign_feature_set_does_not(tmp_path):
     m = costmodel.CostModel.load(os.path.join(AttnTunner(MI355X(), _meta(4, 32, 2048)).cache_path, "costmodel_attn.json"))
     assert m.names == costmodel.FEATURES
