@@ -131,7 +131,7 @@ ret_bwd_chain(const half_t* __restrict__ x, const half_t* __restrict__ y, const 
   if (extents != nullptr) {                       // the streamed tiles in which the mask has a non-zero entry for these rows
     const MaskExtents e = mask_extents_at(extents, H, seq_q, seq_k);
     int lo, hi;
-    if constexpr (COL) mask_col_range(e, bh % H, seq_k, x0, BX, lo, hi);
+    if constexpr (COL) mask_col_range(e, bh % H, seq_q, seq_k, x0, BX, lo, hi);
     else mask_row_range(e, bh % H, seq_q, x0, BX, lo, hi);
     mask_tile_range(lo, hi, BY, j_end, j_begin, j_end);
   } else if (causal) {

@@ -79,7 +79,7 @@ ret_bwd_dk_from_ds(const half_t* __restrict__ q, const half_t* __restrict__ ds, 
   if (extents != nullptr) {
     ext = mask_extents_at(extents, H, seq_q, seq_k);
     int lo, hi;
-    mask_col_range(ext, head, seq_k, x0, BX, lo, hi);
+    mask_col_range(ext, head, seq_q, seq_k, x0, BX, lo, hi);
     mask_tile_range(lo, hi, BY, j_end, j_begin, j_end);
   } else if (causal) {                            // q tiles that reach kv >= x0:  q >= x0 - diag
     const int first = x0 - diag;
