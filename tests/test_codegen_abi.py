@@ -77,10 +77,10 @@ def test_shipping_set_is_built_and_exports_the_abi():
             assert lib.retnet_recurrent_workspace_size(8, 4, 256, 64, 2000, 256) == 0     # unsupported shape
         elif cfg.operation == "attn_bwd":
             assert lib.workspace_size(2, 3, 256, 512) == 2 * 2 * 3 * 256 * 4      # lse2 + delta, fp32 per query row
-        elif cfg.operation in ("ret", "ret_bwd"):       # the mask scan: 4 ranges per band of 32 rows / columns + a byte per 32 x 32 tile
+        elif cfg.operation in ("ret", "ret_bwd"):       # the mask scan: 2 range ends per band of 32 query rows + a byte per 32 x 32 tile
             # a backward built with a stored dS adds the room for it: B*H*S_q*S_kv fp16
             ds = 2 if getattr(cfg, "ds_rows", 0) else 0
-            assert lib.workspace_size(5, 3, 256, 512) == 1024 + ds * 5 * 3 * 256 * 512     # 4 * 3 * (2 * 8 + 2 * 16) + 3 * 8 * 16 = 960, in units of 256
+            assert lib.workspace_size(5, 3, 256, 512) == 768 + ds * 5 * 3 * 256 * 512      # 4 * 3 * 2 * 8 + 3 * 8 * 16 = 576, in units of 256
             assert lib.workspace_size(1, 1, 256, 256) == 256 + ds * 256 * 256              # rounded up to 256 bytes
             assert lib.workspace_size(1, 1, 256, 320) == 256                       # a length its dK kernel cannot tile: the scan alone
         elif getattr(cfg, "kv_splits", 1) == 1:
